@@ -1,0 +1,394 @@
+"""Pins for the CPU oracle: every check here is independent of the oracle's own formulas.
+
+The reference ships no golden files for the MXFP4 path, so the oracle is pinned by
+closed forms, exhaustive enumeration against brute force, counting identities and a
+second scalar model (``oracle/scalar_model.py``).
+"""
+import math
+from fractions import Fraction
+
+import numpy as np
+import pytest
+import torch
+
+import oracle as O
+from oracle import scalar_model as S
+
+
+def bf16_from_bits(bits):
+    return torch.tensor(np.asarray(bits, dtype=np.uint16).astype(np.int16)).view(torch.bfloat16)
+
+
+# ----------------------------------------------------------------------------- Q1 scale
+@pytest.mark.parametrize("bits,expect", [
+    (0x3F80, 125),  # 1.0
+    (0x3FC0, 125),  # 1.5
+    (0x3FDF, 125),  # 1.7421875: largest mantissa that does not carry
+    (0x3FE0, 126),  # 1.75 carries into the exponent
+    (0x40C0, 127),  # 6.0
+    (0x40E0, 128),  # 7.0: separates "round absmax to one mantissa bit" from floor(log2)
+    (0x0000, 1),    # all-zero block
+    (0x0040, 1),    # bf16 subnormal
+    (0x0080, 1),    # smallest normal (e=1 -> -1 -> clamp)
+    (0x7F7F, 253),  # largest finite bf16: exponent 254 carries to 255, minus 2
+])
+def test_scale_known_answers(bits, expect):
+    assert int(O.e8m0_from_absmax(bf16_from_bits([bits]))[0]) == expect
+    assert S.scale_from_absmax_bits(bits, 7) == expect
+
+
+def test_scale_exhaustive_bf16_vs_float_model():
+    bits = np.arange(0, 0x7F80, dtype=np.uint16)  # all non-negative finite bf16
+    got = O.e8m0_from_absmax(bf16_from_bits(bits)).numpy().astype(np.int64)
+    vals = bf16_from_bits(bits).double().numpy()
+    exp = np.ones_like(got)
+    for i, v in enumerate(vals):
+        if v < 2.0 ** -126:  # zero / subnormal: exponent field 0 (+ possible carry to 1) -> clamp
+            exp[i] = 1
+            continue
+        m, e = math.frexp(v)          # v = m * 2^e, m in [0.5, 1)
+        e_unb = e - 1                  # v = (2m) * 2^(e-1), 2m in [1, 2)
+        if 2 * m >= 1.75:
+            e_unb += 1
+        exp[i] = max(e_unb + 127 - 2, 1)
+    assert np.array_equal(got, exp)
+
+
+def test_scale_fp32_vs_scalar_model():
+    g = torch.Generator().manual_seed(3)
+    x = (torch.randn(4096, generator=g) * torch.exp2(torch.randint(-140, 120, (4096,), generator=g).float())).abs()
+    x[:4] = torch.tensor([0.0, 1.75, 7.0, 1e-45])
+    got = O.e8m0_from_absmax(x)
+    for i in range(x.numel()):
+        assert int(got[i]) == S.scale_from_absmax_bits(S.f32_bits(float(x[i])), 23)
+
+
+# ----------------------------------------------------------------------------- Q2 RNE encode
+def brute_force_rne(mag: np.ndarray) -> np.ndarray:
+    """Nearest E2M1 code for non-negative magnitudes; ties to the even code; saturate at 6."""
+    grid = np.array(O.E2M1_GRID, dtype=np.float64)
+    d = np.abs(mag[:, None] - grid[None, :])
+    best = d.min(axis=1)
+    is_best = d == best[:, None]
+    # among tied candidates prefer even code
+    codes = np.arange(8)
+    even_pref = np.where(is_best & (codes % 2 == 0)[None, :], 1, 0)
+    pick_even = even_pref.any(axis=1)
+    first_even = np.argmax(is_best & (codes % 2 == 0)[None, :], axis=1)
+    first_any = np.argmax(is_best, axis=1)
+    out = np.where(pick_even, first_even, first_any)
+    out = np.where(mag >= 6.0, 7, out)
+    return out
+
+
+def test_rne_exhaustive_bf16_times_scales():
+    bits = np.arange(0, 0x10000, dtype=np.uint32)
+    finite = (bits & 0x7F80) != 0x7F80
+    bits = bits[finite].astype(np.uint16)
+    x = bf16_from_bits(bits).float()
+    xd = x.double().numpy()
+    for s in [1, 2, 17, 100, 119, 120, 121, 122, 123, 124, 125, 126, 127, 128, 129, 130, 131, 140, 200, 252, 253]:
+        scale = torch.tensor([s], dtype=torch.int32).bitwise_left_shift(23).view(torch.float32)
+        q = x / scale
+        keep = torch.isfinite(q).numpy()
+        got = O.encode_e2m1_rne(q).numpy()[keep]
+        qd = xd[keep] / float(scale.double())
+        exp = brute_force_rne(np.abs(qd)) | np.where(np.signbit(xd[keep]), 8, 0)
+        assert np.array_equal(got, exp), f"scale {s}"
+
+
+def test_rne_ties_and_specials():
+    q = torch.tensor([0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5.0, 6.0, 100.0, float("inf"), -0.0, -0.25, -0.26, 0.0])
+    exp = [0, 2, 2, 4, 4, 6, 6, 7, 7, 7, 8, 8, 9, 0]
+    assert O.encode_e2m1_rne(q).tolist() == exp
+    assert [S.encode_rne(float(v)) for v in q] == exp
+
+
+def test_seven_encodes_to_eight():
+    x = torch.zeros(1, 32, dtype=torch.bfloat16)
+    x[0, 5] = 7.0
+    c, s = O.quantize(x)
+    assert int(s[0, 0]) == 128
+    d = O.dequantize(c, s, torch.float32)
+    assert float(d[0, 5]) == 8.0
+
+
+# ----------------------------------------------------------------------------- Q3 / Q6 pack + decode
+def test_pack_closed_form_and_roundtrip():
+    codes = torch.arange(16, dtype=torch.uint8).repeat(2, 4)
+    p = O.pack_nibbles(codes)
+    assert p.shape == (2, 32)
+    for j in range(32):
+        assert int(p[0, j]) == int(codes[0, 2 * j]) | (int(codes[0, 2 * j + 1]) << 4)
+    assert torch.equal(O.unpack_nibbles(p), codes)
+
+
+def test_decode_table():
+    vals = O.decode_e2m1(torch.arange(16, dtype=torch.uint8))
+    exp = list(O.E2M1_GRID) + [-v for v in O.E2M1_GRID]
+    assert vals.tolist() == exp
+    assert math.copysign(1.0, float(vals[8])) == -1.0  # 0x8 is -0
+    assert [S.decode(c) for c in range(16)] == exp
+
+
+def test_grid_values_roundtrip_all_scales():
+    grid = torch.tensor(O.E2M1_GRID[1:])
+    for s in [1, 60, 127, 200, 250]:
+        sc = float(torch.tensor([s], dtype=torch.int32).bitwise_left_shift(23).view(torch.float32))
+        v = torch.cat([grid, -grid]) * sc
+        codes = O.encode_e2m1_rne(v / sc)
+        assert torch.equal(O.decode_e2m1(codes) * sc, v)
+
+
+# ----------------------------------------------------------------------------- Q4 SR
+def test_sr_matches_scalar_model_random():
+    g = torch.Generator().manual_seed(11)
+    q = torch.cat([torch.rand(3000, generator=g) * 7.0, torch.rand(2000, generator=g), torch.rand(1000, generator=g) * 1e-3,
+                   torch.tensor([0.0, 0.5, 1.0, 0.4999999, 5.9999995, 6.0, 1.5, 3.0])])
+    q = q * (torch.randint(0, 2, q.shape, generator=g) * 2 - 1).float()
+    r = torch.randint(0, 2 ** 32, q.shape, generator=g, dtype=torch.int64)
+    r[:8] = torch.tensor([0, 0xFFFFFFFF, 0x3FFFFF, 0x400000, 1, 2 ** 31, 2 ** 31 - 1, 0xFFC00000])
+    got = O.encode_e2m1_sr(q, r).tolist()
+    exp = [S.encode_sr(float(a), int(b)) for a, b in zip(q, r)]
+    assert got == exp
+
+
+def test_sr_result_is_a_grid_neighbour():
+    g = torch.Generator().manual_seed(12)
+    q = torch.rand(20000, generator=g) * 6.5
+    r = torch.randint(0, 2 ** 32, q.shape, generator=g, dtype=torch.int64)
+    v = O.decode_e2m1(O.encode_e2m1_sr(q, r)).double().numpy()
+    grid = np.array(O.E2M1_GRID)
+    qn = np.minimum(q.double().numpy(), 6.0)
+    lo = grid[np.searchsorted(grid, qn, side="right") - 1]
+    hi = grid[np.minimum(np.searchsorted(grid, qn, side="left"), 7)]
+    assert np.all((v == lo) | (v == hi))
+
+
+def test_sr_extreme_random_words():
+    q = torch.tensor([0.0, 0.1, 0.3, 0.5, 0.6, 0.99, 1.0, 1.1, 2.0, 2.7, 4.0, 5.5])
+    zero = torch.zeros(q.shape, dtype=torch.int64)
+    ones = torch.full(q.shape, 0xFFFFFFFF, dtype=torch.int64)
+    # r = 0: subnormal lane always rounds UP (q=0 -> 0.5, because the compare is <=); normal lane truncates
+    assert O.decode_e2m1(O.encode_e2m1_sr(q, zero)).tolist() == [0.5, 0.5, 0.5, 1.0, 1.0, 1.0, 1.0, 1.0, 2.0, 2.0, 4.0, 4.0]
+    # r = all ones: subnormal lane rounds DOWN, normal lane rounds up unless exactly representable
+    assert O.decode_e2m1(O.encode_e2m1_sr(q, ones)).tolist() == [0.0, 0.0, 0.0, 0.5, 0.5, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0]
+
+
+def test_sr_counting_identity_normal_lane():
+    # for fixed normal q the number of r in [0, 2^22) that round up equals low22(bits(q))
+    for qv in [1.0, 1.1, 1.4999999, 2.3, 3.9, 5.2]:
+        b = S.f32_bits(qv)
+        low = b & 0x3FFFFF
+        r = torch.arange(0, 2 ** 22, dtype=torch.int64)
+        codes = O.encode_e2m1_sr(torch.full((2 ** 22,), qv), r)
+        base = int(codes.min())
+        assert int((codes != base).sum()) == low
+        assert set(codes.unique().tolist()) <= {base, base + 1}
+
+
+def test_sr_counting_identity_subnormal_lane():
+    # number of 32-bit words giving round-up equals threshold + 1: check by locating the switch point
+    for qv in [0.0, 0.1, 0.3, 0.49, 0.5, 0.7, 0.99]:
+        m = S.to_f32(qv)
+        t = int(S.to_f32(m * 2.0 ** 33)) if m < 0.5 else int(S.to_f32((m * 2 - 1) * 2.0 ** 32))
+        base = 0 if m < 0.5 else 1
+        probe = torch.tensor([0, max(t - 1, 0), t, min(t + 1, 0xFFFFFFFF), 0xFFFFFFFF], dtype=torch.int64)
+        codes = O.encode_e2m1_sr(torch.full((5,), m), probe).tolist()
+        exp = [base + 1, base + 1, base + 1, base + (1 if t + 1 <= t or t == 0xFFFFFFFF else 0), base + (1 if t == 0xFFFFFFFF else 0)]
+        assert codes == exp, (qv, codes, exp)
+
+
+def test_sr_unbiased():
+    g = torch.Generator().manual_seed(13)
+    for qv in [0.2, 0.8, 1.3, 2.6, 4.7]:
+        r = torch.randint(0, 2 ** 32, (400000,), generator=g, dtype=torch.int64)
+        v = O.decode_e2m1(O.encode_e2m1_sr(torch.full((400000,), qv), r)).double().mean()
+        assert abs(float(v) - qv) < 0.01
+
+
+# ----------------------------------------------------------------------------- Q5 layouts + scalar cross-check
+def test_axis_layouts_match_reference_contract():
+    x = torch.randn(64, 128).bfloat16()
+    c, s = O.quantize(x, axis=0)
+    assert c.shape == (32, 128) and c.stride() == (1, 32)      # memory [C][M/2]
+    assert s.shape == (2, 128) and s.stride() == (1, 2)        # memory [C][M/32]
+    c, s = O.quantize(x, axis=-1, is_2d_block=True)
+    assert c.shape == (64, 64) and s.shape == (2, 4)
+    x3 = torch.randn(4, 128, 64)
+    c, s = O.quantize(x3, axis=-2, is_2d_block=True)
+    assert c.shape == (4, 64, 64) and s.shape == (4, 4, 2)
+    c, s = O.quantize(x3, axis=-2)
+    assert c.shape == (4, 64, 64) and s.shape == (4, 4, 64)
+
+
+def test_2d_quantisation_commutes_with_transpose():
+    x = torch.randn(96, 64).bfloat16()
+    c1, s1 = O.quantize(x, axis=-1, is_2d_block=True)
+    c2, s2 = O.quantize(x, axis=0, is_2d_block=True)
+    assert torch.equal(s1, s2)
+    assert torch.equal(O.dequantize(c1, s1, axis=-1, is_2d_block=True), O.dequantize(c2, s2, axis=0, is_2d_block=True))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("sr", [False, True])
+def test_quantize_rows_vs_scalar_model(dtype, sr):
+    g = torch.Generator().manual_seed(21)
+    x = torch.randn(6, 64, generator=g)
+    x[0, 3] *= 50
+    x[1] *= 1e-30
+    x[2, :32] = 0
+    x[3] *= 1e30
+    x = x.to(dtype)
+    r = torch.randint(0, 2 ** 32, x.shape, generator=g, dtype=torch.int64)
+    c, s = O.quantize(x, use_sr=sr, rand_bits=r if sr else None)
+    for row in range(x.shape[0]):
+        if dtype == torch.bfloat16:
+            bits = (x[row].view(torch.int16).to(torch.int32) & 0xFFFF).tolist()
+            mb = 7
+        else:
+            bits = (x[row].view(torch.int32).to(torch.int64) & 0xFFFFFFFF).tolist()
+            mb = 23
+        eb, es = S.quantize_row_1d(bits, mb, rne=not sr, rand=r[row].tolist())
+        assert c[row].tolist() == eb
+        assert s[row].tolist() == es
+
+
+def test_static_clip_and_uos_closed_forms():
+    x = torch.zeros(1, 32, dtype=torch.bfloat16)
+    x[0, 0] = 6.0
+    c, s = O.quantize(x, clip_mode="static")
+    assert int(s[0, 0]) == 127 and int(c[0, 0]) & 0xF == 6   # 4.5 -> tie between 4 and 6 -> even code 6 (4.0)
+    d = O.dequantize(c, s, torch.float32, clip_mode="static")
+    assert abs(float(d[0, 0]) - 4.0 * 4 / 3) < 1e-6
+    x[0, 0] = 7.25
+    c, s = O.quantize(x, use_uos=True)
+    assert int(s[0, 0]) == 127
+    x[0, 0] = 7.3
+    c, s = O.quantize(x, use_uos=True)
+    assert int(s[0, 0]) == 128
+    with pytest.raises(ValueError):
+        O.quantize(x, clip_mode="bogus")
+
+
+# ----------------------------------------------------------------------------- Q7 Hadamard
+def test_hadamard_matrix_properties():
+    g = torch.Generator().manual_seed(1234)
+    signs = torch.randint(0, 2, (32,), generator=g) * 2 - 1
+    perm = torch.randperm(32, generator=g)
+    W = O.hadamard_matrix(signs, perm)
+    assert torch.equal(W.T @ W, 32 * torch.eye(32))
+    for i in [0, 5, 31]:
+        for j in [0, 7, 30]:
+            pi, pj = int(perm[i]), int(perm[j])
+            assert float(W[i, j]) == float(signs[pi]) * (-1) ** bin(pi & pj).count("1")
+    W0 = O.hadamard_matrix(torch.ones(32), None)
+    H = torch.tensor([[1.0]])
+    for _ in range(5):
+        H = torch.vstack((torch.hstack((H, H)), torch.hstack((H, -H))))   # Sylvester
+    assert torch.equal(W0, H)
+
+
+def test_rht_butterfly_vs_dense_fp64():
+    g = torch.Generator().manual_seed(5)
+    signs = torch.randint(0, 2, (32,), generator=g) * 2 - 1
+    perm = torch.randperm(32, generator=g)
+    x = (torch.randn(128, 48, generator=g) * 1e-3).bfloat16()
+    y = O.rht_left(x, signs, perm)
+    yd = O.rht_left_dense(x, signs, perm, torch.float64)
+    ulp = torch.exp2(torch.floor(torch.log2(yd.abs().clamp_min(1e-30))) - 7)
+    assert bool(((y.double() - yd).abs() <= ulp).all())
+    # exactly representable sums: integer-valued inputs give identical results whatever the order
+    xi = torch.randint(-8, 9, (64, 16), generator=g).bfloat16()
+    assert torch.equal(O.rht_left(xi, signs, perm), O.rht_left_dense(xi, signs, perm, torch.float32).bfloat16())
+
+
+def test_rht_preserves_wgrad_product():
+    g = torch.Generator().manual_seed(6)
+    signs = torch.randint(0, 2, (32,), generator=g) * 2 - 1
+    perm = torch.randperm(32, generator=g)
+    a = torch.randn(64, 8, generator=g, dtype=torch.float64)
+    b = torch.randn(64, 12, generator=g, dtype=torch.float64)
+    ha = O.rht_left_dense(a, signs, perm, torch.float64)
+    hb = O.rht_left_dense(b, signs, perm, torch.float64)
+    assert torch.allclose(ha.T @ hb, a.T @ b, atol=1e-9)
+
+
+# ----------------------------------------------------------------------------- Q8-Q10 GEMM
+def test_gemm_ref_vs_exact_rational_bruteforce():
+    g = torch.Generator().manual_seed(9)
+    M, N, K = 4, 3, 64
+    a_q = torch.randint(0, 256, (M, K // 2), generator=g, dtype=torch.uint8)
+    b_q = torch.randint(0, 256, (N, K // 2), generator=g, dtype=torch.uint8)
+    a_s = torch.randint(120, 135, (M, K // 32), generator=g, dtype=torch.uint8)
+    b_s = torch.randint(120, 135, (N, K // 32), generator=g, dtype=torch.uint8)
+    got = O.gemm_ref(a_q, a_s, b_q, b_s, trans_b=True)
+    for i in range(M):
+        for j in range(N):
+            acc = Fraction(0)
+            for k in range(K):
+                ca = (int(a_q[i, k // 2]) >> (4 * (k % 2))) & 15
+                cb = (int(b_q[j, k // 2]) >> (4 * (k % 2))) & 15
+                acc += Fraction(S.decode(ca)) * Fraction(S.decode(cb)) * Fraction(2) ** (int(a_s[i, k // 32]) - 127 + int(b_s[j, k // 32]) - 127)
+            assert float(acc) == float(got[i, j])
+
+
+def test_gemm_ref_flag_orientations_agree():
+    g = torch.Generator().manual_seed(10)
+    a = torch.randn(64, 96, generator=g).bfloat16()
+    b = torch.randn(32, 96, generator=g).bfloat16()
+    aq, as_ = O.quantize(a)
+    bq, bs = O.quantize(b)
+    ref = O.gemm_ref(aq, as_, bq, bs, trans_b=True)
+    # same operands presented as transposed views
+    assert torch.equal(O.gemm_ref(aq.T, as_.T, bq, bs, trans_a=True, trans_b=True), ref)
+    assert torch.equal(O.gemm_ref(aq, as_, bq.T, bs.T), ref)
+    # 2D weight: packed along K or along N gives the same dequantized matrix
+    w = torch.randn(64, 96, generator=g).bfloat16()
+    wq, ws = O.quantize(w, is_2d_block=True)
+    go = torch.randn(32, 64, generator=g).bfloat16()
+    gq, gs = O.quantize(go)
+    dx1 = O.gemm_ref(gq, gs, wq, ws, use_2dblock_b=True, k_pack_b=False)        # reference dgrad call shape
+    wq_t, ws_t = O.quantize(w, axis=0, is_2d_block=True)
+    dx2 = O.gemm_ref(gq, gs, wq_t, ws_t, use_2dblock_b=True, k_pack_b=True)
+    assert torch.equal(dx1, dx2)
+
+
+def test_linear_reference_snr_floors():
+    # the reference's own acceptance floors (tests/unittest/mxfp4/test_mxfp_linear.py:189-197) hold for the oracle
+    g = torch.Generator().manual_seed(1234)
+    x = torch.randn(256, 128, generator=g)
+    w = torch.randn(96, 128, generator=g)
+    go = torch.randn(256, 96, generator=g)
+    signs = torch.randint(0, 2, (32,), generator=g) * 2 - 1
+    perm = torch.randperm(32, generator=g)
+    r = torch.randint(0, 2 ** 32, go.shape, generator=g, dtype=torch.int64)
+    y, saved = O.linear_forward_ref(x.bfloat16(), w.bfloat16(), hadamard=(signs, perm))
+    dx, dw = O.linear_backward_ref(go.bfloat16(), saved, use_sr_grad=True, rand_bits=r, hadamard=(signs, perm))
+
+    def snr(ref, got):
+        return float(10 * torch.log10((ref.double() ** 2).sum() / ((ref.double() - got.double()) ** 2).sum()))
+    assert snr(x @ w.T, y) > 8.4
+    assert snr(go @ w, dx) > 6.9
+    assert snr(go.T @ x, dw) > 6.9
+
+
+def test_grouped_reference_and_offsets():
+    offs = torch.tensor([128, 128, 384, 512], dtype=torch.int32)  # expert 1 is empty
+    idx = O.indices_from_offsets(offs)
+    assert idx.shape == (512,) and idx.dtype == torch.int32
+    assert idx[:128].eq(0).all() and idx[128:384].eq(2).all() and idx[384:].eq(3).all()
+    g = torch.Generator().manual_seed(2)
+    a = torch.randn(512, 64, generator=g).bfloat16()
+    w = torch.randn(4, 32, 64, generator=g).bfloat16()
+    aq, as_ = O.quantize(a)
+    wq, ws = O.quantize(w, axis=-1, is_2d_block=True)
+    out = O.grouped_gemm_ref(aq, as_, wq, ws, idx)
+    for e, (lo, hi) in enumerate([(0, 128), (128, 128), (128, 384), (384, 512)]):
+        if hi > lo:
+            ref = O.gemm_ref(aq[lo:hi], as_[lo:hi], wq[e], ws[e], use_2dblock_b=True, trans_b=True)
+            assert torch.equal(out[lo:hi], ref)
+    # [E, K, N] storage (torchtitan layout, trans_weights=False) gives the same result
+    wt = w.transpose(-1, -2).contiguous()
+    wq2, ws2 = O.quantize(wt, axis=-2, is_2d_block=True)
+    assert torch.equal(O.grouped_gemm_ref(aq, as_, wq2, ws2, idx, trans_weights=False), out)
