@@ -1,0 +1,74 @@
+"""ctypes binding of libalto_mxfp4.so (the C ABI declared in include/alto_mxfp4.h).
+
+The product path has no CPU fallback: if the library is missing or a call fails, an exception is raised.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import threading
+
+from . import build as _build
+
+_lock = threading.Lock()
+_lib = None
+
+c_i64 = ctypes.c_int64
+c_int = ctypes.c_int
+c_vp = ctypes.c_void_p
+c_f32 = ctypes.c_float
+
+# name -> (restype, argtypes); mirrors include/alto_mxfp4.h
+SIGNATURES = {
+    "alto_mxfp4_version": (c_int, []),
+    "alto_mxfp4_last_error": (ctypes.c_char_p, []),
+    "alto_mxfp4_quantize": (c_int, [c_vp, c_int, c_i64, c_i64, c_i64, c_i64, c_i64,
+                                    c_vp, c_vp, c_vp, c_vp,
+                                    c_int, c_int, c_vp, c_i64, c_i64,
+                                    c_int, c_vp, c_vp, c_int, c_int, c_vp]),
+    "alto_mxfp4_hadamard": (c_int, [c_vp, c_int, c_i64, c_i64, c_i64, c_vp, c_i64, c_vp, c_vp, c_vp]),
+    "alto_mxfp4_dequantize": (c_int, [c_vp, c_vp, c_i64, c_i64, c_int, c_vp, c_int, c_i64, c_i64, c_int, c_vp]),
+    "alto_mxfp4_transpose_codes": (c_int, [c_vp, c_i64, c_i64, c_vp, c_vp]),
+    "alto_mxfp4_gemm": (c_int, [c_vp, c_i64, c_vp, c_i64, c_i64, c_int,
+                                c_vp, c_i64, c_vp, c_i64, c_i64, c_int,
+                                c_i64, c_i64, c_i64, c_vp, c_int, c_i64, c_f32, c_vp]),
+    "alto_mxfp4_grouped_gemm": (c_int, [c_vp, c_i64, c_vp, c_i64, c_i64, c_int,
+                                        c_vp, c_i64, c_i64, c_vp, c_i64, c_i64, c_i64, c_int,
+                                        c_vp, c_vp, c_int, c_int, c_i64, c_i64, c_i64, c_vp, c_int, c_i64, c_vp]),
+    "alto_mxfp4_grouped_gemm_dw": (c_int, [c_vp, c_i64, c_vp, c_i64, c_i64,
+                                           c_vp, c_i64, c_vp, c_i64, c_i64,
+                                           c_vp, c_vp, c_int, c_int, c_i64, c_i64, c_i64,
+                                           c_vp, c_int, c_i64, c_i64, c_i64, c_f32, c_vp]),
+}
+
+
+class AltoMxfp4Error(RuntimeError):
+    pass
+
+
+def load():
+    """Load the in-tree shared library (building it first only when it does not exist)."""
+    global _lib
+    with _lock:
+        if _lib is not None:
+            return _lib
+        path = _build.lib_path()
+        if not os.path.exists(path):
+            _build.build(verbose=False)
+        lib = ctypes.CDLL(path)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(lib, name)  # AttributeError if the ABI and the header drifted apart
+            fn.restype = res
+            fn.argtypes = args
+        _lib = lib
+        return lib
+
+
+def check(rc: int, what: str) -> None:
+    if rc != 0:
+        msg = load().alto_mxfp4_last_error().decode("utf-8", "replace")
+        if rc == -1:
+            raise AssertionError(f"{what}: {msg}")
+        if rc == -3:
+            raise NotImplementedError(f"{what}: {msg}")
+        raise AltoMxfp4Error(f"{what} failed with code {rc}: {msg}")

@@ -1,0 +1,94 @@
+// Shared device/host helpers for the MXFP4 kernels (gfx950 only).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdarg.h>
+
+#include "../../include/alto_mxfp4.h"
+
+namespace alto {
+
+// ----------------------------------------------------------------------------- host: error reporting
+void set_error(const char* fmt, ...);
+int check_launch(const char* what);
+
+#define ALTO_REQUIRE(cond, ...)            \
+  do {                                     \
+    if (!(cond)) {                         \
+      alto::set_error(__VA_ARGS__);        \
+      return ALTO_MXFP4_EINVAL;            \
+    }                                      \
+  } while (0)
+
+// ----------------------------------------------------------------------------- device: bit casts
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef int v8i_t __attribute__((ext_vector_type(8)));
+typedef float v4f_t __attribute__((ext_vector_type(4)));
+typedef float v16f_t __attribute__((ext_vector_type(16)));
+
+__device__ __forceinline__ uint32_t f2u(float f) { return __builtin_bit_cast(uint32_t, f); }
+__device__ __forceinline__ float u2f(uint32_t u) { return __builtin_bit_cast(float, u); }
+__device__ __forceinline__ float bf16_lo(uint32_t w) { return u2f(w << 16); }
+__device__ __forceinline__ float bf16_hi(uint32_t w) { return u2f(w & 0xFFFF0000u); }
+
+// fp32 -> bf16 bits, round to nearest even (finite inputs; NaN payloads are not preserved specially)
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
+  uint32_t u = f2u(f);
+  return (u + 0x7FFFu + ((u >> 16) & 1u)) >> 16;
+}
+
+// ----------------------------------------------------------------------------- device: E8M0 scale rule
+// Biased exponent of the block absmax after rounding it to one mantissa bit, minus 2, clamped below at 1.
+__device__ __forceinline__ uint32_t e8m0_from_bf16_bits(uint32_t absbits16) {
+  uint32_t e = ((absbits16 + 0x20u) >> 7) & 0x1FFu;
+  return e > 3u ? e - 2u : 1u;
+}
+__device__ __forceinline__ uint32_t e8m0_from_f32_bits(uint32_t absbits32) {
+  uint32_t e = ((absbits32 + 0x200000u) >> 23) & 0x1FFu;
+  return e > 3u ? e - 2u : 1u;
+}
+// "UOS" rule: ceil(log2(absmax / 7.25)) + 127, all-zero block -> 128, clamped below at 1.
+__device__ __forceinline__ uint32_t e8m0_uos(float absmax) {
+  float s = ceilf(log2f(absmax / 7.25f));
+  if (absmax == 0.0f) s = 1.0f;
+  s += 127.0f;
+  if (s < 1.0f) s = 1.0f;
+  return (uint32_t)s & 0xFFu;
+}
+
+// ----------------------------------------------------------------------------- device: E2M1 encode
+// Stochastic rounding of a non-negative magnitude m (already divided by the scale) with 32 random bits.
+// Returns the 3-bit code (0..7).
+__device__ __forceinline__ uint32_t e2m1_sr_mag(float m, uint32_t r) {
+  uint32_t mb = f2u(m);
+  // normal lane: add the low 22 random bits under the kept mantissa bit, truncate, saturate at 7
+  uint32_t n = mb - 0x3F000000u + (r & 0x3FFFFFu);
+  n = (n < 0x01FFFFFFu ? n : 0x01FFFFFFu) >> 22;
+  // subnormal lane: threshold compare with 32-bit resolution; g = 2m in [0, 2)
+  float g = m + m;
+  float fr = __builtin_amdgcn_fractf(g);
+  uint32_t thr = (uint32_t)__builtin_ldexpf(fr, 32);
+  uint32_t den = (g >= 1.0f ? 1u : 0u) + (r <= thr ? 1u : 0u);
+  return m < 1.0f ? den : n;
+}
+
+// Round-to-nearest-even of a non-negative magnitude; software form (used where the packed HW convert does not fit).
+__device__ __forceinline__ uint32_t e2m1_rne_mag(float m) {
+  uint32_t mb = f2u(m);
+  uint32_t n = mb - 0x3F000000u + 0x1FFFFFu + ((mb >> 22) & 1u);
+  n = (n < 0x01FFFFFFu ? n : 0x01FFFFFFu) >> 22;
+  uint32_t den = f2u(m + 4194304.0f) - 0x4A800000u;
+  return m < 1.0f ? den : n;
+}
+
+// ----------------------------------------------------------------------------- device: cross-lane
+template <int CTRL>
+__device__ __forceinline__ uint32_t dpp_u32(uint32_t v) {
+  return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xF, 0xF, true);
+}
+// quad_perm controls: lane ^ 1 and lane ^ 2 inside each group of 4 lanes
+#define ALTO_DPP_QUAD_XOR1 0xB1
+#define ALTO_DPP_QUAD_XOR2 0x4E
+
+}  // namespace alto

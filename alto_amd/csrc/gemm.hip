@@ -1,0 +1,53 @@
+// Block-scaled MXFP4 GEMM entry point (dense): C[M][N] = A[M][K] . B[N][K]^T on gfx950 scaled MFMA.
+#include "common.h"
+#include "gemm_simple.h"
+#include "gemm_tiled.h"
+
+namespace alto {
+namespace {
+
+template <typename OutT>
+__global__ __launch_bounds__(256) void gemm_simple_kernel(OperandView A, OperandView B, int64_t M, int64_t N, int G,
+                                                          OutT* c, int64_t ldc, float out_scale) {
+  const int wave = threadIdx.x >> 6;
+  const int64_t m0 = (int64_t)blockIdx.y * 64 + (wave >> 1) * 32;
+  const int64_t n0 = (int64_t)blockIdx.x * 64 + (wave & 1) * 32;
+  if (m0 >= M || n0 >= N) return;
+  v16f_t acc = mma_tile_32x32(A, B, m0, n0, 0, M, N, 0, G);
+  store_tile_32x32<OutT>(acc, c, ldc, m0, n0, 0, M, N, out_scale);
+}
+
+}  // namespace
+}  // namespace alto
+
+extern "C" int alto_mxfp4_gemm(const uint8_t* a, int64_t lda, const uint8_t* a_scales, int64_t a_ss_r, int64_t a_ss_k, int a_is_2d,
+                               const uint8_t* b, int64_t ldb, const uint8_t* b_scales, int64_t b_ss_r, int64_t b_ss_k, int b_is_2d,
+                               int64_t M, int64_t N, int64_t K, void* c, int c_dtype, int64_t ldc, float out_scale, void* stream) {
+  using namespace alto;
+  ALTO_REQUIRE(a && b && a_scales && b_scales && c, "gemm: NULL pointer");
+  ALTO_REQUIRE(M >= 0 && N >= 0 && K >= 0, "gemm: negative size");
+  ALTO_REQUIRE(K % 32 == 0, "gemm: K (%lld) must be a multiple of 32", (long long)K);
+  ALTO_REQUIRE(!a_is_2d || M % 32 == 0, "gemm: 2D scales for A need M (%lld) %% 32 == 0", (long long)M);
+  ALTO_REQUIRE(!b_is_2d || N % 32 == 0, "gemm: 2D scales for B need N (%lld) %% 32 == 0", (long long)N);
+  ALTO_REQUIRE(lda >= K / 2 && ldb >= K / 2 && lda % 16 == 0 && ldb % 16 == 0, "gemm: lda/ldb must be >= K/2 and multiples of 16 bytes");
+  ALTO_REQUIRE(((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b)) & 15) == 0, "gemm: a and b must be 16-byte aligned");
+  ALTO_REQUIRE(ldc >= N, "gemm: ldc < N");
+  ALTO_REQUIRE(c_dtype == ALTO_DT_BF16 || c_dtype == ALTO_DT_F32, "gemm: bad c_dtype %d", c_dtype);
+  ALTO_REQUIRE(M < (1ll << 31) && N < (1ll << 31) && K < (1ll << 31), "gemm: size out of range");
+  if (M == 0 || N == 0) return ALTO_MXFP4_OK;
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  OperandView A{a, lda, a_scales, a_ss_r, a_ss_k, a_is_2d};
+  OperandView B{b, ldb, b_scales, b_ss_r, b_ss_k, b_is_2d};
+
+  if (gemm_tiled_supported(A, B, M, N, K, c, c_dtype, ldc)) {
+    gemm_tiled_launch(A, B, M, N, K, c, c_dtype, ldc, out_scale, st);
+    return check_launch("gemm(tiled)");
+  }
+  dim3 grid((unsigned)((N + 63) / 64), (unsigned)((M + 63) / 64));
+  ALTO_REQUIRE(grid.y <= 65535u, "gemm: M too large for the fallback kernel");
+  if (c_dtype == ALTO_DT_BF16)
+    hipLaunchKernelGGL(gemm_simple_kernel<__bf16>, grid, dim3(256), 0, st, A, B, M, N, (int)(K / 32), (__bf16*)c, ldc, out_scale);
+  else
+    hipLaunchKernelGGL(gemm_simple_kernel<float>, grid, dim3(256), 0, st, A, B, M, N, (int)(K / 32), (float*)c, ldc, out_scale);
+  return check_launch("gemm");
+}

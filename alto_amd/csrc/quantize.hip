@@ -1,0 +1,449 @@
+// Fused MXFP4 quantizer for gfx950.
+//
+// One workgroup (256 threads) owns a tile of 32 rows x 256 columns of a row-major matrix and can emit,
+// from a single read of the tile,
+//   * the row output  (blocks of 32 along the contiguous dim):   codes [M][C/2], scales [M][C/32]
+//   * the column output (blocks of 32 along the row dim):        codes [C][M/2], scales [C][M/32]
+//     optionally preceded by the randomized 32-point Hadamard transform along the row dim
+//   * or, for 2D 32x32 blocks, both packings with one shared scale per block.
+//
+// Row phase: a lane holds 8 consecutive elements (one 128-bit load for bf16); 4 lanes form one MX block,
+// so the block absmax is two DPP quad steps.  The raw tile is parked in LDS (at a permuted row when the
+// Hadamard permutation is active).  Column phase: thread t owns column t of the tile and reads its 32 rows
+// from LDS, so the transform, the absmax and the packing along rows are all in-thread.
+#include "common.h"
+
+namespace alto {
+namespace {
+
+constexpr int TILE_C = 256;
+constexpr int STAGE_PITCH = 9;  // dwords per thread in the private byte-permutation scratch (36 B: conflict-free)
+
+struct QuantParams {
+  const void* x;
+  int64_t ld_x, bs_x;
+  int M, C;
+  const uint32_t* rand;
+  int64_t ld_r, bs_r;
+  uint8_t* row_codes;
+  uint8_t* row_scales;
+  uint8_t* col_codes;
+  uint8_t* col_scales;
+  uint32_t sign_mask;    // bit k set: Q[k] == -1 (k = position after the permutation)
+  uint8_t perm[32];      // row j of a block -> position perm[j]
+  uint8_t perm_inv[32];  // position k -> row
+  int clip_row;          // 1: multiply by 3/4 (in the input dtype) before encoding the row output
+  int clip_col;
+  int uos;
+};
+
+typedef unsigned short us2_t __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ uint32_t pk_max_u16(uint32_t a, uint32_t b) {
+  us2_t r = __builtin_elementwise_max(__builtin_bit_cast(us2_t, a), __builtin_bit_cast(us2_t, b));
+  return __builtin_bit_cast(uint32_t, r);
+}
+
+// z / float32(sqrt(32)) correctly rounded, without the full division sequence: one Newton correction with FMAs.
+__device__ __forceinline__ float div_sqrt32(float z) {
+  const float c = 5.656854152679443f;
+  const float rc = 0.17677669529663689f;  // nearest fp32 to 1/c
+  float q = z * rc;
+  float r = __builtin_fmaf(-q, c, z);
+  r = __builtin_fmaxf(r, -3.0e38f);  // z = +-inf gives r = NaN: drop it so that the quotient stays +-inf like a true division
+  return __builtin_fmaf(r, rc, q);
+}
+
+// (z * sign) / float32(sqrt(32)) with `flip` = 0 or 0x80000000.  The sign of the quotient is taken from the dividend so
+// that signed zeros come out as a true division gives them (the FMA correction alone would turn -0 into +0).
+__device__ __forceinline__ float div_sqrt32_signed(float z, uint32_t flip) {
+  uint32_t q = f2u(div_sqrt32(z));
+  uint32_t s = f2u(z) ^ flip;
+  return u2f((q & 0x7FFFFFFFu) | (s & 0x80000000u));
+}
+
+template <typename T>
+__device__ __forceinline__ float round_to_T(float v) {
+  if constexpr (sizeof(T) == 2) return u2f(f32_to_bf16_bits(v) << 16);
+  return v;
+}
+
+template <typename T, bool DO_ROW, bool DO_COL, bool SR, bool RHT, bool B2D, bool GEN>
+__global__ __launch_bounds__(256) void quant_kernel(const QuantParams p) {
+  constexpr bool BF = sizeof(T) == 2;
+  __shared__ __align__(16) T tile[DO_COL ? 32 * TILE_C : 8];
+  __shared__ uint32_t blkmax[8];
+  __shared__ uint32_t stage[(DO_COL && RHT) ? 256 * STAGE_PITCH : 1];
+  __shared__ uint8_t sperm[32];
+
+  const int tid = threadIdx.x;
+  const int col0 = blockIdx.x * TILE_C;
+  const int row0 = blockIdx.y * 32;
+  const int64_t b = blockIdx.z;
+  const int M = p.M, C = p.C;
+
+  if (RHT || B2D) {
+    if (tid == 0) {
+#pragma unroll
+      for (int k = 0; k < 32; ++k) sperm[k] = p.perm[k];
+    }
+    if (tid < 8) blkmax[tid] = 0;
+    __syncthreads();
+  }
+
+  const T* xb = reinterpret_cast<const T*>(p.x) + b * p.bs_x;
+  const uint32_t* rb = SR ? p.rand + b * p.bs_r : nullptr;
+
+  // ------------------------------------------------------------------ row phase
+  const int chunk = tid & 31;
+  const int c = col0 + chunk * 8;
+  uint32_t w[4][BF ? 4 : 8];
+  uint32_t amax_i[4];
+  bool valid[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = (tid >> 5) + 8 * i;
+    valid[i] = (row0 + r < M) && (c < C);
+    if (valid[i]) {
+      const uint4* src = reinterpret_cast<const uint4*>(xb + (int64_t)(row0 + r) * p.ld_x + c);
+      uint4 v0 = src[0];
+      w[i][0] = v0.x; w[i][1] = v0.y; w[i][2] = v0.z; w[i][3] = v0.w;
+      if constexpr (!BF) {
+        uint4 v1 = src[1];
+        w[i][4] = v1.x; w[i][5] = v1.y; w[i][6] = v1.z; w[i][7] = v1.w;
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < (BF ? 4 : 8); ++e) w[i][e] = 0;
+    }
+    if (DO_COL) {
+      const int pos = RHT ? sperm[r] : r;
+      uint4* dst = reinterpret_cast<uint4*>(&tile[pos * TILE_C + chunk * 8]);
+      dst[0] = make_uint4(w[i][0], w[i][1], w[i][2], w[i][3]);
+      if constexpr (!BF) dst[1] = make_uint4(w[i][4], w[i][5], w[i][6], w[i][7]);
+    }
+    if (DO_ROW || B2D) {
+      uint32_t a;
+      if constexpr (BF) {
+        a = pk_max_u16(pk_max_u16(w[i][0] & 0x7FFF7FFFu, w[i][1] & 0x7FFF7FFFu),
+                       pk_max_u16(w[i][2] & 0x7FFF7FFFu, w[i][3] & 0x7FFF7FFFu));
+        a = max(a & 0xFFFFu, a >> 16);
+      } else {
+        a = 0;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) a = max(a, w[i][e] & 0x7FFFFFFFu);
+      }
+      a = max(a, dpp_u32<ALTO_DPP_QUAD_XOR1>(a));
+      a = max(a, dpp_u32<ALTO_DPP_QUAD_XOR2>(a));
+      amax_i[i] = a;
+      if (B2D && (tid & 3) == 0) atomicMax(&blkmax[chunk >> 2], a);
+    }
+  }
+  if (B2D || DO_COL) __syncthreads();
+
+  if (DO_ROW || B2D) {
+    uint32_t blk = B2D ? blkmax[chunk >> 2] : 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int r = (tid >> 5) + 8 * i;
+      const uint32_t a = B2D ? blk : amax_i[i];
+      uint32_t s;
+      if (GEN && p.uos) s = e8m0_uos(BF ? u2f(a << 16) : u2f(a));
+      else s = BF ? e8m0_from_bf16_bits(a) : e8m0_from_f32_bits(a);
+      if (!valid[i]) continue;
+      const int64_t row = row0 + r;
+      // scales
+      if ((tid & 3) == 0) {
+        if (!B2D) {
+          if (DO_ROW) p.row_scales[(b * M + row) * (C / 32) + (c >> 5)] = (uint8_t)s;
+        } else if (r == 0) {
+          if (DO_ROW) p.row_scales[(b * (M / 32) + blockIdx.y) * (C / 32) + (c >> 5)] = (uint8_t)s;
+          if (DO_COL) p.col_scales[(b * (C / 32) + (c >> 5)) * (M / 32) + blockIdx.y] = (uint8_t)s;
+        }
+      }
+      if (!DO_ROW) continue;
+      const float scale_f = u2f(s << 23);
+      float v[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        if constexpr (BF) v[e] = (e & 1) ? bf16_hi(w[i][e >> 1]) : bf16_lo(w[i][e >> 1]);
+        else v[e] = u2f(w[i][e]);
+        if (GEN && p.clip_row) v[e] = round_to_T<T>(v[e] * 0.75f);
+      }
+      uint32_t out = 0;
+      if (!SR) {
+        out = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(out, v[0], v[1], scale_f, 0);
+        out = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(out, v[2], v[3], scale_f, 1);
+        out = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(out, v[4], v[5], scale_f, 2);
+        out = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(out, v[6], v[7], scale_f, 3);
+      } else {
+        const float inv = u2f((254u - s) << 23);
+        const uint4* rs = reinterpret_cast<const uint4*>(rb + row * p.ld_r + c);
+        uint4 r0 = rs[0], r1 = rs[1];
+        uint32_t rr[8] = {r0.x, r0.y, r0.z, r0.w, r1.x, r1.y, r1.z, r1.w};
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          float q = v[e] * inv;
+          uint32_t code = e2m1_sr_mag(__builtin_fabsf(q), rr[e]) | ((f2u(q) >> 28) & 8u);
+          out |= code << (4 * e);
+        }
+      }
+      *reinterpret_cast<uint32_t*>(p.row_codes + (b * M + row) * (C / 2) + (c >> 1)) = out;
+    }
+  }
+
+  // ------------------------------------------------------------------ column phase
+  if (DO_COL) {
+    const int cc = col0 + tid;
+    if (cc >= C) return;
+    float z[32];
+#pragma unroll
+    for (int k = 0; k < 32; ++k) {
+      if (BF) z[k] = u2f((uint32_t)reinterpret_cast<const unsigned short*>(tile)[k * TILE_C + tid] << 16);
+      else z[k] = reinterpret_cast<const float*>(tile)[k * TILE_C + tid];
+    }
+    if (RHT) {
+#pragma unroll
+      for (int h = 1; h < 32; h <<= 1) {
+#pragma unroll
+        for (int k = 0; k < 32; ++k) {
+          if ((k & h) == 0) {
+            float a0 = z[k], a1 = z[k + h];
+            z[k] = a0 + a1;
+            z[k + h] = a0 - a1;
+          }
+        }
+      }
+#pragma unroll
+      for (int k = 0; k < 32; ++k) z[k] = round_to_T<T>(div_sqrt32_signed(z[k], ((p.sign_mask >> k) & 1u) << 31));
+    }
+    uint32_t s;
+    if (B2D) {
+      uint32_t a = blkmax[tid >> 5];
+      if (GEN && p.uos) s = e8m0_uos(BF ? u2f(a << 16) : u2f(a));
+      else s = BF ? e8m0_from_bf16_bits(a) : e8m0_from_f32_bits(a);
+    } else {
+      float am = 0.0f;
+#pragma unroll
+      for (int k = 0; k < 32; ++k) am = __builtin_fmaxf(am, __builtin_fabsf(z[k]));
+      if (GEN && p.uos) s = e8m0_uos(am);
+      else s = BF ? e8m0_from_bf16_bits(f2u(am) >> 16) : e8m0_from_f32_bits(f2u(am));
+      p.col_scales[(b * C + cc) * (M / 32) + blockIdx.y] = (uint8_t)s;
+    }
+    const float scale_f = u2f(s << 23);
+    const float inv = u2f((254u - s) << 23);
+    uint32_t codes[32];
+#pragma unroll
+    for (int k = 0; k < 32; ++k) {
+      float v = z[k];
+      if (GEN && p.clip_col) v = round_to_T<T>(v * 0.75f);
+      if (!SR) {
+        codes[k] = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(0u, v, 0.0f, scale_f, 0) & 0xFu;
+      } else {
+        const int row = RHT ? p.perm_inv[k] : k;
+        uint32_t r = rb[(int64_t)(row0 + row) * p.ld_r + cc];
+        float q = v * inv;
+        codes[k] = e2m1_sr_mag(__builtin_fabsf(q), r) | ((f2u(q) >> 28) & 8u);
+      }
+    }
+    uint32_t out[4];
+    if (RHT) {
+      // undo the permutation: position k belongs to row perm_inv[k]; a private byte scratch in LDS does the indexing
+      uint8_t* sb = reinterpret_cast<uint8_t*>(stage + tid * STAGE_PITCH);
+#pragma unroll
+      for (int k = 0; k < 32; ++k) sb[p.perm_inv[k]] = (uint8_t)codes[k];
+      // same thread reads what it wrote: LDS ops of one wave complete in order, no barrier needed
+      uint32_t d[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) d[j] = stage[tid * STAGE_PITCH + j];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        uint32_t ta = d[2 * j] | (d[2 * j] >> 4);
+        uint32_t tb = d[2 * j + 1] | (d[2 * j + 1] >> 4);
+        out[j] = __builtin_amdgcn_perm(tb, ta, 0x06040200u);
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        uint32_t o = 0;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) o |= codes[8 * j + e] << (4 * e);
+        out[j] = o;
+      }
+    }
+    *reinterpret_cast<uint4*>(p.col_codes + (b * C + cc) * (M / 2) + blockIdx.y * 16) = make_uint4(out[0], out[1], out[2], out[3]);
+  }
+}
+
+// Standalone transform: thread t owns one column, loads the 32 rows of a block in permuted order, runs the same
+// butterfly as the fused quantizer and writes each position back to the row it came from.
+template <typename T>
+__global__ __launch_bounds__(256) void hadamard_kernel(const T* __restrict__ x, int64_t ld_x, T* __restrict__ y, int64_t ld_y, int C,
+                                                       const QuantParams p) {
+  const int cc = blockIdx.x * 256 + threadIdx.x;
+  if (cc >= C) return;
+  const int64_t row0 = (int64_t)blockIdx.y * 32;
+  float z[32];
+#pragma unroll
+  for (int k = 0; k < 32; ++k) {
+    const T v = x[(row0 + p.perm_inv[k]) * ld_x + cc];
+    if constexpr (sizeof(T) == 2) z[k] = u2f((uint32_t)__builtin_bit_cast(unsigned short, v) << 16);
+    else z[k] = v;
+  }
+#pragma unroll
+  for (int h = 1; h < 32; h <<= 1) {
+#pragma unroll
+    for (int k = 0; k < 32; ++k) {
+      if ((k & h) == 0) {
+        float a0 = z[k], a1 = z[k + h];
+        z[k] = a0 + a1;
+        z[k + h] = a0 - a1;
+      }
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < 32; ++k) {
+    float q = div_sqrt32_signed(z[k], ((p.sign_mask >> k) & 1u) << 31);
+    T o;
+    if constexpr (sizeof(T) == 2) o = __builtin_bit_cast(T, (unsigned short)f32_to_bf16_bits(q));
+    else o = q;
+    y[(row0 + p.perm_inv[k]) * ld_y + cc] = o;
+  }
+}
+
+// Validates signs/perm (host arrays) and fills the kernel-side description.
+int fill_hadamard(QuantParams& p, const int8_t* signs, const uint8_t* perm, const char* who) {
+  p.sign_mask = 0;
+  uint32_t seen = 0;
+  ALTO_REQUIRE(signs != nullptr, "%s: hadamard set but signs is NULL", who);
+  for (int j = 0; j < 32; ++j) {
+    int k = perm ? perm[j] : j;
+    ALTO_REQUIRE(k >= 0 && k < 32 && !((seen >> k) & 1u), "%s: perm is not a permutation of 0..31", who);
+    seen |= 1u << k;
+    p.perm[j] = (uint8_t)k;
+    p.perm_inv[k] = (uint8_t)j;
+  }
+  for (int k = 0; k < 32; ++k) {
+    ALTO_REQUIRE(signs[k] == 1 || signs[k] == -1, "%s: signs[%d] = %d is not +1/-1", who, k, (int)signs[k]);
+    if (signs[k] < 0) p.sign_mask |= 1u << k;
+  }
+  return ALTO_MXFP4_OK;
+}
+
+template <typename T, bool DO_ROW, bool DO_COL, bool SR, bool RHT, bool B2D, bool GEN>
+void launch(const QuantParams& p, dim3 grid, hipStream_t st) {
+  hipLaunchKernelGGL((quant_kernel<T, DO_ROW, DO_COL, SR, RHT, B2D, GEN>), grid, dim3(256), 0, st, p);
+}
+
+template <typename T, bool SR, bool GEN>
+void dispatch_mode(const QuantParams& p, dim3 grid, hipStream_t st, bool do_row, bool do_col, bool rht, bool b2d) {
+  if (b2d) {
+    if (do_row && do_col) launch<T, true, true, SR, false, true, GEN>(p, grid, st);
+    else if (do_row) launch<T, true, false, SR, false, true, GEN>(p, grid, st);
+    else launch<T, false, true, SR, false, true, GEN>(p, grid, st);
+  } else if (do_row && do_col) {
+    if (rht) launch<T, true, true, SR, true, false, GEN>(p, grid, st);
+    else launch<T, true, true, SR, false, false, GEN>(p, grid, st);
+  } else if (do_row) {
+    launch<T, true, false, SR, false, false, GEN>(p, grid, st);
+  } else {
+    if (rht) launch<T, false, true, SR, true, false, GEN>(p, grid, st);
+    else launch<T, false, true, SR, false, false, GEN>(p, grid, st);
+  }
+}
+
+template <typename T>
+void dispatch(const QuantParams& p, dim3 grid, hipStream_t st, bool do_row, bool do_col, bool rht, bool b2d, bool sr, bool gen) {
+  if (gen) {
+    if (sr) dispatch_mode<T, true, true>(p, grid, st, do_row, do_col, rht, b2d);
+    else dispatch_mode<T, false, true>(p, grid, st, do_row, do_col, rht, b2d);
+  } else {
+    if (sr) dispatch_mode<T, true, false>(p, grid, st, do_row, do_col, rht, b2d);
+    else dispatch_mode<T, false, false>(p, grid, st, do_row, do_col, rht, b2d);
+  }
+}
+
+}  // namespace
+}  // namespace alto
+
+extern "C" int alto_mxfp4_quantize(const void* x, int dtype, int64_t batch, int64_t M, int64_t C, int64_t ld_x, int64_t bs_x,
+                                   uint8_t* row_codes, uint8_t* row_scales, uint8_t* col_codes, uint8_t* col_scales,
+                                   int is_2d, int rounding, const uint32_t* rand_bits, int64_t ld_rand, int64_t bs_rand,
+                                   int hadamard, const int8_t* signs, const uint8_t* perm,
+                                   int clip_mode, int use_uos, void* stream) {
+  using namespace alto;
+  const bool do_row = row_codes != nullptr, do_col = col_codes != nullptr;
+  ALTO_REQUIRE(x != nullptr, "quantize: x is NULL");
+  ALTO_REQUIRE(dtype == ALTO_DT_BF16 || dtype == ALTO_DT_F32, "quantize: dtype %d is neither bf16 (0) nor f32 (1)", dtype);
+  ALTO_REQUIRE(do_row || do_col, "quantize: neither a row nor a column output was requested");
+  ALTO_REQUIRE(!do_row || row_scales != nullptr, "quantize: row_codes given without row_scales");
+  ALTO_REQUIRE(!do_col || col_scales != nullptr, "quantize: col_codes given without col_scales");
+  ALTO_REQUIRE(batch >= 0 && M >= 0 && C >= 0, "quantize: negative size");
+  ALTO_REQUIRE(M < (1ll << 31) && C < (1ll << 31) && batch < 65536, "quantize: size out of range");
+  ALTO_REQUIRE(C % 8 == 0, "quantize: C (%lld) must be a multiple of 8", (long long)C);
+  ALTO_REQUIRE(!do_row || C % 32 == 0, "quantize: row output needs C (%lld) %% 32 == 0", (long long)C);
+  ALTO_REQUIRE(!(do_col || is_2d) || M % 32 == 0, "quantize: column output / 2D blocks need M (%lld) %% 32 == 0", (long long)M);
+  ALTO_REQUIRE(!is_2d || C % 32 == 0, "quantize: 2D blocks need C (%lld) %% 32 == 0", (long long)C);
+  const int64_t vec = dtype == ALTO_DT_BF16 ? 8 : 4;
+  ALTO_REQUIRE(ld_x >= C && ld_x % vec == 0 && bs_x % vec == 0, "quantize: ld_x/bs_x must be >= C and multiples of %lld elements", (long long)vec);
+  ALTO_REQUIRE((reinterpret_cast<uintptr_t>(x) & 15) == 0, "quantize: x must be 16-byte aligned");
+  ALTO_REQUIRE(rounding == ALTO_ROUND_RNE || rounding == ALTO_ROUND_SR, "quantize: bad rounding mode %d", rounding);
+  if (rounding == ALTO_ROUND_SR) {
+    ALTO_REQUIRE(rand_bits != nullptr, "quantize: stochastic rounding needs rand_bits");
+    ALTO_REQUIRE(ld_rand >= C && ld_rand % 4 == 0 && bs_rand % 4 == 0, "quantize: ld_rand/bs_rand must be >= C and multiples of 4");
+    ALTO_REQUIRE((reinterpret_cast<uintptr_t>(rand_bits) & 15) == 0, "quantize: rand_bits must be 16-byte aligned");
+  }
+  ALTO_REQUIRE(!hadamard || (!is_2d && do_col), "quantize: the Hadamard transform applies to a 1D column output only");
+  ALTO_REQUIRE(clip_mode == ALTO_CLIP_NONE || clip_mode == ALTO_CLIP_STATIC || clip_mode == ALTO_CLIP_DYNAMIC, "quantize: bad clip_mode %d", clip_mode);
+  if (clip_mode == ALTO_CLIP_DYNAMIC) {
+    set_error("quantize: clip_mode=dynamic is not implemented");
+    return ALTO_MXFP4_ENOTIMPL;
+  }
+  if (batch == 0 || M == 0 || C == 0) return ALTO_MXFP4_OK;
+
+  QuantParams p;
+  p.x = x; p.ld_x = ld_x; p.bs_x = bs_x; p.M = (int)M; p.C = (int)C;
+  p.rand = rand_bits; p.ld_r = ld_rand; p.bs_r = bs_rand;
+  p.row_codes = row_codes; p.row_scales = row_scales; p.col_codes = col_codes; p.col_scales = col_scales;
+  p.sign_mask = 0;
+  for (int k = 0; k < 32; ++k) { p.perm[k] = (uint8_t)k; p.perm_inv[k] = (uint8_t)k; }
+  if (hadamard) {
+    int rc = fill_hadamard(p, signs, perm, "quantize");
+    if (rc != ALTO_MXFP4_OK) return rc;
+  }
+  const bool both = do_row && do_col;
+  p.clip_row = (clip_mode == ALTO_CLIP_STATIC && !both) ? 1 : 0;
+  p.clip_col = (clip_mode == ALTO_CLIP_STATIC) ? 1 : 0;
+  if (!do_col) p.clip_col = 0;
+  if (!do_row) p.clip_row = 0;
+  p.uos = use_uos ? 1 : 0;
+  const bool gen = p.clip_row || p.clip_col || p.uos;
+
+  dim3 grid((unsigned)((C + TILE_C - 1) / TILE_C), (unsigned)((M + 31) / 32), (unsigned)batch);
+  ALTO_REQUIRE(grid.y <= 65535u, "quantize: M (%lld) exceeds 65535 row blocks", (long long)M);
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  if (dtype == ALTO_DT_BF16) dispatch<__bf16>(p, grid, st, do_row, do_col, hadamard != 0, is_2d != 0, rounding == ALTO_ROUND_SR, gen);
+  else dispatch<float>(p, grid, st, do_row, do_col, hadamard != 0, is_2d != 0, rounding == ALTO_ROUND_SR, gen);
+  return check_launch("quantize");
+}
+
+extern "C" int alto_mxfp4_hadamard(const void* x, int dtype, int64_t M, int64_t C, int64_t ld_x, void* y, int64_t ld_y,
+                                   const int8_t* signs, const uint8_t* perm, void* stream) {
+  using namespace alto;
+  ALTO_REQUIRE(x && y, "hadamard: NULL pointer");
+  ALTO_REQUIRE(dtype == ALTO_DT_BF16 || dtype == ALTO_DT_F32, "hadamard: bad dtype %d", dtype);
+  ALTO_REQUIRE(M >= 0 && C >= 0 && M % 32 == 0, "hadamard: M (%lld) must be a multiple of 32", (long long)M);
+  ALTO_REQUIRE(ld_x >= C && ld_y >= C, "hadamard: row stride smaller than C");
+  ALTO_REQUIRE(M / 32 <= 65535 && C < (1ll << 31), "hadamard: size out of range");
+  QuantParams p{};
+  int rc = fill_hadamard(p, signs, perm, "hadamard");
+  if (rc != ALTO_MXFP4_OK) return rc;
+  if (M == 0 || C == 0) return ALTO_MXFP4_OK;
+  dim3 grid((unsigned)((C + 255) / 256), (unsigned)(M / 32));
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  if (dtype == ALTO_DT_BF16)
+    hipLaunchKernelGGL(hadamard_kernel<__bf16>, grid, dim3(256), 0, st, (const __bf16*)x, ld_x, (__bf16*)y, ld_y, (int)C, p);
+  else
+    hipLaunchKernelGGL(hadamard_kernel<float>, grid, dim3(256), 0, st, (const float*)x, ld_x, (float*)y, ld_y, (int)C, p);
+  return check_launch("hadamard");
+}

@@ -1,0 +1,33 @@
+"""Entry points of the MXFP4 hot path, named as in ``alto/kernels/fp4/mxfp4/__init__.py:5-26``."""
+from .config import TrainingOpConfig
+from .grouped_gemm import (ALIGN_SIZE_M, MXFP4GroupedGEMM, _quantize_then_mxfp_scaled_grouped_mm,
+                           create_indices_from_offsets_nosync, mxfp4_grouped_gemm, mxfp4_grouped_gemm_backward_inputs,
+                           mxfp4_grouped_gemm_backward_weights, mxfp4_grouped_gemm_forward)
+from .hadamard import HadamardFactory, HadamardTransform
+from .linear import MXFP4LinearFunction, _to_mxfp4_then_scaled_mm, blockwise_mxfp4_gemm, transpose_codes
+from .quantization import BLOCK_SIZE_DEFAULT, convert_from_mxfp4, convert_to_mxfp4, hadamard_left, quantize_rowcol
+from ._runtime import set_rand_bits_source
+
+__all__ = (
+    "_quantize_then_mxfp_scaled_grouped_mm",
+    "_to_mxfp4_then_scaled_mm",
+    "ALIGN_SIZE_M",
+    "BLOCK_SIZE_DEFAULT",
+    "convert_from_mxfp4",
+    "convert_to_mxfp4",
+    "blockwise_mxfp4_gemm",
+    "MXFP4LinearFunction",
+    "mxfp4_grouped_gemm",
+    "MXFP4GroupedGEMM",
+    "mxfp4_grouped_gemm_forward",
+    "mxfp4_grouped_gemm_backward_inputs",
+    "mxfp4_grouped_gemm_backward_weights",
+    "create_indices_from_offsets_nosync",
+    "HadamardFactory",
+    "HadamardTransform",
+    "TrainingOpConfig",
+    "quantize_rowcol",
+    "hadamard_left",
+    "transpose_codes",
+    "set_rand_bits_source",
+)

@@ -1,0 +1,64 @@
+"""Small helpers shared by the host wrappers: device checks, pointers, stream, random bits."""
+from __future__ import annotations
+
+from typing import Callable, Optional
+
+import torch
+
+from .. import _lib
+
+DT_BF16, DT_F32 = 0, 1
+ROUND_RNE, ROUND_SR = 0, 1
+CLIP = {"none": 0, "static": 1, "dynamic": 2}
+
+
+def dtype_code(dt: torch.dtype) -> int:
+    if dt == torch.bfloat16:
+        return DT_BF16
+    if dt == torch.float32:
+        return DT_F32
+    raise AssertionError(f"unsupported dtype {dt}: only bfloat16 and float32")
+
+
+def require_gpu(*tensors: torch.Tensor) -> None:
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise RuntimeError(
+                "alto_amd.mxfp4 runs on MI355X only: got a tensor on device "
+                f"'{t.device}'. There is no CPU fallback for the HIP kernels.")
+
+
+def ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def stream_ptr(device: torch.device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def lib():
+    return _lib.load()
+
+
+# ---------------------------------------------------------------------------------------------- random bits
+# Stochastic rounding consumes 32 random bits per element.  By default they are drawn from torch's CUDA
+# generator; tests and reproducible runs install their own source.
+_rand_source: Optional[Callable[[torch.Size, torch.device], torch.Tensor]] = None
+
+
+def set_rand_bits_source(fn: Optional[Callable[[torch.Size, torch.device], torch.Tensor]]) -> None:
+    """Install ``fn(shape, device) -> int32 tensor`` as the source of stochastic-rounding bits (None restores the default)."""
+    global _rand_source
+    _rand_source = fn
+
+
+def draw_rand_bits(shape, device, seed: Optional[int] = None, offset: Optional[int] = None) -> torch.Tensor:
+    if _rand_source is not None:
+        r = _rand_source(torch.Size(shape), device)
+        assert r.shape == torch.Size(shape) and r.dtype in (torch.int32, torch.uint32)
+        return r
+    gen = None
+    if seed is not None:
+        gen = torch.Generator(device=device)
+        gen.manual_seed(int(seed) * 0x9E3779B1 + (int(offset) if offset is not None else 0) & 0x7FFFFFFFFFFFFFFF)
+    return torch.randint(-2 ** 31, 2 ** 31, tuple(shape), dtype=torch.int32, device=device, generator=gen)

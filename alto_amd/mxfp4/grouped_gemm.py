@@ -1,0 +1,248 @@
+"""Contiguous grouped (MoE) MXFP4 GEMM on the HIP kernels.
+
+Mirrors ``alto/kernels/fp4/mxfp4/mxfp_grouped_gemm``: ``mxfp4_grouped_gemm_forward`` (cg_forward.py:200-303),
+``mxfp4_grouped_gemm_backward_inputs`` / ``_weights`` (cg_backward.py:398-593), ``MXFP4GroupedGEMM`` (:599-930),
+``mxfp4_grouped_gemm`` (:933-991) and ``_quantize_then_mxfp_scaled_grouped_mm`` (functional.py:11-38).
+
+The kernels consume expert row ranges (``offs``: E+1 int32 offsets on the device) instead of a per-row expert
+index; the index form of the reference API is converted on the device without a host sync.  Groups may be ragged
+for 1D activation scales; the reference's 128-row alignment is still required by the weight-gradient kernel at a
+granularity of 32 rows (one MX block along the token dim may not straddle two experts).
+"""
+from __future__ import annotations
+
+from typing import NamedTuple, Optional
+
+import torch
+
+from . import _runtime as rt
+from .._lib import check
+from .hadamard import HadamardFactory, HadamardTransform
+from .linear import transpose_codes, unwrap_weight_wrapper
+from .quantization import convert_to_mxfp4, quantize_rowcol
+
+ALIGN_SIZE_M = 128
+
+
+def create_indices_from_offsets_nosync(m_offsets: torch.Tensor) -> torch.Tensor:
+    """Cumulative group ends -> per-row expert index, no host sync beyond the size read the reference also does
+    (alto/kernels/dsgemm_utils.py:96-112)."""
+    total_size = m_offsets[-1]
+    all_indices = torch.arange(total_size, device=m_offsets.device, dtype=torch.int32)
+    return torch.bucketize(all_indices, m_offsets, right=True, out_int32=True)
+
+
+class Groups(NamedTuple):
+    """Row groups of a grouped GEMM: group g = rows [offs[g], offs[g+1]) served by expert ``expert[g]`` (or g)."""
+    offs: torch.Tensor                # int32 [n + 1] on the device
+    expert: Optional[torch.Tensor]    # int32 [n] on the device, None: expert id == group index
+    n: int
+
+
+def groups_from_indices(expert_indices: torch.Tensor) -> Groups:
+    """Per-row expert ids with one expert per aligned 128-row group (the reference's contract, cg_forward.py:135-136)."""
+    M_total = expert_indices.shape[0]
+    n = M_total // ALIGN_SIZE_M
+    offs = torch.arange(n + 1, device=expert_indices.device, dtype=torch.int32) * ALIGN_SIZE_M
+    return Groups(offs, expert_indices[::ALIGN_SIZE_M].to(torch.int32).contiguous(), n)
+
+
+def groups_from_offsets(offsets: torch.Tensor) -> Groups:
+    """int32 [E+1] offsets with a leading 0: rows sorted by expert, group g == expert g, ragged sizes allowed."""
+    assert offsets.dtype == torch.int32 and offsets.dim() == 1
+    return Groups(offsets.contiguous(), None, offsets.shape[0] - 1)
+
+
+def offsets_from_ends(offs: torch.Tensor) -> torch.Tensor:
+    """Cumulative group ends [E] (torch._grouped_mm convention) -> offsets [E+1] with a leading 0."""
+    return torch.cat([torch.zeros(1, dtype=torch.int32, device=offs.device), offs.to(torch.int32)])
+
+
+def _scale_strides(s: torch.Tensor):
+    return s.stride(0), s.stride(1), s.stride(2)
+
+
+def grouped_forward(a_q, a_s, w_q, w_s, groups: Groups, use_2dblock_x, use_2dblock_w, output_dtype):
+    """out[r] = A[r] . W[e(r)]^T with w_q [E, N, K/2] (unit stride along K) and w_s [E, N or N/32, K/32]."""
+    E, N = w_q.shape[0], w_q.shape[1]
+    K = a_q.shape[1] * 2
+    assert w_q.shape[2] * 2 == K, f"Input K ({K}) must match weight K ({w_q.shape[2] * 2})"
+    if a_q.stride(1) != 1 or a_q.stride(0) % 16:
+        a_q = a_q.contiguous()
+    if w_q.stride(2) != 1 or w_q.stride(1) % 16 or w_q.stride(0) % 16:
+        w_q = w_q.contiguous()
+    out = torch.empty((a_q.shape[0], N), dtype=output_dtype, device=a_q.device)
+    if out.numel() == 0:
+        return out
+    rc = rt.lib().alto_mxfp4_grouped_gemm(
+        a_q.data_ptr(), a_q.stride(0), a_s.data_ptr(), a_s.stride(0), a_s.stride(1), int(use_2dblock_x),
+        w_q.data_ptr(), w_q.stride(0), w_q.stride(1), w_s.data_ptr(), w_s.stride(0), w_s.stride(1), w_s.stride(2), int(use_2dblock_w),
+        groups.offs.data_ptr(), rt.ptr(groups.expert), groups.n, E, a_q.shape[0], N, K, out.data_ptr(), rt.dtype_code(output_dtype), out.stride(0),
+        rt.stream_ptr(a_q.device))
+    check(rc, "alto_mxfp4_grouped_gemm")
+    return out
+
+
+def mxfp4_grouped_gemm_forward(inputs, expert_weights, expert_indices, input_scales, weight_scales, trans_weights=True,
+                               use_2dblock_x=False, use_2dblock_w=True, output_dtype=torch.bfloat16):
+    """cg_forward.py:200-303.  inputs [M_buf, K/2]; expert_weights [E, N, K/2] if trans_weights else [E, K/2, N]."""
+    assert expert_indices.is_contiguous(), "Expert indices tensor must be contiguous"
+    M_total = expert_indices.shape[0]
+    torch._check(M_total > 0)
+    torch._check(M_total % ALIGN_SIZE_M == 0)
+    rt.require_gpu(inputs, expert_weights, expert_indices, input_scales, weight_scales)
+    E = expert_weights.shape[0]
+    w_q = expert_weights if trans_weights else expert_weights.transpose(1, 2)
+    w_s = weight_scales if trans_weights else weight_scales.transpose(1, 2)
+    return grouped_forward(inputs, input_scales, w_q, w_s, groups_from_indices(expert_indices), use_2dblock_x, use_2dblock_w, output_dtype)
+
+
+def mxfp4_grouped_gemm_backward_inputs(grad_output, expert_weights, expert_indices, go_scales, expert_weight_scales,
+                                       trans_weights=True, use_2dblock_x=False, use_2dblock_w=True, k_pack_w=True,
+                                       output_dtype=torch.bfloat16):
+    """dX[r] = dY[r] . W[e(r)] (cg_backward.py:500-593).  Reduction over N; W packed along N iff ``k_pack_w``."""
+    assert expert_indices.is_contiguous(), "Expert indices tensor must be contiguous"
+    M_total = expert_indices.shape[0]
+    torch._check(M_total > 0)
+    torch._check(M_total % ALIGN_SIZE_M == 0)
+    rt.require_gpu(grad_output, expert_weights, expert_indices, go_scales, expert_weight_scales)
+    E = expert_weights.shape[0]
+    # bring the weights to [E, K_out, N/2] packed along N
+    wv = expert_weights if trans_weights else expert_weights.transpose(1, 2)          # [E, N', K'] one dim halved
+    sv = expert_weight_scales if trans_weights else expert_weight_scales.transpose(1, 2)
+    if k_pack_w:
+        w_can = wv.transpose(1, 2)                                                    # [E, K, N/2] view
+    else:
+        w_can = torch.stack([transpose_codes(wv[e]) for e in range(E)])               # [E, N, K/2] -> [E, K, N/2]
+    s_can = sv.transpose(1, 2)                                                        # [E, K(/32), N/32]
+    return grouped_forward(grad_output, go_scales, w_can, s_can, groups_from_indices(expert_indices), use_2dblock_x, use_2dblock_w, output_dtype)
+
+
+def grouped_dw(go_qm, go_sm, x_qm, x_sm, groups: Groups, num_experts, output_dtype, trans_weights=True, out_scale=1.0):
+    """dW[e] = sum_{rows of e} dY^T X with token-packed operands: go_qm [N, M/2], x_qm [K, M/2] (unit stride along tokens)."""
+    N, K = go_qm.shape[0], x_qm.shape[0]
+    M_total = go_qm.shape[1] * 2
+    assert x_qm.shape[1] * 2 == M_total
+    if go_qm.stride(1) != 1 or go_qm.stride(0) % 16:
+        go_qm = go_qm.contiguous()
+    if x_qm.stride(1) != 1 or x_qm.stride(0) % 16:
+        x_qm = x_qm.contiguous()
+    shape = (num_experts, N, K) if trans_weights else (num_experts, K, N)
+    dw = torch.empty(shape, dtype=output_dtype, device=go_qm.device)
+    s_e, s_n, s_k = (dw.stride(0), dw.stride(1), dw.stride(2)) if trans_weights else (dw.stride(0), dw.stride(2), dw.stride(1))
+    rc = rt.lib().alto_mxfp4_grouped_gemm_dw(
+        go_qm.data_ptr(), go_qm.stride(0), go_sm.data_ptr(), go_sm.stride(0), go_sm.stride(1),
+        x_qm.data_ptr(), x_qm.stride(0), x_sm.data_ptr(), x_sm.stride(0), x_sm.stride(1),
+        groups.offs.data_ptr(), rt.ptr(groups.expert), groups.n, num_experts, M_total, N, K, dw.data_ptr(), rt.dtype_code(output_dtype), s_e, s_n, s_k,
+        float(out_scale), rt.stream_ptr(go_qm.device))
+    check(rc, "alto_mxfp4_grouped_gemm_dw")
+    return dw
+
+
+def mxfp4_grouped_gemm_backward_weights(grad_output, inputs, expert_indices, num_experts, go_scales, input_scales,
+                                        trans_weights=True, use_2dblock_go=False, use_2dblock_x=True, k_pack_go=True,
+                                        k_pack_x=True, output_dtype=torch.bfloat16):
+    """cg_backward.py:398-497.  With ``k_pack_*`` the operands are [M/2, N] / [M/2, K] views packed along tokens."""
+    assert expert_indices.is_contiguous(), "Expert indices tensor must be contiguous"
+    M_total = expert_indices.shape[0]
+    torch._check(M_total > 0)
+    torch._check(M_total % ALIGN_SIZE_M == 0)
+    if use_2dblock_go or use_2dblock_x or not (k_pack_go and k_pack_x):
+        raise NotImplementedError("grouped weight gradient: only token-packed 1D-scaled operands are implemented")
+    rt.require_gpu(grad_output, inputs, expert_indices, go_scales, input_scales)
+    return grouped_dw(grad_output.transpose(0, 1), go_scales.transpose(0, 1), inputs.transpose(0, 1), input_scales.transpose(0, 1),
+                      groups_from_indices(expert_indices), num_experts, output_dtype, trans_weights)
+
+
+class MXFP4GroupedGEMM(torch.autograd.Function):
+    """Grouped GEMM with full backward (cg_backward.py:599-930), recipe branch 1D activations / 2D weights."""
+
+    @staticmethod
+    def forward(ctx, inputs, expert_weights, expert_indices, trans_weights=True, use_2dblock_x=False, use_2dblock_w=True,
+                use_sr_grad=False, use_dge=False, clip_mode="none", use_macro_block_scaling=False,
+                hadamard_transform: Optional[HadamardTransform] = None, use_uos: bool = False, offsets: Optional[torch.Tensor] = None):
+        if use_dge:
+            raise NotImplementedError("use_dge is not part of the MXFP4 hot path this build covers")
+        assert not use_macro_block_scaling, "Macro block scaling is not supported in real MXFP4 kernels"
+        if use_2dblock_x or not use_2dblock_w:
+            raise NotImplementedError("grouped MXFP4 GEMM: only use_2dblock_x=False, use_2dblock_w=True is implemented")
+        original_dtype = inputs.dtype
+        expert_weights = unwrap_weight_wrapper(expert_weights)
+        E = expert_weights.shape[0]
+        M_buf = inputs.shape[0]
+        if offsets is None:
+            M_total = expert_indices.shape[0]
+            torch._check(M_total > 0)
+            torch._check(M_total % ALIGN_SIZE_M == 0)
+            groups = groups_from_indices(expert_indices)
+        else:
+            groups = groups_from_offsets(offsets)
+        torch._check(M_buf % 32 == 0)
+        x = inputs if inputs.is_contiguous() else inputs.contiguous()
+        a_q, a_s, a_qm, a_sm = quantize_rowcol(x, False, hadamard=hadamard_transform, clip_mode=clip_mode, use_uos=use_uos)
+        # weights: one pass gives the K-packed codes (forward) and the N-packed codes (dX)
+        w = expert_weights if trans_weights else expert_weights.transpose(1, 2)   # logical [E, N, K]
+        if w.stride(2) == 1:
+            wq_nk, ws_nk, wq_kn = _quantize_experts(w, use_uos)                   # [E,N,K/2], [E,N/32,K/32], [E,K,N/2]
+        else:                                                                     # stored [E, K, N]: same pass, roles swapped
+            wq_kn, ws_kn, wq_nk = _quantize_experts(w.transpose(1, 2), use_uos)
+            ws_nk = ws_kn.transpose(1, 2)
+        out = grouped_forward(a_q, a_s, wq_nk, ws_nk, groups, False, True, original_dtype)
+        ctx.save_for_backward(a_qm, a_sm, wq_kn, ws_nk, groups.offs, groups.expert)
+        ctx.num_groups = groups.n
+        ctx.trans_weights = trans_weights
+        ctx.original_dtype = original_dtype
+        ctx.use_sr_grad = use_sr_grad
+        ctx.hadamard_transform = hadamard_transform
+        ctx.clip_mode = clip_mode
+        ctx.use_uos = use_uos
+        ctx.num_experts = E
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        a_qm, a_sm, wq_kn, ws_nk, g_offs, g_expert = ctx.saved_tensors
+        groups = Groups(g_offs, g_expert, ctx.num_groups)
+        go = grad_output if grad_output.is_contiguous() else grad_output.contiguous()
+        sr = bool(ctx.use_sr_grad)
+        rand = rt.draw_rand_bits(go.shape, go.device) if sr else None
+        go_q, go_s, go_qm, go_sm = quantize_rowcol(go, False, use_sr=sr, rand_bits=rand, hadamard=ctx.hadamard_transform,
+                                                   clip_mode=ctx.clip_mode, use_uos=ctx.use_uos)
+        grad_inputs = grouped_forward(go_q, go_s, wq_kn, ws_nk.transpose(1, 2), groups, False, True, ctx.original_dtype)
+        grad_weights = grouped_dw(go_qm.transpose(0, 1), go_sm.transpose(0, 1), a_qm.transpose(0, 1), a_sm.transpose(0, 1),
+                                  groups, ctx.num_experts, ctx.original_dtype, ctx.trans_weights,
+                                  16.0 / 9.0 if ctx.clip_mode == "static" else 1.0)
+        return (grad_inputs, grad_weights) + (None,) * 11
+
+
+def _quantize_experts(w: torch.Tensor, use_uos: bool):
+    """w [E, R, C] (unit stride along C) -> (codes packed along C [E,R,C/2], 2D scales [E,R/32,C/32], codes packed along R [E,C,R/2])."""
+    from .quantization import _prep, _quantize_call
+    E, R, C = w.shape
+    w3 = _prep(w)
+    rc, rs, cc, _ = _quantize_call(w3, True, True, True, False, None, None, 0, use_uos)
+    return rc, rs, cc
+
+
+def mxfp4_grouped_gemm(inputs, expert_weights, expert_indices, *, trans_weights=True, use_2dblock_x=False, use_2dblock_w=True,
+                       use_sr_grad=False, use_dge=False, use_hadamard=False, clip_mode="none", use_macro_block_scaling=False,
+                       use_uos=False, offsets: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Grouped GEMM with full backward support (cg_backward.py:933-991).
+
+    ``offsets`` (int32 [E+1], leading 0) may be given instead of ``expert_indices`` to describe ragged groups.
+    """
+    if use_hadamard:
+        assert not use_2dblock_x, "Hadamard transform can only be applied if 2D block is not used for activations."
+    if expert_indices is not None and expert_indices.dtype != torch.int32:
+        expert_indices = expert_indices.to(torch.int32)
+    hadamard_transform = HadamardFactory.create_transform(device=expert_weights.device) if use_hadamard else None
+    return MXFP4GroupedGEMM.apply(inputs, expert_weights, expert_indices, trans_weights, use_2dblock_x, use_2dblock_w, use_sr_grad,
+                                  use_dge, clip_mode, use_macro_block_scaling, hadamard_transform, use_uos, offsets)
+
+
+def _quantize_then_mxfp_scaled_grouped_mm(A, B, offs, use_2dblock_x, use_2dblock_w, use_sr_grad, use_dge, use_hadamard, clip_mode,
+                                          use_macro_block_scaling, use_uos=False) -> torch.Tensor:
+    """``torch._grouped_mm(A, B, offs=offs)`` replacement (functional.py:11-38): B is [E, K, N], offs are group ends."""
+    return mxfp4_grouped_gemm(A, B, None, trans_weights=False, use_2dblock_x=use_2dblock_x, use_2dblock_w=use_2dblock_w,
+                              use_sr_grad=use_sr_grad, use_dge=use_dge, use_hadamard=use_hadamard, clip_mode=clip_mode,
+                              use_macro_block_scaling=use_macro_block_scaling, use_uos=use_uos, offsets=offsets_from_ends(offs))

@@ -1,0 +1,210 @@
+"""Block-scaled MXFP4 GEMM and the linear autograd function on the HIP kernels.
+
+Mirrors ``alto/kernels/fp4/mxfp4/mxfp_linear.py``: ``blockwise_mxfp4_gemm`` (:142-255), ``MXFP4LinearFunction``
+(:258-570) and ``_to_mxfp4_then_scaled_mm`` (:573-602), same argument order and meaning.
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from . import _runtime as rt
+from .._lib import check
+from .hadamard import HadamardFactory, HadamardTransform
+from .quantization import BLOCK_SIZE_DEFAULT, convert_to_mxfp4, quantize_rowcol
+
+
+def unwrap_weight_wrapper(weight: torch.Tensor) -> torch.Tensor:
+    """Plain local tensor behind a training-time weight wrapper (alto/kernels/fp4/fp4_common/tensor_wrappers.py:8-30)."""
+    if type(weight) is torch.Tensor:
+        return weight
+    if hasattr(weight, "_data"):
+        return weight._data
+    return weight.as_subclass(torch.Tensor)
+
+
+def transpose_codes(codes: torch.Tensor) -> torch.Tensor:
+    """[R, C/2] bytes packed along C -> [C, R/2] bytes packed along R (same 4-bit codes)."""
+    assert codes.dim() == 2 and codes.dtype == torch.uint8
+    rt.require_gpu(codes)
+    c = codes.contiguous()
+    R, C = c.shape[0], c.shape[1] * 2
+    assert R % 2 == 0
+    out = torch.empty((C, R // 2), dtype=torch.uint8, device=codes.device)
+    check(rt.lib().alto_mxfp4_transpose_codes(c.data_ptr(), R, C, out.data_ptr(), rt.stream_ptr(codes.device)), "alto_mxfp4_transpose_codes")
+    return out
+
+
+def _canonical_operand(t: torch.Tensor, s: torch.Tensor, rows_first: bool, k_pack: bool):
+    """Bring one GEMM operand to the form the kernel consumes: codes [rows, K/2] with unit stride along K.
+
+    ``t`` is the 2D code tensor in the orientation the caller holds (rows x K if ``rows_first`` else K x rows, the
+    packed dim halved); ``s`` the scales in the same orientation.  Returns (codes, scales_view[rows(/32), K/32]).
+    """
+    tv = t if rows_first else t.transpose(0, 1)   # [rows', K'] with one of the dims halved
+    sv = s if rows_first else s.transpose(0, 1)   # [rows or rows/32, K/32]
+    if k_pack:
+        if tv.stride(1) != 1 or tv.stride(0) % 16 != 0 or tv.data_ptr() % 16 != 0:
+            tv = tv.contiguous()
+        return tv, sv
+    # packed along the row dim: memory must be [K][rows/2]; nibble-transpose into [rows][K/2]
+    return transpose_codes(tv.transpose(0, 1)), sv
+
+
+def blockwise_mxfp4_gemm(
+    a: torch.Tensor,
+    a_s: torch.Tensor,
+    b: torch.Tensor,
+    b_s: torch.Tensor,
+    use_2dblock_a: bool = False,
+    use_2dblock_b: bool = False,
+    k_pack_a: bool = True,
+    k_pack_b: bool = True,
+    trans_a: bool = False,
+    trans_b: bool = False,
+    block_size: int = BLOCK_SIZE_DEFAULT,
+    output_dtype: torch.dtype = torch.float32,
+    out_scale: float = 1.0,
+) -> torch.Tensor:
+    """C = op(A) @ op(B) on FP4 codes with E8M0 scales per 32 along K, fp32 accumulation (mxfp_linear.py:142-255).
+
+    M, N, K refer to unpacked FP4 element counts.  ``a`` is ``[M, K]`` (``[K, M]`` if ``trans_a``), ``b`` is
+    ``[K, N]`` (``[N, K]`` if ``trans_b``), each with its packed dim halved: packed along K when ``k_pack_*``.
+    """
+    assert a.dim() == 2 and b.dim() == 2
+    assert block_size == BLOCK_SIZE_DEFAULT
+    rt.require_gpu(a, a_s, b, b_s)
+    if trans_a:
+        K, M = a.shape
+    else:
+        M, K = a.shape
+    if k_pack_a:
+        K *= 2
+    else:
+        M *= 2
+    a_rows_s = M // block_size if use_2dblock_a else M
+    exp_as = (K // block_size, a_rows_s) if trans_a else (a_rows_s, K // block_size)
+    assert a_s.shape == torch.Size(exp_as), f"A scale has shape {a_s.shape}, but {exp_as} is expected."
+    if trans_b:
+        N, KB = b.shape
+    else:
+        KB, N = b.shape
+    if k_pack_b:
+        KB *= 2
+    else:
+        N *= 2
+    assert KB == K, f"Input B has unpacked reduction shape ({KB}) but {(K)} is expected."
+    b_rows_s = N // block_size if use_2dblock_b else N
+    exp_bs = (b_rows_s, K // block_size) if trans_b else (K // block_size, b_rows_s)
+    assert b_s.shape == torch.Size(exp_bs)
+    assert output_dtype in (torch.float32, torch.bfloat16)
+
+    ac, asv = _canonical_operand(a, a_s, rows_first=not trans_a, k_pack=k_pack_a)
+    bc, bsv = _canonical_operand(b, b_s, rows_first=trans_b, k_pack=k_pack_b)
+    c = torch.empty((M, N), dtype=output_dtype, device=a.device)
+    if M == 0 or N == 0:
+        return c
+    if K == 0:
+        return c.zero_()
+    rc = rt.lib().alto_mxfp4_gemm(
+        ac.data_ptr(), ac.stride(0), asv.data_ptr(), asv.stride(0), asv.stride(1), int(use_2dblock_a),
+        bc.data_ptr(), bc.stride(0), bsv.data_ptr(), bsv.stride(0), bsv.stride(1), int(use_2dblock_b),
+        M, N, K, c.data_ptr(), rt.dtype_code(output_dtype), c.stride(0), float(out_scale), rt.stream_ptr(a.device))
+    check(rc, "alto_mxfp4_gemm")
+    return c
+
+
+class MXFP4LinearFunction(torch.autograd.Function):
+    """``y = x @ W^T`` with MXFP4 operands in forward and in both backward GEMMs (mxfp_linear.py:258-570).
+
+    Recipe branch ``use_2dblock_x=False, use_2dblock_w=True`` runs on three fused launches per direction:
+    forward = one pass over x (row codes for fprop + Hadamard/column codes saved for wgrad), one pass over W
+    (both packings of its 2D-block codes), one GEMM; backward = one pass over dY (row + Hadamard/column codes,
+    stochastic rounding) and two GEMMs.  Other flag combinations follow the reference's call sequence with the
+    same kernels.
+    """
+
+    @staticmethod
+    def forward(ctx, x, weight, use_2dblock_x, use_2dblock_w, use_sr_grad, use_dge, clip_mode,
+                use_macro_block_scaling, hadamard_transform: Optional[HadamardTransform] = None, use_uos: bool = False):
+        if use_dge:
+            raise NotImplementedError("use_dge is not part of the MXFP4 hot path this build covers")
+        assert not use_macro_block_scaling, "Macro block scaling is not supported in real MXFP4 kernels"
+        weight = unwrap_weight_wrapper(weight)
+        original_shape = x.shape
+        original_dtype = x.dtype
+        x2 = x.reshape(-1, original_shape[-1])
+        M = x2.shape[0]
+
+        fuse_x = (not use_2dblock_x) and M % 32 == 0
+        if fuse_x:
+            x_q, x_s, x_qm, x_sm = quantize_rowcol(x2, False, hadamard=hadamard_transform, clip_mode=clip_mode, use_uos=use_uos)
+        else:
+            x_q, x_s = convert_to_mxfp4(x2, axis=-1, is_2d_block=use_2dblock_x, use_uos=use_uos)
+            if use_2dblock_x:
+                x_qm, x_sm = x_q, x_s
+            else:  # token count not a multiple of 32: the reference fails in its axis=0 quantisation as well
+                x_qm, x_sm = convert_to_mxfp4(x2, axis=0, clip_mode=clip_mode, use_uos=use_uos, hadamard=hadamard_transform)
+
+        if use_2dblock_w:
+            w_q, w_s, w_qt, _ = quantize_rowcol(weight, True, use_uos=use_uos)
+            w_bwd, w_bwd_s = w_qt, w_s            # [N/2, K] view over [K][N/2] memory, scales [N/32, K/32]
+        else:
+            w_q, w_s = convert_to_mxfp4(weight, axis=-1, is_2d_block=False, use_uos=use_uos)
+            w_bwd, w_bwd_s = convert_to_mxfp4(weight, axis=0, is_2d_block=False, use_uos=use_uos)
+
+        y = blockwise_mxfp4_gemm(x_q, x_s, w_q, w_s, use_2dblock_a=use_2dblock_x, use_2dblock_b=use_2dblock_w,
+                                 trans_b=True, output_dtype=original_dtype)
+        ctx.save_for_backward(x_qm, x_sm, w_bwd, w_bwd_s)
+        ctx.use_2dblock_x = use_2dblock_x
+        ctx.use_2dblock_w = use_2dblock_w
+        ctx.original_dtype = original_dtype
+        ctx.use_sr_grad = use_sr_grad
+        ctx.hadamard_transform = hadamard_transform
+        ctx.clip_mode = clip_mode
+        ctx.use_uos = use_uos
+        return y.view(*original_shape[:-1], -1)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        original_shape = grad_output.shape
+        go = grad_output.reshape(-1, original_shape[-1])
+        x_qm, x_sm, w_bwd, w_bwd_s = ctx.saved_tensors
+        sr = bool(ctx.use_sr_grad)
+        rand = rt.draw_rand_bits(go.shape, go.device) if sr else None
+        if ctx.use_2dblock_x:
+            go_q, go_s = convert_to_mxfp4(go, axis=-1, is_2d_block=True, use_sr=sr, rand_bits=rand, use_uos=ctx.use_uos)
+            go_qm, go_sm = go_q, go_s
+        else:
+            go_q, go_s, go_qm, go_sm = quantize_rowcol(go, False, use_sr=sr, rand_bits=rand, hadamard=ctx.hadamard_transform,
+                                                       clip_mode=ctx.clip_mode, use_uos=ctx.use_uos)
+        # dgrad: reduction over N.  The saved weight operand is already packed along N (both layouts of a 2D-block
+        # quantisation hold the same codes), so no k_pack=False repack is needed here.
+        grad_inputs = blockwise_mxfp4_gemm(go_q, go_s, w_bwd, w_bwd_s, use_2dblock_a=ctx.use_2dblock_x,
+                                           use_2dblock_b=ctx.use_2dblock_w, k_pack_b=True, output_dtype=ctx.original_dtype)
+        # wgrad: reduction over tokens
+        grad_weights = blockwise_mxfp4_gemm(go_qm, go_sm, x_qm, x_sm, use_2dblock_a=ctx.use_2dblock_x,
+                                            use_2dblock_b=ctx.use_2dblock_x, trans_a=True,
+                                            k_pack_a=not ctx.use_2dblock_x, k_pack_b=not ctx.use_2dblock_x,
+                                            output_dtype=ctx.original_dtype,
+                                            out_scale=16.0 / 9.0 if ctx.clip_mode == "static" else 1.0)
+        return grad_inputs.view(*original_shape[:-1], -1), grad_weights, None, None, None, None, None, None, None, None
+
+
+def _to_mxfp4_then_scaled_mm(
+    a: torch.Tensor,
+    b: torch.Tensor,
+    use_2dblock_x: bool,
+    use_2dblock_w: bool,
+    use_sr_grad: int,
+    use_dge: bool,
+    clip_mode: str,
+    use_hadamard: bool,
+    use_macro_block_scaling: bool = False,
+    use_uos: bool = False,
+) -> torch.Tensor:
+    """``a @ b.T`` through ``MXFP4LinearFunction`` with a fresh random Hadamard per call (mxfp_linear.py:573-602)."""
+    hadamard_transform = HadamardFactory.create_transform(device=b.device) if use_hadamard else None
+    return MXFP4LinearFunction.apply(a, b, use_2dblock_x, use_2dblock_w, use_sr_grad, use_dge, clip_mode,
+                                     use_macro_block_scaling, hadamard_transform, use_uos)

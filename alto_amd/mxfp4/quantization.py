@@ -1,0 +1,264 @@
+"""MXFP4 quantize / dequantize entry points backed by the HIP kernels.
+
+Same names, argument meaning and error behaviour as the reference's
+``alto/kernels/fp4/mxfp4/mxfp_quantization.py:410-545`` (``convert_to_mxfp4`` / ``convert_from_mxfp4``), plus two
+explicit inputs the reference draws from hidden state: ``rand_bits`` (the 32 random bits per element that
+stochastic rounding consumes) and ``hadamard`` (a ``HadamardTransform`` fused in front of an ``axis=-2``
+quantisation).  ``quantize_rowcol`` exposes the fused row + column quantizer the linear layer uses.
+"""
+from __future__ import annotations
+
+import math
+from typing import Optional, Tuple
+
+import torch
+
+from . import _runtime as rt
+from .._lib import check
+from .hadamard import HadamardTransform
+
+BLOCK_SIZE_DEFAULT = 32
+
+
+def _clip_code(clip_mode: str) -> int:
+    if clip_mode not in rt.CLIP:
+        raise ValueError(f"Invalid clip mode: {clip_mode}")
+    return rt.CLIP[clip_mode]
+
+
+def _as_i32(r: torch.Tensor) -> torch.Tensor:
+    if r.dtype == torch.uint32:
+        return r.view(torch.int32)
+    assert r.dtype == torch.int32, f"rand_bits must be int32/uint32, got {r.dtype}"
+    return r
+
+
+def _signs_perm_ptrs(h: Optional[HadamardTransform]):
+    if h is None:
+        return 0, None, None
+    return 1, h.signs.data_ptr(), (None if h.perm is None else h.perm.data_ptr())
+
+
+def _quantize_call(x3: torch.Tensor, want_row: bool, want_col: bool, is_2d: bool, use_sr: bool,
+                   rand3: Optional[torch.Tensor], hadamard: Optional[HadamardTransform], clip: int, use_uos: bool):
+    """x3: [B, M, C] with unit stride along C and uniform row / batch strides. Returns dense outputs (or None)."""
+    B, M, C = x3.shape
+    dev = x3.device
+    row_codes = row_scales = col_codes = col_scales = None
+    if want_row:
+        row_codes = torch.empty((B, M, C // 2), dtype=torch.uint8, device=dev)
+        row_scales = torch.empty((B, M // 32, C // 32) if is_2d else (B, M, C // 32), dtype=torch.uint8, device=dev)
+    if want_col:
+        col_codes = torch.empty((B, C, M // 2), dtype=torch.uint8, device=dev)
+        col_scales = torch.empty((B, C // 32, M // 32) if is_2d else (B, C, M // 32), dtype=torch.uint8, device=dev)
+    had, sp, pp = _signs_perm_ptrs(hadamard)
+    ld_x = x3.stride(1) if M > 1 else C
+    bs_x = x3.stride(0) if B > 1 else M * ld_x
+    ld_r = bs_r = 0
+    if use_sr:
+        ld_r = rand3.stride(1) if M > 1 else C
+        bs_r = rand3.stride(0) if B > 1 else M * ld_r
+    rc = rt.lib().alto_mxfp4_quantize(
+        x3.data_ptr(), rt.dtype_code(x3.dtype), B, M, C, ld_x, bs_x,
+        rt.ptr(row_codes), rt.ptr(row_scales), rt.ptr(col_codes), rt.ptr(col_scales),
+        int(is_2d), rt.ROUND_SR if use_sr else rt.ROUND_RNE, rt.ptr(rand3), ld_r, bs_r,
+        had, sp, pp, clip, int(use_uos), rt.stream_ptr(dev))
+    check(rc, "alto_mxfp4_quantize")
+    return row_codes, row_scales, col_codes, col_scales
+
+
+def _batched_view(t: torch.Tensor) -> Optional[torch.Tensor]:
+    """[..., M, C] -> [B, M, C] view with unit stride along C and uniform strides, or None if a copy is needed."""
+    if t.dim() < 2 or (t.shape[-1] != 1 and t.stride(-1) != 1):
+        return None
+    if t.dim() == 2:
+        return t.unsqueeze(0)
+    for d in range(t.dim() - 3):  # leading dims must collapse into a single batch stride
+        if t.shape[d] != 1 and t.stride(d) != t.stride(d + 1) * t.shape[d + 1]:
+            return None
+    batch = int(math.prod(t.shape[:-2]))
+    return t.as_strided((batch, t.shape[-2], t.shape[-1]), (t.stride(-3), t.stride(-2), 1))
+
+
+def _aligned(t: torch.Tensor) -> bool:
+    vec = 8 if t.dtype == torch.bfloat16 else 4
+    return t.data_ptr() % 16 == 0 and all(s % vec == 0 for s in t.stride()[:-1])
+
+
+def _prep(t: torch.Tensor) -> torch.Tensor:
+    """Return a [B, M, C] view the kernel accepts (copying only when the strides force it)."""
+    v = _batched_view(t)
+    if v is None or not _aligned(v):
+        v = _batched_view(t.contiguous())
+    return v
+
+
+def convert_to_mxfp4(
+    data_hp: torch.Tensor,
+    block_size: int = BLOCK_SIZE_DEFAULT,
+    axis: int = -1,
+    is_2d_block: bool = False,
+    use_sr: bool = False,
+    use_asm: Optional[bool] = None,
+    philox_seed: Optional[int] = None,
+    philox_offset: Optional[int] = None,
+    clip_mode: str = "none",
+    use_uos: bool = False,
+    *,
+    rand_bits: Optional[torch.Tensor] = None,
+    hadamard: Optional[HadamardTransform] = None,
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """bf16/fp32 tensor -> (packed E2M1 codes uint8, E8M0 scales uint8).
+
+    Layout contract of the reference (mxfp_quantization.py:439-448,484): the quantisation axis is moved last,
+    the results are computed densely in that orientation and returned transposed back, so ``axis=-2`` on
+    ``[M, C]`` yields logical ``[M/2, C]`` codes backed by ``[C][M/2]`` memory.
+
+    ``use_asm`` is accepted for signature compatibility and ignored (there is one implementation).
+    ``use_sr`` consumes ``rand_bits`` (int32/uint32, same shape as ``data_hp``; element ``[i, j]`` uses
+    ``rand_bits[i, j]``); when omitted the bits are drawn from torch's CUDA generator (seeded by
+    ``philox_seed``/``philox_offset`` if given).  ``hadamard`` fuses ``hadamard(x, left_mul=True)`` in front of
+    an ``axis=-2`` quantisation of a 2D tensor.
+    """
+    assert block_size == BLOCK_SIZE_DEFAULT, "only block_size=32 is implemented"
+    torch._check(data_hp.shape[axis] % block_size == 0)
+    assert not is_2d_block or data_hp.size(-2) % block_size == 0
+    assert data_hp.dtype in [torch.float32, torch.bfloat16]
+    clip = _clip_code(clip_mode)
+    rt.require_gpu(data_hp)
+    nd = data_hp.dim()
+    ax = axis % nd
+    if use_sr:
+        if rand_bits is None:
+            rand_bits = rt.draw_rand_bits(data_hp.shape, data_hp.device, philox_seed, philox_offset)
+        assert rand_bits.shape == data_hp.shape, "rand_bits must have the shape of data_hp"
+        rt.require_gpu(rand_bits)
+        rand_bits = _as_i32(rand_bits)
+    if hadamard is not None:
+        assert nd == 2 and ax == 0 and not is_2d_block, "hadamard fuses with a 1D axis=-2 quantisation of a 2D tensor"
+
+    if data_hp.numel() == 0:
+        xt = data_hp.transpose(ax, -1)
+        shp = xt.shape
+        codes = torch.empty((*shp[:-1], shp[-1] // 2), dtype=torch.uint8, device=data_hp.device)
+        ss = (*shp[:-2], shp[-2] // 32, shp[-1] // 32) if is_2d_block else (*shp[:-1], shp[-1] // 32)
+        return codes.transpose(ax, -1), torch.empty(ss, dtype=torch.uint8, device=data_hp.device).transpose(ax, -1)
+
+    if nd >= 2 and ax == nd - 2 and data_hp.shape[-1] % 8 == 0:
+        # quantise along the second-to-last dim: column output of the [.., M, C] matrices
+        x3 = _prep(data_hp)
+        r3 = None
+        if use_sr:
+            r3 = rand_bits.expand_as(data_hp)
+            r3 = _batched_view(r3 if r3.is_contiguous() else r3.contiguous())
+        _, _, cc, cs = _quantize_call(x3, False, True, is_2d_block, use_sr, r3, hadamard, clip, use_uos)
+        lead = data_hp.shape[:-2]
+        M, C = data_hp.shape[-2], data_hp.shape[-1]
+        codes = cc.reshape(*lead, C, M // 2).transpose(-1, -2)
+        scales = cs.reshape(*lead, C // 32 if is_2d_block else C, M // 32).transpose(-1, -2)
+        return codes, scales
+
+    # general case: move the axis last (view), then quantise along the contiguous dim
+    xt = data_hp.transpose(ax, -1)
+    shp = xt.shape
+    rtens = rand_bits.transpose(ax, -1) if use_sr else None
+    if is_2d_block:
+        x3 = _prep(xt)
+        r3 = None
+        if use_sr:
+            r3 = _batched_view(rtens.contiguous())
+        rcodes, rscales, _, _ = _quantize_call(x3, True, False, True, use_sr, r3, None, clip, use_uos)
+        codes = rcodes.reshape(*shp[:-1], shp[-1] // 2)
+        scales = rscales.reshape(*shp[:-2], shp[-2] // 32, shp[-1] // 32)
+    else:
+        x2 = xt.reshape(-1, shp[-1])
+        if x2.stride(-1) != 1 or not _aligned(x2):
+            x2 = x2.contiguous()
+        r3 = None
+        if use_sr:
+            r3 = rtens.reshape(-1, shp[-1]).contiguous().unsqueeze(0)
+        rcodes, rscales, _, _ = _quantize_call(x2.unsqueeze(0), True, False, False, use_sr, r3, None, clip, use_uos)
+        codes = rcodes.reshape(*shp[:-1], shp[-1] // 2)
+        scales = rscales.reshape(*shp[:-1], shp[-1] // 32)
+    return codes.transpose(ax, -1), scales.transpose(ax, -1)
+
+
+def quantize_rowcol(
+    x: torch.Tensor,
+    is_2d_block: bool = False,
+    use_sr: bool = False,
+    rand_bits: Optional[torch.Tensor] = None,
+    hadamard: Optional[HadamardTransform] = None,
+    clip_mode: str = "none",
+    use_uos: bool = False,
+):
+    """One pass over a 2D ``x [M, C]`` producing BOTH quantisations the linear layer needs.
+
+    Returns ``(row_codes [M, C/2], row_scales, col_codes, col_scales)`` where the column pair equals
+    ``convert_to_mxfp4(hadamard(x) if hadamard else x, axis=0, ...)`` (transposed views over ``[C][M/2]`` memory,
+    ``clip_mode`` applied there) and the row pair equals ``convert_to_mxfp4(x, axis=-1, ...)`` (no transform, no
+    clipping).  Fuses mxfp_linear.py:310-315 with :383-396 (forward, x) and
+    :466-494 (backward, dY); for 2D blocks it yields both packings of a weight from one read.
+    """
+    assert x.dim() == 2 and x.dtype in (torch.float32, torch.bfloat16)
+    rt.require_gpu(x)
+    M, C = x.shape
+    torch._check(M % 32 == 0 and C % 32 == 0)
+    clip = _clip_code(clip_mode)
+    x3 = _prep(x)
+    r3 = None
+    if use_sr:
+        if rand_bits is None:
+            rand_bits = rt.draw_rand_bits(x.shape, x.device)
+        assert rand_bits.shape == x.shape
+        r3 = _as_i32(rand_bits)
+        r3 = _batched_view(r3 if r3.stride(-1) == 1 and r3.stride(0) % 4 == 0 and r3.data_ptr() % 16 == 0 else r3.contiguous())
+    rc, rs, cc, cs = _quantize_call(x3, True, True, is_2d_block, use_sr, r3, hadamard, clip, use_uos)
+    return rc[0], rs[0], cc[0].transpose(0, 1), cs[0].transpose(0, 1)
+
+
+def hadamard_left(x: torch.Tensor, h: HadamardTransform) -> torch.Tensor:
+    """``h(x, left_mul=True)``: the transform along dim 0 in blocks of 32 rows, output in the dtype of ``x``."""
+    assert x.dim() == 2 and x.dtype in (torch.float32, torch.bfloat16)
+    rt.require_gpu(x)
+    torch._check(x.shape[0] % 32 == 0)
+    xc = x if x.stride(-1) == 1 else x.contiguous()
+    y = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+    M, C = x.shape
+    if M == 0 or C == 0:
+        return y
+    rc = rt.lib().alto_mxfp4_hadamard(xc.data_ptr(), rt.dtype_code(x.dtype), M, C, xc.stride(0), y.data_ptr(), y.stride(0),
+                                      h.signs.data_ptr(), None if h.perm is None else h.perm.data_ptr(), rt.stream_ptr(x.device))
+    check(rc, "alto_mxfp4_hadamard")
+    return y
+
+
+def convert_from_mxfp4(
+    data_lp: torch.Tensor,
+    scales: torch.Tensor,
+    output_dtype: torch.dtype = torch.float32,
+    block_size: int = BLOCK_SIZE_DEFAULT,
+    axis: int = -1,
+    is_2d_block: bool = False,
+    use_asm: Optional[bool] = None,
+    clip_mode: str = "none",
+) -> torch.Tensor:
+    """(packed codes, scales) -> tensor of ``output_dtype`` (mxfp_quantization.py:487-545)."""
+    assert output_dtype in [torch.float32, torch.bfloat16]
+    assert block_size == BLOCK_SIZE_DEFAULT
+    clip = _clip_code(clip_mode)
+    rt.require_gpu(data_lp, scales)
+    lt = data_lp.transpose(axis, -1)
+    st = scales.transpose(axis, -1)
+    orig = (*lt.shape[:-1], lt.shape[-1] * 2)
+    l2 = lt.reshape(-1, lt.shape[-1]).contiguous()
+    R, C = l2.shape[0], l2.shape[1] * 2
+    s2 = st.reshape(-1, C // 32).contiguous()
+    out = torch.empty((R, C), dtype=output_dtype, device=data_lp.device)
+    if R and C:
+        if is_2d_block:
+            assert orig[-2] % 32 == 0
+        rc = rt.lib().alto_mxfp4_dequantize(l2.data_ptr(), s2.data_ptr(), R, C, int(is_2d_block), out.data_ptr(),
+                                            rt.dtype_code(output_dtype), C, 1, clip, rt.stream_ptr(data_lp.device))
+        check(rc, "alto_mxfp4_dequantize")
+    return out.reshape(orig).transpose(axis, -1)

@@ -1,0 +1,220 @@
+"""GPU parity of the HIP quantizer / dequantizer / Hadamard against the CPU oracle: packed codes and scales bit-exact."""
+import numpy as np
+import pytest
+import torch
+
+import oracle as O
+from tests.helpers import assert_bytes_equal, hadamard_from_seed, laplace, rand_bits, randn_outliers
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def m():
+    import alto_amd.mxfp4 as mod
+    assert torch.cuda.is_available(), "GPU tests need an MI355X"
+    return mod
+
+
+def _check_pair(got, exp, what):
+    assert_bytes_equal(got[1], exp[1], what + " scales")
+    assert_bytes_equal(got[0], exp[0], what + " codes")
+
+
+# the reference's own matrix (tests/unittest/mxfp4/test_mxfp_quantization.py:23-31), with explicit random bits for SR
+@pytest.mark.parametrize("shape", [(128, 64), (2048, 2048), (4, 128, 64)])
+@pytest.mark.parametrize("axis", [-1, -2])
+@pytest.mark.parametrize("is_2d", [False, True])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("use_sr", [False, True])
+def test_quantize_matches_oracle(m, shape, axis, is_2d, dtype, use_sr):
+    x = randn_outliers(shape, dtype, seed=1234)
+    r = rand_bits(shape, seed=99) if use_sr else None
+    exp = O.quantize(x, axis=axis, is_2d_block=is_2d, use_sr=use_sr, rand_bits=r)
+    got = m.convert_to_mxfp4(x.to(DEV), axis=axis, is_2d_block=is_2d, use_sr=use_sr, rand_bits=None if r is None else r.to(DEV))
+    assert got[0].stride() == exp[0].stride() and got[1].stride() == exp[1].stride(), "layout contract (transposed views)"
+    _check_pair(got, exp, f"quantize{shape} axis={axis} 2d={is_2d} {dtype} sr={use_sr}")
+    # dequantize: GPU vs oracle on the GPU's own codes (exact: same fp32 product, one cast)
+    for out_dtype in (torch.float32, torch.bfloat16):
+        dq = m.convert_from_mxfp4(got[0], got[1], out_dtype, axis=axis, is_2d_block=is_2d)
+        dq_ref = O.dequantize(exp[0], exp[1], out_dtype, axis=axis, is_2d_block=is_2d)
+        assert dq.shape == dq_ref.shape
+        assert torch.equal(dq.cpu(), dq_ref)
+
+
+@pytest.mark.parametrize("clip_mode,use_uos", [("static", False), ("none", True)])
+@pytest.mark.parametrize("axis", [-1, 0])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("use_sr", [False, True])
+def test_quantize_clip_and_uos(m, clip_mode, use_uos, axis, dtype, use_sr):
+    x = randn_outliers((256, 192), dtype, seed=7)
+    r = rand_bits(x.shape, seed=8) if use_sr else None
+    exp = O.quantize(x, axis=axis, use_sr=use_sr, rand_bits=r, clip_mode=clip_mode, use_uos=use_uos)
+    got = m.convert_to_mxfp4(x.to(DEV), axis=axis, use_sr=use_sr, rand_bits=None if r is None else r.to(DEV), clip_mode=clip_mode, use_uos=use_uos)
+    _check_pair(got, exp, f"clip={clip_mode} uos={use_uos} axis={axis}")
+    dq = m.convert_from_mxfp4(got[0], got[1], dtype, axis=axis, clip_mode=clip_mode)
+    assert torch.equal(dq.cpu(), O.dequantize(exp[0], exp[1], dtype, axis=axis, clip_mode=clip_mode))
+
+
+def _exhaustive_bf16_rows():
+    """Every finite bf16 value appears under many block scales: rows of 32 = one anchor (sets the absmax) + 31 payload values."""
+    bits = np.arange(0, 0x10000, dtype=np.uint32)
+    bits = bits[(bits & 0x7F80) != 0x7F80].astype(np.uint16)            # finite
+    rows = []
+    anchors = [0x0000, 0x0001, 0x007F, 0x0080, 0x00C0, 0x0200, 0x1000, 0x3F80, 0x3FC0, 0x3FDF, 0x3FE0, 0x40C0, 0x40E0,
+               0x4780, 0x5F00, 0x7000, 0x7E80, 0x7F7F]
+    for a in anchors:
+        keep = bits[(bits & 0x7FFF) <= a]                                 # payload never exceeds the anchor
+        if keep.size == 0:
+            keep = np.array([0], dtype=np.uint16)
+        pad = (-keep.size) % 31
+        keep = np.concatenate([keep, np.zeros(pad, dtype=np.uint16)])
+        blk = keep.reshape(-1, 31)
+        rows.append(np.concatenate([np.full((blk.shape[0], 1), a, dtype=np.uint16), blk], axis=1))
+    allrows = np.concatenate(rows, axis=0)
+    pad = (-allrows.shape[0]) % 32
+    allrows = np.concatenate([allrows, np.zeros((pad, 32), dtype=np.uint16)])
+    return torch.from_numpy(allrows.astype(np.int16)).view(torch.bfloat16)
+
+
+@pytest.mark.parametrize("use_sr", [False, True])
+def test_quantize_exhaustive_bf16(m, use_sr):
+    x = _exhaustive_bf16_rows()
+    r = rand_bits(x.shape, seed=5) if use_sr else None
+    if use_sr:  # force the compare-with-threshold corner cases to occur
+        r[:, 1] = 0
+        r[:, 2] = -1
+        r[:, 3] = 0x3FFFFF
+    exp = O.quantize(x, use_sr=use_sr, rand_bits=r)
+    got = m.convert_to_mxfp4(x.to(DEV), use_sr=use_sr, rand_bits=None if r is None else r.to(DEV))
+    _check_pair(got, exp, f"exhaustive bf16 sr={use_sr}")
+    # same values as fp32 input: identical codes (bf16 -> fp32 is exact), scales by the fp32 rule
+    xf = x.float()
+    exp = O.quantize(xf, use_sr=use_sr, rand_bits=r)
+    got = m.convert_to_mxfp4(xf.to(DEV), use_sr=use_sr, rand_bits=None if r is None else r.to(DEV))
+    _check_pair(got, exp, f"exhaustive bf16-as-fp32 sr={use_sr}")
+
+
+@pytest.mark.parametrize("use_sr", [False, True])
+def test_quantize_fp32_wide_exponents(m, use_sr):
+    g = torch.Generator().manual_seed(31)
+    x = torch.randn(512, 256, generator=g) * torch.exp2(torch.randint(-140, 120, (512, 256 // 32), generator=g).float()).repeat_interleave(32, dim=1)
+    x[0, :32] = 0
+    x[1, :32] = torch.tensor(1e-45)
+    r = rand_bits(x.shape, seed=32) if use_sr else None
+    exp = O.quantize(x, use_sr=use_sr, rand_bits=r)
+    got = m.convert_to_mxfp4(x.to(DEV), use_sr=use_sr, rand_bits=None if r is None else r.to(DEV))
+    _check_pair(got, exp, f"fp32 wide exponents sr={use_sr}")
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("shape", [(32, 8), (64, 40), (256, 512), (1024, 2880)])
+def test_hadamard_standalone_bit_exact(m, dtype, shape):
+    signs, perm = hadamard_from_seed(1234)
+    x = laplace(shape, 1e-3, dtype, seed=3)
+    h = m.HadamardTransform(signs, perm)
+    y = h(x.to(DEV), left_mul=True)
+    assert torch.equal(y.cpu(), O.rht_left(x, signs, perm))
+    # against the reference's dense formulation in fp64: one rounding of the output dtype plus the fp32 summation error,
+    # which scales with the magnitude of the 32 terms (the two differ only in summation order)
+    yd = O.rht_left_dense(x, signs, perm, torch.float64)
+    eps = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -24
+    sum_err = 2.0 ** -21 * float(x.abs().max()) * 32 ** 0.5
+    assert bool(((y.cpu().double() - yd).abs() <= eps * yd.abs() + sum_err).all())
+    h0 = m.HadamardTransform(torch.ones(32, dtype=torch.int8), None)
+    assert torch.equal(h0(x.to(DEV), left_mul=True).cpu(), O.rht_left(x, torch.ones(32), None))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("use_sr", [False, True])
+@pytest.mark.parametrize("use_h", [False, True])
+@pytest.mark.parametrize("clip_mode", ["none", "static"])
+def test_fused_rowcol_equals_two_reference_calls(m, dtype, use_sr, use_h, clip_mode):
+    """One pass == convert_to_mxfp4(x, axis=-1) and convert_to_mxfp4(H(x), axis=0) of the reference (mxfp_linear.py:466-494)."""
+    M, C = 512, 320
+    x = laplace((M, C), 1e-3, dtype, seed=11)
+    r = rand_bits((M, C), seed=12) if use_sr else None
+    signs, perm = hadamard_from_seed(1234)
+    h = m.HadamardTransform(signs, perm) if use_h else None
+    rq, rs, cq, cs = m.quantize_rowcol(x.to(DEV), False, use_sr=use_sr, rand_bits=None if r is None else r.to(DEV), hadamard=h, clip_mode=clip_mode)
+    _check_pair((rq, rs), O.quantize(x, axis=-1, use_sr=use_sr, rand_bits=r), "fused row")  # the row copy is never clipped
+    xh = O.rht_left(x, signs, perm) if use_h else x
+    _check_pair((cq, cs), O.quantize(xh, axis=0, use_sr=use_sr, rand_bits=r, clip_mode=clip_mode), "fused col")
+    # and the unfused HIP path gives the same bytes
+    c2 = m.convert_to_mxfp4(x.to(DEV), axis=0, use_sr=use_sr, rand_bits=None if r is None else r.to(DEV), hadamard=h, clip_mode=clip_mode)
+    assert torch.equal(c2[0], cq) and torch.equal(c2[1], cs)
+
+
+def test_fused_2d_weight_gives_both_packings(m):
+    w = randn_outliers((384, 256), torch.bfloat16, seed=4) * 0.02
+    rq, rs, cq, cs = m.quantize_rowcol(w.to(DEV), True)
+    _check_pair((rq, rs), O.quantize(w, axis=-1, is_2d_block=True), "2D row packing")
+    _check_pair((cq, cs), O.quantize(w, axis=0, is_2d_block=True), "2D col packing")
+    assert torch.equal(m.transpose_codes(rq).cpu(), cq.T.contiguous().cpu())
+
+
+def test_config1_roundtrip_full_size(m):
+    """BASELINE config 1: bf16 [4096, 4096] ~ N(0,1) with 1% entries x50, 1D blocks, RNE, no Hadamard."""
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(4096, 4096, generator=g)
+    x = torch.where(torch.rand(4096, 4096, generator=g) < 0.01, x * 50, x).bfloat16()
+    exp = O.quantize(x)
+    got = m.convert_to_mxfp4(x.to(DEV))
+    assert got[0].shape == (4096, 2048) and got[1].shape == (4096, 128)
+    _check_pair(got, exp, "config1")
+    dq = m.convert_from_mxfp4(got[0], got[1], torch.bfloat16)
+    assert torch.equal(dq.cpu(), O.dequantize(exp[0], exp[1], torch.bfloat16))
+    # idempotence: dequantized values are representable, so re-quantizing them reproduces codes and scales
+    again = m.convert_to_mxfp4(dq)
+    dq2 = m.convert_from_mxfp4(again[0], again[1], torch.bfloat16)
+    assert torch.equal(dq2, dq)
+
+
+def test_config2_fused_gradient_quantizer_full_size(m):
+    """BASELINE config 2: bf16 [8192, 4096] ~ Laplace(0, 1e-3), row copy + Hadamard column copy, SR with supplied bits."""
+    M, C = 8192, 4096
+    x = laplace((M, C), 1e-3, torch.bfloat16, seed=21)
+    r = rand_bits((M, C), seed=22)
+    signs, perm = hadamard_from_seed(1234)
+    h = m.HadamardTransform(signs, perm)
+    rq, rs, cq, cs = m.quantize_rowcol(x.to(DEV), False, use_sr=True, rand_bits=r.to(DEV), hadamard=h)
+    assert rq.shape == (M, C // 2) and rs.shape == (M, C // 32)
+    assert cq.shape == (M // 2, C) and cq.stride() == (1, M // 2) and cs.shape == (M // 32, C) and cs.stride() == (1, M // 32)
+    # oracle on a spread of 32-row blocks (quantisation is local to a block row, so slices compare exactly)
+    for b0 in [0, 37, 100, 255]:
+        sl = slice(32 * b0, 32 * (b0 + 4))
+        exp_r = O.quantize(x[sl], axis=-1, use_sr=True, rand_bits=r[sl])
+        _check_pair((rq[sl], rs[sl]), exp_r, f"cfg2 row blocks {b0}")
+        exp_c = O.quantize(O.rht_left(x[sl], signs, perm), axis=0, use_sr=True, rand_bits=r[sl])
+        _check_pair((cq[16 * b0:16 * (b0 + 4)], cs[b0:b0 + 4]), exp_c, f"cfg2 col blocks {b0}")
+    # whole-tensor property: stochastic rounding is unbiased, so the dequantized row copy averages to the input
+    dq = m.convert_from_mxfp4(rq, rs, torch.float32)
+    xd = x.to(DEV).float()
+    rel = float((dq - xd).mean().abs() / xd.abs().mean())
+    assert rel < 2e-3, rel
+    # the transform is orthogonal: energy of the dequantized column copy ~ energy of the input
+    dqc = m.convert_from_mxfp4(cq, cs, torch.float32, axis=0)
+    e = float((dqc ** 2).sum() / (xd ** 2).sum())
+    assert 0.9 < e < 1.15, e
+
+
+def test_edge_cases(m):
+    # empty
+    c, s = m.convert_to_mxfp4(torch.zeros(0, 64, device=DEV))
+    assert c.shape == (0, 32) and s.shape == (0, 2)
+    # all-zero and tiny blocks
+    x = torch.zeros(32, 64, dtype=torch.bfloat16)
+    x[0, 0] = 1e-40
+    exp = O.quantize(x)
+    _check_pair(m.convert_to_mxfp4(x.to(DEV)), exp, "zeros/subnormals")
+    # rows not a multiple of the tile, columns ragged vs the 256-wide tile
+    x = randn_outliers((37, 288), torch.bfloat16, seed=9)
+    _check_pair(m.convert_to_mxfp4(x.to(DEV)), O.quantize(x), "ragged rows")
+    # non-contiguous input
+    xt = randn_outliers((96, 160), torch.float32, seed=10).T
+    _check_pair(m.convert_to_mxfp4(xt.to(DEV).T.contiguous().T, axis=-1), O.quantize(xt, axis=-1), "transposed input")
+    with pytest.raises(RuntimeError):
+        m.convert_to_mxfp4(torch.zeros(32, 48, device=DEV))
+    with pytest.raises(NotImplementedError):
+        m.convert_to_mxfp4(torch.zeros(32, 64, device=DEV), clip_mode="dynamic")

@@ -1,0 +1,96 @@
+"""CPU-side checks: the C-ABI library builds, loads and exports what the header declares; host logic without a GPU."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def header_symbols():
+    text = open(os.path.join(ROOT, "include", "alto_mxfp4.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(alto_mxfp4_\w+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    from alto_amd import _lib
+    lib = _lib.load()
+    names = header_symbols()
+    assert "alto_mxfp4_quantize" in names and "alto_mxfp4_gemm" in names and len(names) >= 9
+    for n in names:
+        assert hasattr(lib, n), f"{n} is declared in include/alto_mxfp4.h but not exported"
+    assert set(names) == set(_lib.SIGNATURES), "ctypes signature table and header disagree"
+    assert lib.alto_mxfp4_version() >= 1
+
+
+def test_argument_validation_needs_no_gpu():
+    from alto_amd import _lib
+    lib = _lib.load()
+    # NULL input is rejected before any HIP call
+    rc = lib.alto_mxfp4_quantize(None, 0, 1, 32, 32, 32, 1024, None, None, None, None, 0, 0, None, 0, 0, 0, None, None, 0, 0, None)
+    assert rc == -1 and b"NULL" in lib.alto_mxfp4_last_error()
+    buf = ctypes.create_string_buffer(4096)
+    p = ctypes.addressof(buf)
+    p += (-p) % 16
+    rc = lib.alto_mxfp4_quantize(p, 0, 1, 32, 40, 40, 1280, p, p, None, None, 0, 0, None, 0, 0, 0, None, None, 0, 0, None)
+    assert rc == -1 and b"C (40)" in lib.alto_mxfp4_last_error()
+    rc = lib.alto_mxfp4_quantize(p, 0, 1, 32, 32, 32, 1024, p, p, None, None, 0, 0, None, 0, 0, 0, None, None, 2, 0, None)
+    assert rc == -3  # dynamic clip: declared, not implemented
+    rc = lib.alto_mxfp4_gemm(p, 16, p, 1, 1, 0, p, 16, p, 1, 1, 0, 32, 32, 48, p, 0, 32, 1.0, None)
+    assert rc == -1 and b"K (48)" in lib.alto_mxfp4_last_error()
+    bad_perm = (ctypes.c_uint8 * 32)(*([0] * 32))
+    signs = (ctypes.c_int8 * 32)(*([1] * 32))
+    rc = lib.alto_mxfp4_hadamard(p, 0, 32, 8, 8, p, 8, ctypes.addressof(signs), ctypes.addressof(bad_perm), None)
+    assert rc == -1 and b"permutation" in lib.alto_mxfp4_last_error()
+
+
+def test_ops_refuse_cpu_tensors():
+    import alto_amd.mxfp4 as m
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        m.convert_to_mxfp4(torch.randn(32, 32))
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        m.convert_from_mxfp4(torch.zeros(32, 16, dtype=torch.uint8), torch.zeros(32, 1, dtype=torch.uint8))
+    with pytest.raises(ValueError, match="Invalid clip mode"):
+        m.convert_to_mxfp4(torch.randn(32, 32), clip_mode="bogus")
+    with pytest.raises(RuntimeError):
+        m.convert_to_mxfp4(torch.randn(32, 48))  # torch._check on the block divisibility
+
+
+def test_hadamard_factory_matches_reference_draw_order():
+    import oracle as O
+    from alto_amd.mxfp4 import HadamardFactory
+    from tests.helpers import hadamard_from_seed
+    HadamardFactory.configure(seed=1234)
+    t = HadamardFactory.create_transform()
+    signs, perm = hadamard_from_seed(1234)
+    assert torch.equal(t.signs, signs) and torch.equal(t.perm.long(), perm)
+    assert torch.equal(t.weight, O.hadamard_matrix(signs, perm))
+    t2 = HadamardFactory.create_transform()          # the class-level generator advances between calls
+    assert not (torch.equal(t2.signs, t.signs) and torch.equal(t2.perm, t.perm))
+    with pytest.raises(NotImplementedError):
+        t(torch.zeros(32, 8), left_mul=False)
+
+
+def test_training_op_config():
+    from alto_amd.mxfp4 import TrainingOpConfig
+    c = TrainingOpConfig()
+    assert (c.use_2dblock_x, c.use_2dblock_w, c.use_hadamard, c.use_sr_grad, c.use_dge, c.clip_mode) == (False, True, True, True, False, "none")
+    with pytest.raises(ValueError):
+        TrainingOpConfig(precision="nvfp4")
+    with pytest.raises(ValueError):
+        TrainingOpConfig(clip_mode="x")
+
+
+def test_group_helpers():
+    import oracle as O
+    from alto_amd.mxfp4 import grouped_gemm as G
+    ends = torch.tensor([128, 128, 384, 512], dtype=torch.int32)
+    idx = G.create_indices_from_offsets_nosync(ends)
+    assert torch.equal(idx, O.indices_from_offsets(ends))
+    g = G.groups_from_indices(idx)
+    assert g.n == 4 and g.offs.tolist() == [0, 128, 256, 384, 512] and g.expert.tolist() == [0, 2, 2, 3]
+    off = G.offsets_from_ends(ends)
+    assert off.tolist() == [0, 128, 128, 384, 512] and G.groups_from_offsets(off).n == 4
