@@ -24,6 +24,7 @@ int check_launch(const char* what);
 // ----------------------------------------------------------------------------- device: bit casts
 typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
 typedef int v8i_t __attribute__((ext_vector_type(8)));
+typedef int v4i_t __attribute__((ext_vector_type(4)));
 typedef float v4f_t __attribute__((ext_vector_type(4)));
 typedef float v16f_t __attribute__((ext_vector_type(16)));
 

@@ -1,0 +1,339 @@
+#!/usr/bin/env python3
+"""Benchmark of the MXFP4 hot path on one MI355X.
+
+``python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]`` prints ONE JSON line.
+
+The default workload is the MXFP4 fprop GEMM at the Llama-3-8B MLP up-projection shape (config 3 of BASELINE.json):
+a "step" is one GEMM launch on operands already quantized and resident in HBM; ``value`` is TFLOP/s.  The same line
+carries the fused RHT+SR gradient quantizer (config 2, GB/s) and the other GEMM shapes under ``"others"``, a
+``roofline`` object for the dominant kernel of the selected workload (duration measured live with HIP events on the
+launch stream) and a ``cpu_baseline`` (the CPU oracle timed on a bounded sample of the same workload on this box's
+host cores).  All data is synthetic (seeded torch generators) and random-init; nothing is read from disk.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_MXFP4_TFLOPS = 10100.0   # MI355X dense FP4 MFMA peak (published), TFLOP/s
+PEAK_HBM_GBS = 8000.0         # MI355X HBM3E peak (published), GB/s
+METRIC = "MXFP4 GEMM TFLOPS (% MFMA peak) + quantizer GB/s, Llama-3-8B shapes, 1 MI355X"
+
+
+def _laplace(shape, scale, device, gen):
+    import torch
+    u = (torch.rand(shape, device=device, generator=gen) - 0.5).clamp(-0.4999999, 0.4999999)
+    return (-scale * torch.sign(u) * torch.log1p(-2 * u.abs())).bfloat16()
+
+
+def _time_steps(fn, steps, warmup):
+    """Average milliseconds per call of fn, HIP events on the current stream bracketing exactly `steps` calls."""
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(steps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    return e0.elapsed_time(e1) / steps, wall_ms
+
+
+# ------------------------------------------------------------------------------------------------ workloads
+class Workload:
+    name = ""
+    bound = "mfma"
+    kernel = ""
+
+    def setup(self, dev, gen):
+        raise NotImplementedError
+
+    def step(self):
+        raise NotImplementedError
+
+    work = 0.0  # algorithmic FLOPs (mfma) or bytes (hbm) per step
+
+    def cpu_sample(self):
+        """-> (callable, work_of_sample, description)"""
+        raise NotImplementedError
+
+
+class FusedGradQuant(Workload):
+    """Config 2: dY bf16 [8192, 4096] ~ Laplace(0, 1e-3) -> row copy (SR) + Hadamard column copy (SR), supplied random bits."""
+    name = "cfg2_fused_rht_sr_quantizer[8192x4096]"
+    bound = "hbm"
+    kernel = "quant_kernel<bf16, row+col, SR, RHT>"
+    M, C = 8192, 4096
+
+    def setup(self, dev, gen):
+        import torch
+        import alto_amd.mxfp4 as m
+        self.m = m
+        self.x = _laplace((self.M, self.C), 1e-3, dev, gen)
+        self.r = torch.randint(-2 ** 31, 2 ** 31, (self.M, self.C), dtype=torch.int32, device=dev, generator=gen)
+        m.HadamardFactory.configure(seed=1234)
+        self.h = m.HadamardFactory.create_transform()
+        # algorithmic bytes: dY + random bits in, two code tensors + two scale tensors out
+        self.work = self.M * self.C * 2 + self.M * self.C * 4 + 2 * (self.M * self.C // 2 + self.M * self.C // 32)
+
+    def step(self):
+        return self.m.quantize_rowcol(self.x, False, use_sr=True, rand_bits=self.r, hadamard=self.h)
+
+    def cpu_sample(self):
+        import oracle as O
+        rows = 512
+        x = self.x[:rows].cpu()
+        r = self.r[:rows].cpu()
+        signs, perm = self.h.signs, self.h.perm.long()
+
+        def run():
+            O.quantize(x, axis=-1, use_sr=True, rand_bits=r)
+            O.quantize(O.rht_left(x, signs, perm), axis=0, use_sr=True, rand_bits=r)
+        return run, self.work * rows / self.M, f"first {rows} of {self.M} rows, both copies"
+
+
+class RneQuant(Workload):
+    """Config 1: bf16 [4096, 4096] ~ N(0,1) with 1% x50 outliers, 1D-32 blocks, RNE, no Hadamard."""
+    name = "cfg1_rne_quantizer[4096x4096]"
+    bound = "hbm"
+    kernel = "quant_kernel<bf16, row, RNE>"
+    M, C = 4096, 4096
+
+    def setup(self, dev, gen):
+        import torch
+        import alto_amd.mxfp4 as m
+        self.m = m
+        x = torch.randn(self.M, self.C, device=dev, generator=gen)
+        self.x = torch.where(torch.rand(self.M, self.C, device=dev, generator=gen) < 0.01, x * 50, x).bfloat16()
+        self.work = self.M * self.C * 2 + self.M * self.C // 2 + self.M * self.C // 32
+
+    def step(self):
+        return self.m.convert_to_mxfp4(self.x)
+
+    def cpu_sample(self):
+        import oracle as O
+        rows = 1024
+        x = self.x[:rows].cpu()
+        return (lambda: O.quantize(x)), self.work * rows / self.M, f"first {rows} of {self.M} rows"
+
+
+class Gemm(Workload):
+    """Dense NT GEMM on pre-quantized operands: C[M,N] = A[M,K] . B[N,K]^T."""
+    bound = "mfma"
+    kernel = "gemm"
+
+    def __init__(self, name, M, N, K, a_2d, b_2d, a_kind, b_kind):
+        self.name, self.M, self.N, self.K = name, M, N, K
+        self.a_2d, self.b_2d, self.a_kind, self.b_kind = a_2d, b_2d, a_kind, b_kind
+        self.work = 2.0 * M * N * K
+
+    def _operand(self, rows, kind, is_2d, dev, gen):
+        import torch
+        if kind == "act":
+            t = torch.randn(rows, self.K, device=dev, generator=gen).bfloat16()
+        elif kind == "weight":
+            t = (torch.randn(rows, self.K, device=dev, generator=gen) * 0.02).bfloat16()
+        else:
+            t = _laplace((rows, self.K), 1e-3, dev, gen)
+        return self.m.convert_to_mxfp4(t, is_2d_block=is_2d)
+
+    def setup(self, dev, gen):
+        import torch
+        import alto_amd.mxfp4 as m
+        self.m = m
+        self.aq, self.as_ = self._operand(self.M, self.a_kind, self.a_2d, dev, gen)
+        self.bq, self.bs = self._operand(self.N, self.b_kind, self.b_2d, dev, gen)
+
+    def step(self):
+        import torch
+        return self.m.blockwise_mxfp4_gemm(self.aq, self.as_, self.bq, self.bs, use_2dblock_a=self.a_2d, use_2dblock_b=self.b_2d,
+                                           trans_b=True, output_dtype=torch.bfloat16)
+
+    def cpu_sample(self):
+        import torch
+        import oracle as O
+        rows = 256
+        aq, as_ = self.aq[:rows].cpu(), (self.as_[:rows // 32] if self.a_2d else self.as_[:rows]).cpu()
+        bq, bs = self.bq.cpu(), self.bs.cpu()
+
+        def run():  # the reference's dequantize-then-matmul branch (mxfp_linear.py:337-356)
+            O.gemm_ref(aq, as_, bq, bs, self.a_2d, self.b_2d, trans_b=True, dtype=torch.float32)
+        return run, self.work * rows / self.M, f"{rows} of {self.M} rows of A against all of B, dequantize + fp32 matmul"
+
+
+class GroupedGemm(Workload):
+    """Config 5: 32 experts, hidden 2880 -> 5760, 65536 routed rows with Zipf(1.1) expert skew, ragged int32 offsets [33]."""
+    name = "cfg5_grouped_gemm[65536x5760x2880,E=32]"
+    bound = "mfma"
+    kernel = "grouped_gemm"
+    E, N, K, T, TOPK = 32, 5760, 2880, 16384, 4
+
+    def setup(self, dev, gen):
+        import torch
+        import alto_amd.mxfp4 as m
+        from alto_amd.mxfp4 import grouped_gemm as G
+        self.m, self.G = m, G
+        rows = self.T * self.TOPK
+        logits = torch.randn(self.T, self.E, device=dev, generator=gen)
+        skew = torch.log(1.0 / torch.arange(1, self.E + 1, device=dev).float() ** 1.1)
+        top = torch.topk(torch.softmax(logits + skew, dim=-1), self.TOPK, dim=-1).indices.reshape(-1)
+        counts = torch.bincount(top, minlength=self.E)
+        offs = torch.cat([torch.zeros(1, dtype=torch.int64, device=dev), counts.cumsum(0)]).to(torch.int32)
+        self.groups = G.groups_from_offsets(offs)
+        a = torch.randn(rows, self.K, device=dev, generator=gen).bfloat16()
+        self.aq, self.as_ = m.convert_to_mxfp4(a)
+        del a
+        w = (torch.randn(self.E, self.N, self.K, device=dev, generator=gen) * 0.02).bfloat16()
+        self.wq, self.ws = m.convert_to_mxfp4(w, is_2d_block=True)
+        del w
+        self.rows = rows
+        self.work = 2.0 * rows * self.N * self.K
+
+    def step(self):
+        import torch
+        return self.G.grouped_forward(self.aq, self.as_, self.wq, self.ws, self.groups, False, True, torch.bfloat16)
+
+    def cpu_sample(self):
+        import torch
+        import oracle as O
+        offs = self.groups.offs.cpu()
+        e = int(torch.argmax(offs[1:] - offs[:-1]))
+        lo = int(offs[e])
+        rows = min(256, int(offs[e + 1]) - lo)
+        aq, as_ = self.aq[lo:lo + rows].cpu(), self.as_[lo:lo + rows].cpu()
+        wq, ws = self.wq[e].cpu(), self.ws[e].cpu()
+
+        def run():
+            O.gemm_ref(aq, as_, wq, ws, False, True, trans_b=True, dtype=torch.float32)
+        return run, 2.0 * rows * self.N * self.K, f"{rows} rows of the largest expert, dequantize + fp32 matmul"
+
+
+def make_workloads():
+    return {
+        "cfg3_fprop": Gemm("cfg3_fprop_gemm[8192x14336x4096]", 8192, 14336, 4096, False, True, "act", "weight"),
+        "cfg2_quant": FusedGradQuant(),
+        "cfg1_quant": RneQuant(),
+        # config 4: dgrad dX[8192,14336] = dY[8192,4096] . W^T-packed[14336,4096]; wgrad dW[4096,14336] over 8192 tokens
+        "cfg4_dgrad": Gemm("cfg4_dgrad_gemm[8192x14336x4096]", 8192, 14336, 4096, False, True, "grad", "weight"),
+        "cfg4_wgrad": Gemm("cfg4_wgrad_gemm[4096x14336x8192]", 4096, 14336, 8192, False, False, "grad", "act"),
+        "cfg5_grouped": GroupedGemm(),
+    }
+
+
+def measure(w, dev, gen, steps, warmup):
+    import torch
+    w.setup(dev, gen)
+    torch.cuda.synchronize()
+    ms, wall_ms = _time_steps(w.step, steps, warmup)
+    if w.bound == "mfma":
+        achieved, peak, unit = w.work / (ms * 1e-3) / 1e12, PEAK_MXFP4_TFLOPS, "TFLOP/s"
+    else:
+        achieved, peak, unit = w.work / (ms * 1e-3) / 1e9, PEAK_HBM_GBS, "GB/s"
+    return {"workload": w.name, "kernel": w.kernel, "ms": ms, "wall_ms": wall_ms, "achieved": achieved, "peak": peak, "unit": unit,
+            "bound": w.bound, "frac": achieved / peak}
+
+
+def cpu_baseline(w):
+    import torch
+    torch.set_num_threads(min(os.cpu_count() or 1, 16))
+    fn, work, desc = w.cpu_sample()
+    fn()  # warm-up
+    times = []
+    t_all = time.perf_counter()
+    while len(times) < 3 and time.perf_counter() - t_all < 30:
+        t0 = time.perf_counter()
+        fn()
+        times.append(time.perf_counter() - t0)
+    t = sorted(times)[len(times) // 2]
+    if w.bound == "mfma":
+        value, unit = work / t / 1e12, "TFLOP/s"
+    else:
+        value, unit = work / t / 1e9, "GB/s"
+    return {"value": value, "unit": unit, "cores": torch.get_num_threads(), "kind": "port", "sample": desc, "seconds": t}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="cfg3_fprop", help="primary workload; one of " + ", ".join(make_workloads()))
+    ap.add_argument("--only", action="store_true", help="measure the primary workload only (for profiling runs)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (every kernel is per-shard; see DESIGN.md). "
+              "Run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py needs an MI355X: torch.cuda.is_available() is False", file=sys.stderr)
+        sys.exit(1)
+    from alto_amd import _lib
+    _lib.load()  # fail loudly if the HIP library is missing
+    dev = torch.device("cuda:0")
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(1234)
+    props = torch.cuda.get_device_properties(0)
+
+    wl = make_workloads()
+    if args.workload not in wl:
+        print(f"unknown workload {args.workload}", file=sys.stderr)
+        sys.exit(2)
+    primary = wl[args.workload]
+    res = measure(primary, dev, gen, args.steps, args.warmup)
+    cpu = None if args.no_cpu else cpu_baseline(primary)
+    others = {}
+    if not args.only:
+        for key, w in wl.items():
+            if key == args.workload:
+                continue
+            primary_mem_release = None  # noqa: F841
+            try:
+                r = measure(w, dev, gen, max(5, args.steps // 2), max(2, args.warmup // 2))
+                others[key] = {"workload": r["workload"], "ms": round(r["ms"], 4), "achieved": round(r["achieved"], 2), "unit": r["unit"],
+                               "bound": r["bound"], "frac": round(r["frac"], 4)}
+            finally:
+                for attr in list(vars(w)):
+                    if attr not in ("name", "work"):
+                        setattr(w, attr, None)
+                torch.cuda.empty_cache()
+
+    line = {
+        "metric": METRIC,
+        "value": round(res["achieved"], 3),
+        "unit": res["unit"],
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(res["ms"], 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "mxfp4 (e2m1 codes, e8m0 scales), fp32 accumulate" if res["bound"] == "mfma" else "bf16 -> e2m1/e8m0 (u8 bit ops, fp32 transform)",
+        "data": "synthetic",
+        "config": {"workload": res["workload"], "device": props.name, "cus": props.multi_processor_count,
+                   "clock_mhz": props.clock_rate // 1000 if hasattr(props, "clock_rate") else None},
+        "roofline": {"bound": res["bound"], "achieved": round(res["achieved"], 3), "peak": res["peak"], "unit": res["unit"],
+                     "frac": round(res["frac"], 4), "traffic": None, "kernel": res["kernel"], "kernel_ms": round(res["ms"], 5)},
+        "cpu_baseline": cpu,
+        "others": others,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()
