@@ -1,4 +1,4 @@
-// Tuned LDS-tiled MXFP4 GEMM for gfx950: dense entry (one 256x256 tile per workgroup, XCD-aware tile order).
+// Tuned LDS-tiled MXFP4 GEMM for gfx950: dense entry (one 256x256 tile per 512-thread workgroup, XCD-aware tile order).
 #include "gemm_tiled.h"
 #include "gemm_tile.h"
 
@@ -25,7 +25,7 @@ __device__ __forceinline__ bool tile_coords(int wg, int tiles_m, int tiles_n, in
 }
 
 template <typename OutT, bool KTAIL>
-__global__ __launch_bounds__(256) void gemm_tiled_kernel(OperandView A, OperandView B, int64_t M, int64_t N, int G,
+__global__ __launch_bounds__(GT_THREADS) void gemm_tiled_kernel(OperandView A, OperandView B, int64_t M, int64_t N, int G,
                                                          OutT* c, int64_t ldc, float out_scale, int tiles_m, int tiles_n) {
   extern __shared__ __align__(16) uint8_t smem[];
   int tm, tn;
@@ -47,7 +47,7 @@ int launch_tiled(const OperandView& A, const OperandView& B, int64_t M, int64_t 
   const int tiles_m = (int)((M + GT_TM - 1) / GT_TM), tiles_n = (int)((N + GT_TN - 1) / GT_TN);
   const int T = tiles_m * tiles_n;
   const int per_xcd = (T + 7) / 8;
-  hipLaunchKernelGGL(kern, dim3((unsigned)(per_xcd * 8)), dim3(256), GT_LDS_BYTES, st, A, B, M, N, (int)(K / 32), (OutT*)c, ldc, out_scale, tiles_m, tiles_n);
+  hipLaunchKernelGGL(kern, dim3((unsigned)(per_xcd * 8)), dim3(GT_THREADS), GT_LDS_BYTES, st, A, B, M, N, (int)(K / 32), (OutT*)c, ldc, out_scale, tiles_m, tiles_n);
   return 0;
 }
 
@@ -57,11 +57,11 @@ bool gemm_tiled_supported(const OperandView& A, const OperandView& B, int64_t M,
   (void)c_dtype;
   // small problems do not fill 256x256 tiles; the direct kernel handles them
   if (M < 128 || N < 128 || K < 128) return false;
-  // the tile kernel reads scale rows with unit stride along K and stores C in aligned groups of 4 columns
+  // the tile kernel reads scale rows with unit stride along K and stores C in aligned 16-byte groups
   if (A.ss_k != 1 || B.ss_k != 1) return false;
   if (M * A.ld >= (1ll << 31) || N * B.ld >= (1ll << 31)) return false;   // 32-bit buffer offsets
   if (M * A.ss_r >= (1ll << 31) || N * B.ss_r >= (1ll << 31)) return false;
-  if (N % 4 != 0 || ldc % 4 != 0 || (reinterpret_cast<uintptr_t>(c) & 15) != 0) return false;
+  if (N % 8 != 0 || ldc % 8 != 0 || (reinterpret_cast<uintptr_t>(c) & 15) != 0) return false;
   const int64_t tiles = ((M + GT_TM - 1) / GT_TM) * ((N + GT_TN - 1) / GT_TN);
   return tiles < (1ll << 28);
 }
