@@ -39,12 +39,25 @@ struct TileArgs {
   int64_t as_bytes, bs_bytes;  // extent of the scale buffers in bytes (< 2^31)
 };
 
-// One 256x256 tile.  KTAIL = false requires G % 4 == 0 (K a multiple of 128): then every scale dword of a row is
-// either fully inside K or fully beyond it and the main loop is branch-free.  KTAIL = true additionally handles a last
-// partial dword of a scale row with byte loads.  Requirements checked by the host: unit-stride scale rows, N % 8 == 0,
-// ldc % 8 == 0, 16-byte aligned c, operand extents below 2^31 bytes.
-template <typename OutT, bool KTAIL>
-__device__ __forceinline__ void gemm_tile_256x256(const TileArgs& ta, OutT* __restrict__ c, int64_t ldc, uint8_t* smem) {
+typedef v16f_t TileAcc[4][2];   // per wave: 4 (M) x 2 (N) MFMA tiles of 32x32
+
+__device__ __forceinline__ void gemm_tile_zero(TileAcc& acc) {
+#pragma unroll
+  for (int t = 0; t < 4; ++t)
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[t][u][v] = 0.0f;
+}
+
+// K loop of one 256x256 tile: acc += A[m0.., :] . B[n0.., :]^T over G groups of 32.  KTAIL = false requires G % 4 == 0
+// (K a multiple of 128): then every scale dword of a row is either fully inside K or fully beyond it and the main loop
+// is branch-free.  KTAIL = true additionally handles a last partial dword of a scale row with byte loads.  Requirements
+// checked by the host: unit-stride scale rows, operand extents below 2^31 bytes.  Every thread of the workgroup must
+// call it; it may be called again (same or other operands) to keep accumulating.
+template <bool KTAIL>
+__device__ __forceinline__ void gemm_tile_mainloop(const TileArgs& ta, TileAcc& acc, uint8_t* smem) {
+  __syncthreads();   // the LDS ring may still be read by a previous call
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;   // the wave index lives in a scalar register
   const int wm = wave >> 2, wn = wave & 3;
@@ -114,14 +127,6 @@ __device__ __forceinline__ void gemm_tile_256x256(const TileArgs& ta, OutT* __re
     }
   }
   uint32_t sreg[4];
-
-  v16f_t acc[4][2];
-#pragma unroll
-  for (int t = 0; t < 4; ++t)
-#pragma unroll
-    for (int u = 0; u < 2; ++u)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) acc[t][u][v] = 0.0f;
 
   // Direct-to-LDS load of stage s into ring slot `slot`: lane l of instruction i lands at chunk base + 16 l.
   typedef __attribute__((address_space(3))) uint8_t lds_u8;
@@ -268,9 +273,18 @@ __device__ __forceinline__ void gemm_tile_256x256(const TileArgs& ta, OutT* __re
   }
   // loads of the (zero-filled) stages past the end may still be landing in the ring the epilogue reuses
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+}
 
-  // ---- epilogue: accumulator register v of tile (t, u) is C[m][n] with
-  //   m = m0 + 128 wm + 32 t + r,  n = n0 + 64 wn + 32 u + 8 (v / 4) + 4 h + v % 4
+// Stores the tile: accumulator register v of MFMA tile (t, u) is C[m][n] with
+//   m = m0 + 128 wm + 32 t + r,  n = n0 + 64 wn + 32 u + 8 (v / 4) + 4 h + v % 4.
+// Rows outside [m_lo, m_hi) and columns at or beyond n_hi are not written.  Host-checked: N % 8 == 0, ldc % 8 == 0,
+// 16-byte aligned c.
+template <typename OutT>
+__device__ __forceinline__ void gemm_tile_store(const TileArgs& ta, TileAcc& acc, OutT* __restrict__ c, int64_t ldc, uint8_t* smem) {
+  const int tid = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+  const int wm = wave >> 2, wn = wave & 3;
+  const int r = lane & 31, h = lane >> 5;
   if constexpr (sizeof(OutT) == 2) {
     // bf16: the 256x256 tile (128 KB) is assembled in LDS as rows of 32 16-byte chunks, chunk index XORed with row % 32
     // (conflict-free for the 8-byte writes of 32 different rows and for the row-wise 16-byte reads), then stored as
@@ -319,6 +333,14 @@ __device__ __forceinline__ void gemm_tile_256x256(const TileArgs& ta, OutT* __re
       }
     }
   }
+}
+
+template <typename OutT, bool KTAIL>
+__device__ __forceinline__ void gemm_tile_256x256(const TileArgs& ta, OutT* __restrict__ c, int64_t ldc, uint8_t* smem) {
+  TileAcc acc;
+  gemm_tile_zero(acc);
+  gemm_tile_mainloop<KTAIL>(ta, acc, smem);
+  gemm_tile_store<OutT>(ta, acc, c, ldc, smem);
 }
 
 }  // namespace alto

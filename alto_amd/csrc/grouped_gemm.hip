@@ -1,6 +1,7 @@
 // Ragged grouped MXFP4 GEMMs for MoE experts (gfx950): forward / dX (rows grouped by expert) and dW (reduction grouped by expert).
 #include "common.h"
 #include "gemm_simple.h"
+#include "gemm_tile.h"
 
 namespace alto {
 namespace {
@@ -105,6 +106,233 @@ __global__ __launch_bounds__(256) void grouped_dw_simple_kernel(OperandView GO, 
   }
 }
 
+// ----------------------------------------------------------------------------- 256x256 tiles (large problems)
+__device__ __forceinline__ int clamp_off(const int32_t* offs, int g, int64_t M_total) {
+  const int64_t v = offs[g];
+  return (int)(v < 0 ? 0 : (v > M_total ? M_total : v));
+}
+
+// Same XCD-aware tile order as the dense kernel: an XCD works on 8 neighbouring N-tiles of one band of rows at a time.
+__device__ __forceinline__ bool grouped_tile_coords(int wg, int tiles_m, int tiles_n, int& tm, int& tn) {
+  const int T = tiles_m * tiles_n;
+  const int per_xcd = (T + 7) / 8;
+  const int u = (wg & 7) * per_xcd + (wg >> 3);
+  if ((wg >> 3) >= per_xcd || u >= T) return false;
+  const int GN = 8;
+  const int in_group = GN * tiles_m;
+  const int group = u / in_group;
+  const int first_n = group * GN;
+  const int gsize = (tiles_n - first_n) < GN ? (tiles_n - first_n) : GN;
+  const int w = u % in_group;
+  tn = first_n + w % gsize;
+  tm = w / gsize;
+  return true;
+}
+
+template <typename OutT>
+__device__ __forceinline__ void zero_rows(OutT* out, int64_t ldo, int64_t r0, int64_t r1, int64_t n0, int64_t n1) {
+  constexpr int PER = 16 / sizeof(OutT);
+  const int chunks = (int)((n1 - n0) / PER);   // N % 8 == 0 and n0 % 256 == 0: whole 16-byte chunks
+  const int64_t total = (r1 - r0) * chunks;
+  for (int64_t i = threadIdx.x; i < total; i += GT_THREADS) {
+    const int64_t row = r0 + i / chunks;
+    const int ch = (int)(i % chunks);
+    *reinterpret_cast<uint4*>(out + row * ldo + n0 + (int64_t)ch * PER) = make_uint4(0, 0, 0, 0);
+  }
+}
+
+// The tile as a real function: inlined into the segment loop below, its address set-up competes with the loop's own
+// state for registers and spills.
+template <typename OutT, bool KTAIL>
+__device__ __noinline__ void grouped_tile_call(const TileArgs& ta, OutT* out, int64_t ldo) {
+  extern __shared__ __align__(16) uint8_t smem[];
+  gemm_tile_256x256<OutT, KTAIL>(ta, out, ldo, smem);
+}
+
+// One workgroup owns rows [256 tm, 256 tm + 256) x columns [256 tn, 256 tn + 256) of the output.  The rows are cut
+// into segments of one expert each (adjacent groups of the same expert merge); every segment is one pass of the tile
+// with its rows masked, rows that belong to no group or to an invalid expert are zero-filled.
+template <typename OutT, bool KTAIL>
+__global__ __launch_bounds__(GT_THREADS) void grouped_tiled_kernel(OperandView A, const uint8_t* w, int64_t w_stride_e, int64_t ldw,
+                                                                   const uint8_t* w_scales, int64_t ws_stride_e, int64_t ws_r, int w_is_2d,
+                                                                   const int32_t* offs, const int32_t* group_expert, int num_groups, int num_experts,
+                                                                   int64_t M_total, int64_t N, int G, OutT* out, int64_t ldo, int tiles_m, int tiles_n) {
+  extern __shared__ __align__(16) uint8_t smem[];
+  int tm, tn;
+  if (!grouped_tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn)) return;
+  const int n0 = tn * GT_TN;
+  const int n1 = n0 + GT_TN < (int)N ? n0 + GT_TN : (int)N;
+  const int Mt = (int)M_total;   // the host checks M_total < 2^31
+  const int row0 = tm * GT_TM;
+  const int row1 = row0 + GT_TM < Mt ? row0 + GT_TM : Mt;
+  // first group that ends after row0 (binary search over the group ends)
+  int lo = 0, hi = num_groups;
+  while (lo < hi) {
+    const int mid = (lo + hi) >> 1;
+    if (clamp_off(offs, mid + 1, M_total) > row0) hi = mid; else lo = mid + 1;
+  }
+  int g = lo;
+  int cur = row0;
+  while (cur < row1) {
+    // next segment [cur, seg_end): expert e, or -1 for rows to zero-fill
+    int e = -1, seg_end = row1;
+    while (g < num_groups && clamp_off(offs, g + 1, M_total) <= cur) ++g;
+    if (g < num_groups) {
+      const int start = clamp_off(offs, g, M_total);
+      if (start > cur) {   // rows before the next group
+        seg_end = start < row1 ? start : row1;
+      } else {
+        e = group_expert ? group_expert[g] : g;
+        int end = clamp_off(offs, g + 1, M_total);
+        while (end < row1 && g + 1 < num_groups && (group_expert ? group_expert[g + 1] : g + 1) == e) {
+          ++g;
+          const int e2 = clamp_off(offs, g + 1, M_total);
+          end = e2 > end ? e2 : end;
+        }
+        seg_end = end < row1 ? end : row1;
+        ++g;
+        if (e >= num_experts) e = -1;
+      }
+    }
+    if (e < 0) {
+      zero_rows<OutT>(out, ldo, cur, seg_end, n0, n1);
+    } else {
+      OperandView B{w + e * w_stride_e, ldw, w_scales + e * ws_stride_e, ws_r, 1, w_is_2d};
+      TileArgs ta{A, B, row0, n0, cur, seg_end, N, G, 1.0f,
+                  (M_total - 1) * A.ld + G * 16, (N - 1) * ldw + G * 16,
+                  ((A.is_2d ? M_total / 32 : M_total) - 1) * A.ss_r + G, ((w_is_2d ? N / 32 : N) - 1) * ws_r + G};
+      grouped_tile_call<OutT, KTAIL>(ta, out, ldo);
+      __syncthreads();   // the next segment reuses the LDS the store staged through
+    }
+    cur = seg_end;
+  }
+}
+
+// dW[e] tile: rows [256 tm, +256) of the first operand (P) x rows [256 tn, +256) of the second (Q), reduced over the
+// token ranges of expert e.  With per-group expert ids, the runs of adjacent groups of this expert are found with one
+// ballot per 64 groups (bit masks kept in LDS behind the tile's own buffers); every run is one pass of the K loop into
+// the same accumulators, in increasing token order.
+constexpr int GT_DW_MAX_GROUPS = 32768;
+constexpr int GT_DW_LDS_BYTES = GT_LDS_BYTES + 2 * (GT_DW_MAX_GROUPS / 64) * 8;   // + 8 KB of masks
+
+template <typename OutT>
+__global__ __launch_bounds__(GT_THREADS) void grouped_dw_tiled_kernel(OperandView P, OperandView Q, int64_t NP, int64_t NQ,
+                                                                      const int32_t* offs, const int32_t* group_expert, int num_groups,
+                                                                      int64_t M_total, OutT* dw, int64_t s_e, int64_t ld, float out_scale,
+                                                                      int tiles_p, int tiles_q) {
+  extern __shared__ __align__(16) uint8_t smem[];
+  const int e = blockIdx.y;
+  int tm, tn;
+  if (!grouped_tile_coords(blockIdx.x, tiles_p, tiles_q, tm, tn)) return;
+  TileAcc acc;
+  gemm_tile_zero(acc);
+  const int64_t p_bytes = (NP - 1) * P.ld + M_total / 2, q_bytes = (NQ - 1) * Q.ld + M_total / 2;
+  const int64_t ps_bytes = (NP - 1) * P.ss_r + M_total / 32, qs_bytes = (NQ - 1) * Q.ss_r + M_total / 32;
+  auto tok = [&](int g) { return (int64_t)(clamp_off(offs, g, M_total) & ~31); };
+  uint64_t* mstart = reinterpret_cast<uint64_t*>(smem + GT_LDS_BYTES);
+  uint64_t* mend = mstart + GT_DW_MAX_GROUPS / 64;
+  const int words = group_expert ? (num_groups + 63) >> 6 : 0;
+  for (int base = 0; base < words * 64; base += GT_THREADS) {
+    const int gi = base + (int)threadIdx.x;
+    bool first = false, last = false;
+    if (gi < num_groups && group_expert[gi] == e) {
+      first = gi == 0 || group_expert[gi - 1] != e;
+      last = gi == num_groups - 1 || group_expert[gi + 1] != e;
+    }
+    const uint64_t bs = __ballot(first), be = __ballot(last);
+    if ((threadIdx.x & 63) == 0 && (gi >> 6) < words) {
+      mstart[gi >> 6] = bs;
+      mend[gi >> 6] = be;
+    }
+  }
+  __syncthreads();
+  auto word = [&](const uint64_t* p, int i) {   // same LDS word for every lane -> scalar registers
+    const uint64_t v = p[i];
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return ((uint64_t)hi << 32) | lo;
+  };
+  int wi = -1;           // current mask word; -1: not started
+  uint64_t ms = 0, me = 0;
+  int64_t t0 = 0, t1 = 0;
+  bool direct_done = false;
+  while (true) {
+    // next run [t0, t1) of this expert's tokens
+    bool have = false;
+    if (group_expert == nullptr) {
+      if (!direct_done) {
+        t0 = tok(e);
+        t1 = tok(e + 1);
+        direct_done = true;
+        have = true;
+      }
+    } else {
+      while (true) {
+        if (ms == 0 && me == 0) {
+          if (++wi >= words) break;
+          ms = word(mstart, wi);
+          me = word(mend, wi);
+          continue;
+        }
+        const int bs = ms ? __builtin_ctzll(ms) : 64, be = me ? __builtin_ctzll(me) : 64;
+        if (bs <= be) {   // a run starts at this group; its end is this bit or a later one
+          t0 = tok(wi * 64 + bs);
+          ms &= ms - 1;
+        } else {
+          t1 = tok(wi * 64 + be + 1);
+          me &= me - 1;
+          have = true;
+          break;
+        }
+      }
+    }
+    if (!have) break;
+    if (t1 <= t0) continue;
+    OperandView Pv = P, Qv = Q;
+    Pv.codes += t0 / 2;
+    Qv.codes += t0 / 2;
+    Pv.scales += t0 / 32;
+    Qv.scales += t0 / 32;
+    TileArgs ta{Pv, Qv, (int64_t)tm * GT_TM, (int64_t)tn * GT_TN, 0, NP, NQ, (int)((t1 - t0) / 32), out_scale,
+                p_bytes - t0 / 2, q_bytes - t0 / 2, ps_bytes - t0 / 32, qs_bytes - t0 / 32};
+    gemm_tile_mainloop<true>(ta, acc, smem);
+  }
+  TileArgs ta{P, Q, (int64_t)tm * GT_TM, (int64_t)tn * GT_TN, 0, NP, NQ, 0, out_scale, 0, 0, 0, 0};
+  gemm_tile_store<OutT>(ta, acc, dw + e * s_e, ld, smem);
+}
+
+template <typename OutT, bool KTAIL>
+int launch_grouped_tiled(const OperandView& A, const uint8_t* w, int64_t w_stride_e, int64_t ldw, const uint8_t* w_scales, int64_t ws_stride_e,
+                         int64_t ws_r, int w_is_2d, const int32_t* offs, const int32_t* group_expert, int num_groups, int num_experts,
+                         int64_t M_total, int64_t N, int64_t K, void* out, int64_t ldo, hipStream_t st) {
+  static bool attr_set = false;  // the opt-in for > 64 KB of dynamic LDS is per function, set once per process
+  auto kern = grouped_tiled_kernel<OutT, KTAIL>;
+  if (!attr_set) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, GT_LDS_BYTES) != hipSuccess) return -1;
+    attr_set = true;
+  }
+  const int tiles_m = (int)((M_total + GT_TM - 1) / GT_TM), tiles_n = (int)((N + GT_TN - 1) / GT_TN);
+  const int per_xcd = (tiles_m * tiles_n + 7) / 8;
+  hipLaunchKernelGGL(kern, dim3((unsigned)(per_xcd * 8)), dim3(GT_THREADS), GT_LDS_BYTES, st, A, w, w_stride_e, ldw, w_scales, ws_stride_e, ws_r,
+                     w_is_2d, offs, group_expert, num_groups, num_experts, M_total, N, (int)(K / 32), (OutT*)out, ldo, tiles_m, tiles_n);
+  return 0;
+}
+
+template <typename OutT>
+int launch_dw_tiled(const OperandView& P, const OperandView& Q, int64_t NP, int64_t NQ, const int32_t* offs, const int32_t* group_expert,
+                    int num_groups, int num_experts, int64_t M_total, void* dw, int64_t s_e, int64_t ld, float out_scale, hipStream_t st) {
+  static bool attr_set = false;
+  auto kern = grouped_dw_tiled_kernel<OutT>;
+  if (!attr_set) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, GT_DW_LDS_BYTES) != hipSuccess) return -1;
+    attr_set = true;
+  }
+  const int tiles_p = (int)((NP + GT_TM - 1) / GT_TM), tiles_q = (int)((NQ + GT_TN - 1) / GT_TN);
+  const int per_xcd = (tiles_p * tiles_q + 7) / 8;
+  hipLaunchKernelGGL(kern, dim3((unsigned)(per_xcd * 8), (unsigned)num_experts), dim3(GT_THREADS), GT_DW_LDS_BYTES, st, P, Q, NP, NQ, offs,
+                     group_expert, num_groups, M_total, (OutT*)dw, s_e, ld, out_scale, tiles_p, tiles_q);
+  return 0;
+}
+
 }  // namespace
 }  // namespace alto
 
@@ -129,6 +357,27 @@ extern "C" int alto_mxfp4_grouped_gemm(const uint8_t* a, int64_t lda, const uint
   if (M_total == 0 || N == 0) return ALTO_MXFP4_OK;
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   OperandView A{a, lda, a_scales, a_ss_r, a_ss_k, a_is_2d};
+  // 256x256 tiles when the problem fills them and the layouts fit their loads (unit-stride scale rows, 32-bit buffer
+  // offsets, 16-byte output chunks); otherwise the direct kernel below
+  const bool tiled = M_total >= 128 && N >= 128 && K >= 128 && a_ss_k == 1 && ws_k == 1 && N % 8 == 0 && ldo % 8 == 0 &&
+                     (reinterpret_cast<uintptr_t>(out) & 15) == 0 && M_total * lda < (1ll << 31) && N * ldw < (1ll << 31) &&
+                     M_total * a_ss_r < (1ll << 31) && N * ws_r < (1ll << 31) &&
+                     ((M_total + GT_TM - 1) / GT_TM) * ((N + GT_TN - 1) / GT_TN) < (1ll << 28);
+  if (tiled) {
+    const bool tail = (K / 32) % 4 != 0;
+    int rc;
+    if (out_dtype == ALTO_DT_BF16)
+      rc = tail ? launch_grouped_tiled<__bf16, true>(A, w, w_stride_e, ldw, w_scales, ws_stride_e, ws_r, w_is_2d, offs, group_expert, num_groups, num_experts, M_total, N, K, out, ldo, st)
+                : launch_grouped_tiled<__bf16, false>(A, w, w_stride_e, ldw, w_scales, ws_stride_e, ws_r, w_is_2d, offs, group_expert, num_groups, num_experts, M_total, N, K, out, ldo, st);
+    else
+      rc = tail ? launch_grouped_tiled<float, true>(A, w, w_stride_e, ldw, w_scales, ws_stride_e, ws_r, w_is_2d, offs, group_expert, num_groups, num_experts, M_total, N, K, out, ldo, st)
+                : launch_grouped_tiled<float, false>(A, w, w_stride_e, ldw, w_scales, ws_stride_e, ws_r, w_is_2d, offs, group_expert, num_groups, num_experts, M_total, N, K, out, ldo, st);
+    if (rc != 0) {
+      set_error("grouped_gemm: could not reserve %d bytes of LDS", GT_LDS_BYTES);
+      return ALTO_MXFP4_ELAUNCH;
+    }
+    return check_launch("grouped_gemm");
+  }
   // upper bound on row tiles: every expert (and the zero tail) may end with one partial tile
   const int64_t tiles = M_total / 64 + num_groups + 2;
   ALTO_REQUIRE(tiles <= 65535, "grouped_gemm: M_total too large for the fallback kernel");
@@ -161,6 +410,29 @@ extern "C" int alto_mxfp4_grouped_gemm_dw(const uint8_t* go, int64_t ld_go, cons
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   OperandView GO{go, ld_go, go_scales, gs_r, gs_k, 0};
   OperandView X{x, ld_xq, x_scales, xs_r, xs_k, 0};
+  {
+    // 256x256 tiles: the output's unit-stride dim becomes the GEMM's column dim, so the operands swap roles for dW stored [E, K, N]
+    const bool n_major = dw_stride_k == 1;   // dW[e] is [N][K]
+    const OperandView& P = n_major ? GO : X;
+    const OperandView& Q = n_major ? X : GO;
+    const int64_t NP = n_major ? N : K, NQ = n_major ? K : N;
+    const int64_t ld = n_major ? dw_stride_n : dw_stride_k;
+    const bool unit = n_major || dw_stride_n == 1;
+    const bool tiled = unit && M_total >= 128 && N >= 128 && K >= 128 && gs_k == 1 && xs_k == 1 && NQ % 8 == 0 && ld % 8 == 0 && dw_stride_e % 8 == 0 &&
+                       (reinterpret_cast<uintptr_t>(dw) & 15) == 0 && N * ld_go < (1ll << 31) && K * ld_xq < (1ll << 31) &&
+                       N * gs_r < (1ll << 31) && K * xs_r < (1ll << 31) && num_groups <= GT_DW_MAX_GROUPS && num_experts <= 65535 &&
+                       ((NP + GT_TM - 1) / GT_TM) * ((NQ + GT_TN - 1) / GT_TN) < (1ll << 28);
+    if (tiled) {
+      const int rc = dw_dtype == ALTO_DT_BF16
+                         ? launch_dw_tiled<__bf16>(P, Q, NP, NQ, offs, group_expert, num_groups, num_experts, M_total, dw, dw_stride_e, ld, out_scale, st)
+                         : launch_dw_tiled<float>(P, Q, NP, NQ, offs, group_expert, num_groups, num_experts, M_total, dw, dw_stride_e, ld, out_scale, st);
+      if (rc != 0) {
+        set_error("grouped_gemm_dw: could not reserve %d bytes of LDS", GT_DW_LDS_BYTES);
+        return ALTO_MXFP4_ELAUNCH;
+      }
+      return check_launch("grouped_gemm_dw");
+    }
+  }
   dim3 grid((unsigned)((K + 63) / 64), (unsigned)((N + 63) / 64), (unsigned)num_experts);
   ALTO_REQUIRE(grid.y <= 65535u, "grouped_gemm_dw: N too large");
   if (dw_dtype == ALTO_DT_BF16)

@@ -183,12 +183,11 @@ class MXFP4GroupedGEMM(torch.autograd.Function):
         # weights: one pass gives the K-packed codes (forward) and the N-packed codes (dX)
         w = expert_weights if trans_weights else expert_weights.transpose(1, 2)   # logical [E, N, K]
         if w.stride(2) == 1:
-            wq_nk, ws_nk, wq_kn = _quantize_experts(w, use_uos)                   # [E,N,K/2], [E,N/32,K/32], [E,K,N/2]
+            wq_nk, ws_nk, wq_kn, ws_kn = _quantize_experts(w, use_uos)            # [E,N,K/2], [E,N/32,K/32], [E,K,N/2], [E,K/32,N/32]
         else:                                                                     # stored [E, K, N]: same pass, roles swapped
-            wq_kn, ws_kn, wq_nk = _quantize_experts(w.transpose(1, 2), use_uos)
-            ws_nk = ws_kn.transpose(1, 2)
+            wq_kn, ws_kn, wq_nk, ws_nk = _quantize_experts(w.transpose(1, 2), use_uos)
         out = grouped_forward(a_q, a_s, wq_nk, ws_nk, groups, False, True, original_dtype)
-        ctx.save_for_backward(a_qm, a_sm, wq_kn, ws_nk, groups.offs, groups.expert)
+        ctx.save_for_backward(a_qm, a_sm, wq_kn, ws_kn, groups.offs, groups.expert)
         ctx.num_groups = groups.n
         ctx.trans_weights = trans_weights
         ctx.original_dtype = original_dtype
@@ -201,14 +200,14 @@ class MXFP4GroupedGEMM(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, grad_output):
-        a_qm, a_sm, wq_kn, ws_nk, g_offs, g_expert = ctx.saved_tensors
+        a_qm, a_sm, wq_kn, ws_kn, g_offs, g_expert = ctx.saved_tensors
         groups = Groups(g_offs, g_expert, ctx.num_groups)
         go = grad_output if grad_output.is_contiguous() else grad_output.contiguous()
         sr = bool(ctx.use_sr_grad)
         rand = rt.draw_rand_bits(go.shape, go.device) if sr else None
         go_q, go_s, go_qm, go_sm = quantize_rowcol(go, False, use_sr=sr, rand_bits=rand, hadamard=ctx.hadamard_transform,
                                                    clip_mode=ctx.clip_mode, use_uos=ctx.use_uos)
-        grad_inputs = grouped_forward(go_q, go_s, wq_kn, ws_nk.transpose(1, 2), groups, False, True, ctx.original_dtype)
+        grad_inputs = grouped_forward(go_q, go_s, wq_kn, ws_kn, groups, False, True, ctx.original_dtype)
         grad_weights = grouped_dw(go_qm.transpose(0, 1), go_sm.transpose(0, 1), a_qm.transpose(0, 1), a_sm.transpose(0, 1),
                                   groups, ctx.num_experts, ctx.original_dtype, ctx.trans_weights,
                                   16.0 / 9.0 if ctx.clip_mode == "static" else 1.0)
@@ -216,12 +215,12 @@ class MXFP4GroupedGEMM(torch.autograd.Function):
 
 
 def _quantize_experts(w: torch.Tensor, use_uos: bool):
-    """w [E, R, C] (unit stride along C) -> (codes packed along C [E,R,C/2], 2D scales [E,R/32,C/32], codes packed along R [E,C,R/2])."""
+    """w [E, R, C] (unit stride along C) -> codes packed along C [E,R,C/2], 2D scales [E,R/32,C/32], codes packed along R
+    [E,C,R/2] and the same scales stored transposed [E,C/32,R/32] (each operand of a GEMM wants unit stride along its K)."""
     from .quantization import _prep, _quantize_call
     E, R, C = w.shape
     w3 = _prep(w)
-    rc, rs, cc, _ = _quantize_call(w3, True, True, True, False, None, None, 0, use_uos)
-    return rc, rs, cc
+    return _quantize_call(w3, True, True, True, False, None, None, 0, use_uos)
 
 
 def mxfp4_grouped_gemm(inputs, expert_weights, expert_indices, *, trans_weights=True, use_2dblock_x=False, use_2dblock_w=True,

@@ -148,8 +148,10 @@ class MXFP4LinearFunction(torch.autograd.Function):
                 x_qm, x_sm = convert_to_mxfp4(x2, axis=0, clip_mode=clip_mode, use_uos=use_uos, hadamard=hadamard_transform)
 
         if use_2dblock_w:
-            w_q, w_s, w_qt, _ = quantize_rowcol(weight, True, use_uos=use_uos)
-            w_bwd, w_bwd_s = w_qt, w_s            # [N/2, K] view over [K][N/2] memory, scales [N/32, K/32]
+            w_q, w_s, w_qt, w_st = quantize_rowcol(weight, True, use_uos=use_uos)
+            # [N/2, K] view over [K][N/2] memory; scales [N/32, K/32] as a view over [K/32][N/32] memory (same values as
+            # w_s, stored so that the dgrad GEMM reads them with unit stride along its reduction dim N)
+            w_bwd, w_bwd_s = w_qt, w_st
         else:
             w_q, w_s = convert_to_mxfp4(weight, axis=-1, is_2d_block=False, use_uos=use_uos)
             w_bwd, w_bwd_s = convert_to_mxfp4(weight, axis=0, is_2d_block=False, use_uos=use_uos)

@@ -240,3 +240,50 @@ def test_grouped_unaligned_rows_forward(m):
     ref = O.grouped_gemm_ref(aq, as_, wq, ws, idx)
     assert O.rel_frobenius(out.cpu(), ref) < 1e-5
     assert bool((out[201:] == 0).all())
+
+
+def test_grouped_small_problem_direct_kernels(m):
+    """Shapes below one 256x256 tile run on the direct (untiled) grouped kernels: forward, dX and dW."""
+    E, N, K = 3, 96, 64
+    sizes = [32, 64, 32]
+    ends = torch.tensor(sizes).cumsum(0).to(torch.int32)
+    M_buf = int(ends[-1])
+    a, w = _grouped_inputs(M_buf, N, K, E, seed=70)
+    go = randn_outliers((M_buf, N), torch.bfloat16, seed=72) / (M_buf * N)
+    ag = a.to(DEV).requires_grad_(True)
+    wg = w.transpose(1, 2).contiguous().to(DEV).requires_grad_(True)
+    out = m._quantize_then_mxfp_scaled_grouped_mm(ag, wg, ends.to(DEV), False, True, False, False, False, "none", False)
+    out.backward(go.to(DEV))
+    idx = O.indices_from_offsets(ends)
+    aq, as_ = O.quantize(a)
+    wq, ws = O.quantize(w, axis=-1, is_2d_block=True)
+    assert O.rel_frobenius(out.detach().cpu(), O.grouped_gemm_ref(aq, as_, wq, ws, idx)) < 4e-3
+    gq, gs = O.quantize(go)
+    assert O.rel_frobenius(ag.grad.cpu(), O.grouped_gemm_dx_ref(gq, gs, wq, ws, idx, k_pack_w=False)) < 4e-3
+    gqm, gsm = O.quantize(go, axis=0)
+    aqm, asm = O.quantize(a, axis=0)
+    assert O.rel_frobenius(wg.grad.cpu(), O.grouped_gemm_dw_ref(gqm, gsm, aqm, asm, idx, E, trans_weights=False)) < 4e-3
+
+
+def test_grouped_many_groups_sorted_runs(m):
+    """2048 rows in 16 groups of 128 whose experts come in runs (sorted routing): adjacent groups of one expert merge
+    into one pass per tile in forward/dX and into one reduction range in dW; expert 2 owns two separate runs."""
+    M_total, N, K, E = 2048, 384, 640, 4
+    a, w = _grouped_inputs(M_total, N, K, E, seed=80)
+    experts = torch.tensor([0, 0, 0, 2, 2, 1, 1, 1, 1, 1, 2, 2, 2, 0, 1, 1], dtype=torch.int32)   # expert 3 unused
+    idx = experts.repeat_interleave(128)
+    go = randn_outliers((M_total, N), torch.bfloat16, seed=82) / (M_total * N)
+    ag = a.to(DEV).requires_grad_(True)
+    wg = w.to(DEV).requires_grad_(True)
+    out = m.mxfp4_grouped_gemm(ag, wg, idx.to(DEV), trans_weights=True)
+    out.backward(go.to(DEV))
+    aq, as_ = O.quantize(a)
+    wq, ws = O.quantize(w, axis=-1, is_2d_block=True)
+    assert O.rel_frobenius(out.detach().cpu(), O.grouped_gemm_ref(aq, as_, wq, ws, idx)) < 4e-3
+    gq, gs = O.quantize(go)
+    assert O.rel_frobenius(ag.grad.cpu(), O.grouped_gemm_dx_ref(gq, gs, wq, ws, idx, k_pack_w=False)) < 4e-3
+    gqm, gsm = O.quantize(go, axis=0)
+    aqm, asm = O.quantize(a, axis=0)
+    dw_ref = O.grouped_gemm_dw_ref(gqm, gsm, aqm, asm, idx, E, trans_weights=True)
+    assert O.rel_frobenius(wg.grad.cpu(), dw_ref) < 4e-3
+    assert bool((wg.grad[3] == 0).all())
