@@ -88,8 +88,20 @@ class FusedGradQuant(Workload):
         # algorithmic bytes: dY + random bits in, two code tensors + two scale tensors out
         self.work = self.M * self.C * 2 + self.M * self.C * 4 + 2 * (self.M * self.C // 2 + self.M * self.C // 32)
 
+        # outputs allocated once: a step is one launch through the C ABI, as a caller that owns its buffers makes it
+        from alto_amd.mxfp4 import _runtime as rt
+        M, C = self.M, self.C
+        u8 = dict(dtype=torch.uint8, device=dev)
+        self.out = (torch.empty((M, C // 2), **u8), torch.empty((M, C // 32), **u8), torch.empty((C, M // 2), **u8), torch.empty((C, M // 32), **u8))
+        self.rt, self.stream = rt, rt.stream_ptr(dev)
+
     def step(self):
-        return self.m.quantize_rowcol(self.x, False, use_sr=True, rand_bits=self.r, hadamard=self.h)
+        rt, (rc, rs, cc, cs) = self.rt, self.out
+        code = rt.lib().alto_mxfp4_quantize(self.x.data_ptr(), rt.dtype_code(self.x.dtype), 1, self.M, self.C, self.C, self.M * self.C,
+                                            rc.data_ptr(), rs.data_ptr(), cc.data_ptr(), cs.data_ptr(), 0, rt.ROUND_SR,
+                                            self.r.data_ptr(), self.C, self.M * self.C, 1, self.h.signs.data_ptr(), self.h.perm.data_ptr(),
+                                            0, 0, self.stream)
+        assert code == 0, code
 
     def cpu_sample(self):
         import oracle as O
@@ -119,8 +131,16 @@ class RneQuant(Workload):
         self.x = torch.where(torch.rand(self.M, self.C, device=dev, generator=gen) < 0.01, x * 50, x).bfloat16()
         self.work = self.M * self.C * 2 + self.M * self.C // 2 + self.M * self.C // 32
 
+        from alto_amd.mxfp4 import _runtime as rt
+        u8 = dict(dtype=torch.uint8, device=dev)
+        self.out = (torch.empty((self.M, self.C // 2), **u8), torch.empty((self.M, self.C // 32), **u8))
+        self.rt, self.stream = rt, rt.stream_ptr(dev)
+
     def step(self):
-        return self.m.convert_to_mxfp4(self.x)
+        rt, (rc, rs) = self.rt, self.out
+        code = rt.lib().alto_mxfp4_quantize(self.x.data_ptr(), rt.dtype_code(self.x.dtype), 1, self.M, self.C, self.C, self.M * self.C,
+                                            rc.data_ptr(), rs.data_ptr(), None, None, 0, rt.ROUND_RNE, None, 0, 0, 0, None, None, 0, 0, self.stream)
+        assert code == 0, code
 
     def cpu_sample(self):
         import oracle as O
@@ -220,6 +240,38 @@ class GroupedGemm(Workload):
         return run, 2.0 * rows * self.N * self.K, f"{rows} rows of the largest expert, dequantize + fp32 matmul"
 
 
+class CopyCalibration(Workload):
+    """Plain device copy of 256 MiB (torch's elementwise copy kernel): the known-size launch against which the
+    FETCH_SIZE / WRITE_SIZE counters of the other kernels are scaled.  Not part of the product path."""
+    name = "copy_calibration[256MiB]"
+    bound = "hbm"
+    kernel = "torch elementwise copy"
+    BYTES = 256 << 20
+
+    def setup(self, dev, gen):
+        import torch
+        self.src = torch.randint(0, 255, (self.BYTES,), dtype=torch.uint8, device=dev, generator=gen).view(torch.int32)
+        self.dst = torch.empty_like(self.src)
+        self.work = 2 * self.BYTES
+
+    def step(self):
+        self.dst.copy_(self.src)
+
+    def cpu_sample(self):
+        src = self.src.cpu()
+        dst = src.clone()
+        return (lambda: dst.copy_(src)), self.work, "the same 256 MiB copy on the host"
+
+
+def load_traffic(key):
+    """HBM bytes per launch of the workload's dominant kernel, from the committed rocprofv3 counter summaries (or None)."""
+    try:
+        with open(os.path.join(ROOT, "profiles", "traffic.json")) as f:
+            return json.load(f).get(key, {}).get("hbm_bytes_per_launch")
+    except (OSError, ValueError):
+        return None
+
+
 def make_workloads():
     return {
         "cfg3_fprop": Gemm("cfg3_fprop_gemm[8192x14336x4096]", 8192, 14336, 4096, False, True, "act", "weight"),
@@ -229,6 +281,7 @@ def make_workloads():
         "cfg4_dgrad": Gemm("cfg4_dgrad_gemm[8192x14336x4096]", 8192, 14336, 4096, False, True, "grad", "weight"),
         "cfg4_wgrad": Gemm("cfg4_wgrad_gemm[4096x14336x8192]", 4096, 14336, 8192, False, False, "grad", "act"),
         "cfg5_grouped": GroupedGemm(),
+        "copy_calib": CopyCalibration(),
     }
 
 
@@ -299,7 +352,7 @@ def main():
     others = {}
     if not args.only:
         for key, w in wl.items():
-            if key == args.workload:
+            if key == args.workload or key == "copy_calib":
                 continue
             primary_mem_release = None  # noqa: F841
             try:
@@ -328,7 +381,7 @@ def main():
         "config": {"workload": res["workload"], "device": props.name, "cus": props.multi_processor_count,
                    "clock_mhz": props.clock_rate // 1000 if hasattr(props, "clock_rate") else None},
         "roofline": {"bound": res["bound"], "achieved": round(res["achieved"], 3), "peak": res["peak"], "unit": res["unit"],
-                     "frac": round(res["frac"], 4), "traffic": None, "kernel": res["kernel"], "kernel_ms": round(res["ms"], 5)},
+                     "frac": round(res["frac"], 4), "traffic": load_traffic(args.workload), "kernel": res["kernel"], "kernel_ms": round(res["ms"], 5)},
         "cpu_baseline": cpu,
         "others": others,
     }

@@ -1,0 +1,92 @@
+"""Committed vectors (tests/golden/mxfp4_vectors.npz, written by tests/golden/make_vectors.py): the oracle and the HIP
+path must both reproduce every byte.  The reference holds no stored vectors for this path; these freeze the pinned
+oracle's outputs on small inputs."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import oracle as O
+from tests.helpers import assert_bytes_equal
+
+V = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "mxfp4_vectors.npz"))
+
+
+def t(name):
+    return torch.from_numpy(V[name])
+
+
+def bf16(name):
+    return t(name).view(torch.bfloat16)
+
+
+# ----------------------------------------------------------------------------------------------- oracle (CPU)
+def test_oracle_rne_vectors():
+    q, s = O.quantize(bf16("rne_x_bf16bits"))
+    assert_bytes_equal(q, t("rne_codes"), "codes")
+    assert_bytes_equal(s, t("rne_scales"), "scales")
+    dq = O.dequantize(q, s, torch.bfloat16)
+    assert_bytes_equal(dq.view(torch.int16), t("rne_dequant_bf16bits"), "dequantised bf16 bits")
+    q, s = O.quantize(t("w2d_x_f32"), is_2d_block=True)
+    assert_bytes_equal(q, t("w2d_codes"), "2D codes")
+    assert_bytes_equal(s, t("w2d_scales"), "2D scales")
+
+
+def test_oracle_sr_rht_vectors():
+    g, r = bf16("sr_x_bf16bits"), t("sr_rand")
+    q, s = O.quantize(g, use_sr=True, rand_bits=r)
+    assert_bytes_equal(q, t("sr_row_codes"), "row codes")
+    assert_bytes_equal(s, t("sr_row_scales"), "row scales")
+    gh = O.rht_left(g, t("had_signs"), t("had_perm"))
+    assert_bytes_equal(gh.view(torch.int16), t("sr_rht_bf16bits"), "transformed bf16 bits")
+    qc, sc = O.quantize(gh, axis=0, use_sr=True, rand_bits=r)
+    assert_bytes_equal(qc.contiguous(), t("sr_col_codes"), "column codes")
+    assert_bytes_equal(sc.contiguous(), t("sr_col_scales"), "column scales")
+
+
+def test_oracle_gemm_vector():
+    c = O.gemm_ref(t("gemm_a_codes"), t("gemm_a_scales"), t("gemm_b_codes"), t("gemm_b_scales"), use_2dblock_b=True, trans_b=True)
+    assert torch.equal(c.float(), t("gemm_c_f32"))
+
+
+# ----------------------------------------------------------------------------------------------- HIP path (GPU)
+@pytest.fixture(scope="module")
+def m():
+    import alto_amd.mxfp4 as mod
+    return mod
+
+
+@pytest.mark.gpu
+def test_hip_rne_vectors(m):
+    q, s = m.convert_to_mxfp4(bf16("rne_x_bf16bits").cuda())
+    assert_bytes_equal(q, t("rne_codes"), "codes")
+    assert_bytes_equal(s, t("rne_scales"), "scales")
+    dq = m.convert_from_mxfp4(q, s, torch.bfloat16)
+    assert_bytes_equal(dq.view(torch.int16), t("rne_dequant_bf16bits"), "dequantised bf16 bits")
+    q, s = m.convert_to_mxfp4(t("w2d_x_f32").cuda(), is_2d_block=True)
+    assert_bytes_equal(q, t("w2d_codes"), "2D codes")
+    assert_bytes_equal(s, t("w2d_scales"), "2D scales")
+
+
+@pytest.mark.gpu
+def test_hip_sr_rht_vectors(m):
+    g, r = bf16("sr_x_bf16bits").cuda(), t("sr_rand").cuda()
+    h = m.HadamardTransform(t("had_signs"), t("had_perm"))
+    rq, rs, cq, cs = m.quantize_rowcol(g, False, use_sr=True, rand_bits=r, hadamard=h)
+    assert_bytes_equal(rq, t("sr_row_codes"), "row codes")
+    assert_bytes_equal(rs, t("sr_row_scales"), "row scales")
+    assert_bytes_equal(cq.contiguous(), t("sr_col_codes"), "column codes")
+    assert_bytes_equal(cs.contiguous(), t("sr_col_scales"), "column scales")
+    gh = m.hadamard_left(g, h)
+    assert_bytes_equal(gh.view(torch.int16), t("sr_rht_bf16bits"), "transformed bf16 bits")
+
+
+@pytest.mark.gpu
+def test_hip_gemm_vector(m):
+    c = m.blockwise_mxfp4_gemm(t("gemm_a_codes").cuda(), t("gemm_a_scales").cuda(), t("gemm_b_codes").cuda(), t("gemm_b_scales").cuda(),
+                               use_2dblock_b=True, trans_b=True, output_dtype=torch.float32)
+    ref = t("gemm_c_f32")
+    # products of E2M1 values are exact and these sums stay far below 2^24 ulps of their scale: fp32 accumulation in any
+    # order differs from the float64 reference by rounding only (tolerance of the GEMM parity bar: 1e-2 relative Frobenius)
+    assert O.rel_frobenius(c.cpu(), ref) < 1e-5
