@@ -2,15 +2,19 @@
 // C = A . B^T with v_mfma_scale_f32_32x32x64_f8f6f4; each wave owns 128 (M) x 64 (N) = 4 x 2 MFMA tiles (128 accumulator
 // registers), so two waves share every SIMD and cover each other's waits.
 //
-// Data path per K stage of 128 elements (64 B per operand row):
-//   global --buffer_load_dwordx4 ... lds (no register staging, two stages in flight)--> LDS ring of 4 stages (32 KB each)
-//   LDS --ds_read_b128--> MFMA operands.  (LDS instructions cost issue time on the SIMD that also issues the MFMAs -- about
-//   12 clocks per ds_read_b128 and 40 per ds_write_b128 -- so the operand tiles never pass through ds_write.)  A 16-byte piece holds one MX block (32 codes); lane (r, h) of the MFMA takes
-//   piece 2h + j of row r at K step j, so a row's four pieces are XOR-swizzled by (row / 4) % 4 inside its 64 bytes:
-//   16 consecutive rows of a fragment read then cover the 64 LDS banks exactly once (ds_read_b128 serves 16 lanes per clock).
+// Data path per macro stage of 256 K elements (128 B = one cache line per operand row):
+//   global --buffer_load_dwordx4 ... lds (no register staging)--> LDS ring of 2 stages (64 KB each)
+//   LDS --ds_read_b128--> MFMA operands, four K steps of 64 per stage.
+//   The loads ask for whole 128-byte lines (8 lanes per row): the path from L2 into the compute unit moves whole lines,
+//   so half-line requests (a 128-K stage) cost twice the fill bandwidth, which is what bounds this kernel before the
+//   MFMA pipe does.  LDS instructions cost issue time on the SIMD that also issues the MFMAs -- about 12 clocks per
+//   ds_read_b128 and 40 per ds_write_b128 -- so the operand tiles never pass through ds_write.
+//   A 16-byte piece holds one MX block (32 codes); lane (r, h) of the MFMA takes piece 2j + h of row r at K step j, so a
+//   row's eight pieces are XOR-swizzled by (row / 2) % 8 inside its 128 bytes: 16 consecutive rows of a fragment read
+//   then cover the 64 LDS banks exactly once (ds_read_b128 serves 16 lanes per clock).
 // Scales: one byte per row per 32 K (1D) or per 32 rows (2D).  They are staged through LDS per block of 512 K (16 bytes
 //   per row, rows at a 20-byte pitch) so that 1D and 2D scales look alike to the MFMA loop; inside a row the bytes are
-//   regrouped so that the 8 bytes a lane needs for the 4 stages of a block are contiguous, and op_sel picks the byte.
+//   regrouped so that the 8 bytes a lane needs for the 8 K steps of a block are contiguous, and op_sel picks the byte.
 // The MFMA takes B rows as its first operand: accumulator registers then run along N (4 consecutive columns per lane).
 // bf16 results go through LDS (swizzled 16-byte chunks) so that the global stores are whole 512-byte row segments.
 #pragma once
@@ -20,10 +24,10 @@
 
 namespace alto {
 
-constexpr int GT_TM = 256, GT_TN = 256, GT_TK = 128;
+constexpr int GT_TM = 256, GT_TN = 256, GT_TK = 256;
 constexpr int GT_THREADS = 512;
-constexpr int GT_STAGE_BYTES = (GT_TM + GT_TN) * (GT_TK / 2);   // 32768
-constexpr int GT_NSTAGE = 4;
+constexpr int GT_STAGE_BYTES = (GT_TM + GT_TN) * (GT_TK / 2);   // 65536
+constexpr int GT_NSTAGE = 2;
 constexpr int GT_SCALE_PITCH = 5;                                // dwords per row (16 B + 4 B pad)
 constexpr int GT_SCALE_BUF_DW = (GT_TM + GT_TN) * GT_SCALE_PITCH;  // one buffer, in dwords
 constexpr int GT_LDS_BYTES = GT_NSTAGE * GT_STAGE_BYTES + 2 * GT_SCALE_BUF_DW * 4;  // 131072 + 20480 = 151552
@@ -38,6 +42,43 @@ struct TileArgs {
   int64_t a_bytes, b_bytes;    // extent of the code buffers in bytes (< 2^31), for the buffer descriptors
   int64_t as_bytes, bs_bytes;  // extent of the scale buffers in bytes (< 2^31)
 };
+
+// Every field of TileArgs is the same for all lanes.  When the struct arrives through memory (a real function call) the
+// compiler no longer knows that and would wrap each buffer load in a per-lane loop; this copies the fields into
+// scalar registers.
+__device__ __forceinline__ int64_t uniform_i64(int64_t v) {
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)((uint64_t)v >> 32));
+  return (int64_t)(((uint64_t)hi << 32) | lo);
+}
+__device__ __forceinline__ OperandView uniform_view(const OperandView& v) {
+  OperandView o;
+  o.codes = reinterpret_cast<const uint8_t*>(uniform_i64(reinterpret_cast<int64_t>(v.codes)));
+  o.ld = uniform_i64(v.ld);
+  o.scales = reinterpret_cast<const uint8_t*>(uniform_i64(reinterpret_cast<int64_t>(v.scales)));
+  o.ss_r = uniform_i64(v.ss_r);
+  o.ss_k = uniform_i64(v.ss_k);
+  o.is_2d = __builtin_amdgcn_readfirstlane(v.is_2d);
+  return o;
+}
+__device__ __forceinline__ TileArgs uniform_args(const TileArgs& t) {
+  TileArgs o;
+  o.A = uniform_view(t.A);
+  o.B = uniform_view(t.B);
+  o.m0 = uniform_i64(t.m0); o.n0 = uniform_i64(t.n0);
+  o.m_lo = uniform_i64(t.m_lo); o.m_hi = uniform_i64(t.m_hi); o.n_hi = uniform_i64(t.n_hi);
+  o.G = __builtin_amdgcn_readfirstlane(t.G);
+  o.out_scale = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, t.out_scale)));
+  o.a_bytes = uniform_i64(t.a_bytes); o.b_bytes = uniform_i64(t.b_bytes);
+  o.as_bytes = uniform_i64(t.as_bytes); o.bs_bytes = uniform_i64(t.bs_bytes);
+  return o;
+}
+
+// two floats -> packed bf16 (round to nearest even), one v_cvt_pk_bf16_f32
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  typedef float f2_t __attribute__((ext_vector_type(2)));
+  bf16x2_t p = __builtin_convertvector(f2_t{lo, hi}, bf16x2_t);
+  return __builtin_bit_cast(uint32_t, p);
+}
 
 typedef v16f_t TileAcc[4][2];   // per wave: 4 (M) x 2 (N) MFMA tiles of 32x32
 
@@ -63,53 +104,35 @@ __device__ __forceinline__ void gemm_tile_mainloop(const TileArgs& ta, TileAcc& 
   const int wm = wave >> 2, wn = wave & 3;
   const int r = lane & 31, h = lane >> 5;
   uint32_t* sscale = reinterpret_cast<uint32_t*>(smem + GT_NSTAGE * GT_STAGE_BYTES);
-  const int KB = (ta.G + 15) / 16;       // loop iterations: blocks of 512 K = 4 stages of 128 K
+  const int KB = (ta.G + 15) / 16;       // loop iterations: blocks of 512 K = 2 macro stages
   const int kbytes = ta.G * 16;
 
-  // ---- global -> register staging: instruction i (0..3) of this thread moves one 16-byte piece.
-  // Piece (i, wave, lane): operand = i / 2 (0: A, 1: B); chunk q = 8 * (i % 2) + wave covers tile rows 16q .. 16q+15;
-  // lane l holds row 16q + l / 4, slot l % 4, which stores global piece (l % 4) ^ ((l / 16) % 4) of that row.
-  // Raw buffer loads: 32-bit per-lane byte offsets, the K offset of the stage rides in the scalar offset, and a piece
-  // beyond the end of K gets an out-of-range offset, for which the hardware returns zeros.
+  // ---- global -> LDS: instruction i (0..7) of this wave moves chunk q = 8 i + wave = 8 tile rows x 128 bytes (whole
+  // cache lines).  Chunks 0..31 are A rows, 32..63 B rows.  Lane l holds row 8 q + l / 8, slot l % 8, which stores
+  // global piece (l % 8) ^ ((row / 2) % 8) of that row.  Raw buffer loads: 32-bit per-lane byte offsets, the K offset
+  // of the stage rides in the scalar offset, and a piece beyond the end of K gets an out-of-range offset, for which the
+  // hardware returns zeros.
   const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(ta.A.codes), 0, (int)ta.a_bytes, 0x00020000);
   const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(ta.B.codes), 0, (int)ta.b_bytes, 0x00020000);
-  uint32_t goff[4];
-  uint32_t ldst[4];
-  int gpiece;
+  // (per-load offsets are recomputed at every stage rather than kept in 8 registers: three VALU ops per 1 KB load)
+  const int gpiece = (lane & 7) ^ ((4 * (wave & 1) + (lane >> 4)) & 7);
+  const int arow0 = (int)ta.m0 + 8 * wave + (lane >> 3), brow0 = (int)ta.n0 + 8 * wave + (lane >> 3);
+  const int a_last = (int)ta.m_hi - 1, a_first = (int)ta.m_lo, b_last = (int)ta.n_hi - 1;
+  const uint32_t ld_a = (uint32_t)ta.A.ld, ld_b = (uint32_t)ta.B.ld;
+  // ---- fragment read offsets (bytes inside a stage): row * 128 + ((2 j + h) ^ ((row / 2) % 8)) * 16; the j-dependent
+  // part is an XOR with 32 j
+  uint32_t a_off, b_off;   // for j = 0
   {
-    const int rr = lane >> 2;
-    gpiece = (lane & 3) ^ ((rr >> 2) & 3);
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int q = 8 * (i & 1) + wave;
-      const int trow = 16 * q + rr;
-      if (i < 2) {
-        int64_t row = ta.m0 + trow;
-        row = row < ta.m_hi ? row : ta.m_hi - 1;
-        row = row < ta.m_lo ? ta.m_lo : row;
-        goff[i] = (uint32_t)(row * ta.A.ld + gpiece * 16);
-      } else {
-        int64_t row = ta.n0 + trow;
-        row = row < ta.n_hi ? row : ta.n_hi - 1;
-        goff[i] = (uint32_t)(row * ta.B.ld + gpiece * 16);
-      }
-      ldst[i] = (i < 2 ? 0 : GT_TM * 64) + q * 1024;   // wave-uniform chunk base; the hardware adds 16 * lane
-    }
-  }
-  // ---- fragment read offsets (bytes inside a stage): rows of this wave's sub-tiles, pieces 2h + j swizzled
-  uint32_t a_off, b_off;   // for j = 0; j = 1 is the same address ^ 16
-  {
-    const int sw = (r >> 2) & 3;
-    const int slot = (r & 15) * 4 + ((2 * h) ^ sw);
-    a_off = (uint32_t)((128 * wm + r) >> 4) * 1024 + slot * 16;
-    b_off = GT_TM * 64 + (uint32_t)((64 * wn + r) >> 4) * 1024 + slot * 16;
+    const int c0 = (h ^ ((r >> 1) & 7)) << 4;
+    a_off = (uint32_t)(128 * wm + r) * 128 + c0;
+    b_off = GT_TM * 128 + (uint32_t)(64 * wn + r) * 128 + c0;
   }
   // scale read offsets (bytes): row * 20 + 8h within a block buffer
   const uint32_t sa_off = (uint32_t)(128 * wm + r) * (GT_SCALE_PITCH * 4) + 8 * h;
   const uint32_t sb_off = (uint32_t)(GT_TM + 64 * wn + r) * (GT_SCALE_PITCH * 4) + 8 * h;
 
   // scale staging: thread t owns tile row t of A (t < 256) or tile row t - 256 of B (unit stride along K, any alignment)
-  const bool s_is_a = tid < GT_TM;   // wave-uniform
+  const bool s_is_a = wave < GT_TM / 64;   // scalar: the descriptor choice below must be provably wave-uniform
   const __amdgpu_buffer_rsrc_t rsrc_s = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<uint8_t*>(s_is_a ? ta.A.scales : ta.B.scales), 0, (int)(s_is_a ? ta.as_bytes : ta.bs_bytes), 0x00020000);
   uint32_t soff;
@@ -132,13 +155,26 @@ __device__ __forceinline__ void gemm_tile_mainloop(const TileArgs& ta, TileAcc& 
   typedef __attribute__((address_space(3))) uint8_t lds_u8;
   lds_u8* const lds = (lds_u8*)smem;
   auto gload = [&](int s, int slot) {
-    const int koff = s * 64;
+    const int koff = __builtin_amdgcn_readfirstlane(s * 128);   // scalar offset operand: must live in an SGPR
     // a piece beyond K gets bit 31 set in its offset: out of range for the descriptor, so zeros land in LDS
     const uint32_t oob = (koff + gpiece * 16 < kbytes) ? 0u : 0x80000000u;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const uint32_t off = goff[i] | oob;
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(i < 2 ? rsrc_a : rsrc_b, (__attribute__((address_space(3))) void*)(lds + slot * GT_STAGE_BYTES + ldst[i]),
+    for (int i = 0; i < 8; ++i) {
+      int row;
+      uint32_t off;
+      if (i < 4) {
+        row = arow0 + 64 * i;
+        row = row < a_last ? row : a_last;
+        row = row > a_first ? row : a_first;
+        off = (uint32_t)row * ld_a;
+      } else {
+        row = brow0 + 64 * (i - 4);
+        row = row < b_last ? row : b_last;
+        off = (uint32_t)row * ld_b;
+      }
+      off = (off + gpiece * 16) | oob;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(i < 4 ? rsrc_a : rsrc_b,
+                                               (__attribute__((address_space(3))) void*)(lds + slot * GT_STAGE_BYTES + (8 * i + wave) * 1024),
                                                16, (int)off, koff, 0, 0);
     }
   };
@@ -146,30 +182,42 @@ __device__ __forceinline__ void gemm_tile_mainloop(const TileArgs& ta, TileAcc& 
   // codes of a K tail never meet a NaN scale byte.
   auto sload = [&](int kb) {
     const int rem = ta.G - kb * 16;   // wave-uniform
+    const int kb16 = __builtin_amdgcn_readfirstlane(kb * 16);
+    if constexpr (!KTAIL) {   // rows are dword-aligned and every dword is all inside or all beyond K: one 16-byte load
+      v4i_t w4 = __builtin_amdgcn_raw_buffer_load_b128(rsrc_s, (int)soff, kb16, 0);
+#pragma unroll
+      for (int d = 0; d < 4; ++d) sreg[d] = rem - 4 * d >= 4 ? (uint32_t)w4[d] : 0x7F7F7F7Fu;
+      return;
+    }
+    // K tail: the row's last dword may be partial (G % 4 bytes).  Those bytes are fetched one by one, so that nothing
+    // is trusted from beyond the row (a dword load there may cross the end of the buffer and come back as zeros).
+    // Branch-free: all selections are mask arithmetic on wave-uniform values.
+    const int tail_at = __builtin_amdgcn_readfirstlane(ta.G & ~3);
+    uint32_t t0 = __builtin_amdgcn_raw_buffer_load_b8(rsrc_s, (int)soff, tail_at, 0);
+    uint32_t t1 = __builtin_amdgcn_raw_buffer_load_b8(rsrc_s, (int)soff, tail_at + 1, 0);
+    uint32_t t2 = __builtin_amdgcn_raw_buffer_load_b8(rsrc_s, (int)soff, tail_at + 2, 0);
+    asm volatile("" : "+v"(t0), "+v"(t1), "+v"(t2));
+    const uint32_t w_tail = (t0 & 0xFFu) | ((t1 & 0xFFu) << 8) | ((t2 & 0xFFu) << 16);
 #pragma unroll
     for (int d = 0; d < 4; ++d) {
-      const int n = rem - 4 * d;
-      uint32_t w = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rsrc_s, (int)soff, kb * 16 + 4 * d, 0);
-      const uint32_t keep = n >= 4 ? 0xFFFFFFFFu : 0u;
-      w = (w & keep) | (0x7F7F7F7Fu & ~keep);
-      if (KTAIL && n > 0 && n < 4) {   // last, partial dword of the row: bytes one by one, never past the row
-        uint32_t b0 = __builtin_amdgcn_raw_buffer_load_b8(rsrc_s, (int)soff, kb * 16 + 4 * d, 0);
-        uint32_t b1 = 127, b2 = 127;
-        if (n > 1) b1 = __builtin_amdgcn_raw_buffer_load_b8(rsrc_s, (int)soff, kb * 16 + 4 * d + 1, 0);
-        if (n > 2) b2 = __builtin_amdgcn_raw_buffer_load_b8(rsrc_s, (int)soff, kb * 16 + 4 * d + 2, 0);
-        w = (b0 & 0xFF) | ((b1 & 0xFF) << 8) | ((b2 & 0xFF) << 16) | (127u << 24);
-      }
-      sreg[d] = w;
+      const int n = rem - 4 * d;   // valid groups from this dword's first byte
+      uint32_t w = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rsrc_s, (int)soff, kb16 + 4 * d, 0);
+      asm volatile("" : "+v"(w));   // keep the load unconditional: a branch around it would split the MFMA loop
+      const int nn = n < 1 ? 1 : (n > 3 ? 3 : n);
+      const uint32_t part = (w_tail & ~(0xFFFFFFFFu << (8 * nn))) | (0x7F7F7F7Fu << (8 * nn));
+      const uint32_t m_full = (uint32_t)((3 - n) >> 31);               // all ones iff n >= 4 (mask arithmetic, no branch)
+      const uint32_t m_part = (uint32_t)((-n) >> 31) & ~m_full;        // all ones iff 0 < n < 4
+      sreg[d] = (w & m_full) | (part & m_part) | (0x7F7F7F7Fu & ~(m_full | m_part));
     }
   };
-  // LDS row layout (4 dwords): [h=0: stages 0,1 | h=0: stages 2,3 | h=1: stages 0,1 | h=1: stages 2,3], where the
-  // half-wave h of the MFMA uses groups 4i + 2h + {0, 1} at stage i; byte (2 (i % 2) + j) of dword (2h + i / 2).
+  // LDS row layout (4 dwords): [h=0: K 0..255 | h=0: K 256..511 | h=1: K 0..255 | h=1: K 256..511], where the half-wave h
+  // of the MFMA uses group 8 ms + 2 j + h at K step j of macro stage ms: byte j of dword 2 h + ms.
   auto swrite = [&](int kb) {
     uint32_t* row = sscale + (kb & 1) * GT_SCALE_BUF_DW + tid * GT_SCALE_PITCH;
-    row[0] = __builtin_amdgcn_perm(sreg[1], sreg[0], 0x05040100u);
-    row[1] = __builtin_amdgcn_perm(sreg[3], sreg[2], 0x05040100u);
-    row[2] = __builtin_amdgcn_perm(sreg[1], sreg[0], 0x07060302u);
-    row[3] = __builtin_amdgcn_perm(sreg[3], sreg[2], 0x07060302u);
+    row[0] = __builtin_amdgcn_perm(sreg[1], sreg[0], 0x06040200u);   // groups 0, 2, 4, 6
+    row[1] = __builtin_amdgcn_perm(sreg[3], sreg[2], 0x06040200u);   // groups 8, 10, 12, 14
+    row[2] = __builtin_amdgcn_perm(sreg[1], sreg[0], 0x07050301u);   // groups 1, 3, 5, 7
+    row[3] = __builtin_amdgcn_perm(sreg[3], sreg[2], 0x07050301u);   // groups 9, 11, 13, 15
   };
 
   // Fragment / scale registers: F0 = pieces of K step j = 0 of the current stage (read during the previous stage),
@@ -180,12 +228,12 @@ __device__ __forceinline__ void gemm_tile_mainloop(const TileArgs& ta, TileAcc& 
     const uint8_t* base = smem + slot * GT_STAGE_BYTES;
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
-      uint4 a4 = *reinterpret_cast<const uint4*>(base + ((a_off + t * 2048) ^ (j * 16)));
+      uint4 a4 = *reinterpret_cast<const uint4*>(base + ((a_off ^ (j * 32)) + t * 4096));
       fa[t] = v8i_t{(int)a4.x, (int)a4.y, (int)a4.z, (int)a4.w, 0, 0, 0, 0};
     }
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
-      uint4 b4 = *reinterpret_cast<const uint4*>(base + ((b_off + u * 2048) ^ (j * 16)));
+      uint4 b4 = *reinterpret_cast<const uint4*>(base + ((b_off ^ (j * 32)) + u * 4096));
       fb[u] = v8i_t{(int)b4.x, (int)b4.y, (int)b4.z, (int)b4.w, 0, 0, 0, 0};
     }
   };
@@ -203,73 +251,73 @@ __device__ __forceinline__ void gemm_tile_mainloop(const TileArgs& ta, TileAcc& 
       xb[u][1] = (int)p[1];
     }
   };
-  // 8 MFMAs of K step J of stage I (inside its block)
-  auto mfma8 = [&](auto ic, auto jc, const v8i_t (&fa)[4], const v8i_t (&fb)[2]) {
-    constexpr int I = decltype(ic)::value, J = decltype(jc)::value;
-    constexpr int SEL = 2 * (I & 1) + J, D = I >> 1;
+  // 8 MFMAs of K step J (0..3) of macro stage MS (0..1 inside its 512-K block): scale byte J of dword MS
+  auto mfma8 = [&](auto msc, auto jc, const v8i_t (&fa)[4], const v8i_t (&fb)[2]) {
+    constexpr int MS = decltype(msc)::value, J = decltype(jc)::value;
 #pragma unroll
     for (int t = 0; t < 4; ++t)
 #pragma unroll
       for (int u = 0; u < 2; ++u)
-        acc[t][u] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[u], fa[t], acc[t][u], 4, 4, SEL, sb[u][D], SEL, sa[t][D]);
+        acc[t][u] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[u], fa[t], acc[t][u], 4, 4, J, sb[u][MS], J, sa[t][MS]);
   };
-  // Barrier between stages.  At most the 4 loads of the youngest stage may still be in flight, so the stage read next is
-  // complete for this wave (vmcnt is in issue order), its LDS writes (scales) are done, and after the barrier that holds
-  // for every wave.  The asm keeps the compiler from moving LDS accesses across it.
-  auto stage_barrier = [&]() { asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
-
-  // One stage s = 4 kb + I: LDS slot I; the next stage lives in slot (I + 1) % 4.
-  //   barrier (stage s+1 has landed for every wave); issue the loads of stage s+3 into the slot stage s-1 used;
-  //   6 x {MFMA, LDS read}   j=0 MFMAs 0-5 + the j=1 pieces of this stage;  2 more j=0 MFMAs
-  //   6 x {MFMA, LDS read}   j=1 MFMAs 0-5 + the next stage's j=0 pieces;   2 more j=1 MFMAs
-  auto stage = [&](auto ic, int s) {
-    constexpr int I = decltype(ic)::value;
-    stage_barrier();
-    gload(s + 3, (I + 3) & 3);
-    read_frags(I, 1, fa1, fb1);
-    mfma8(ic, std::integral_constant<int, 0>{}, fa0, fb0);
-    read_frags((I + 1) & 3, 0, fa0, fb0);
-    mfma8(ic, std::integral_constant<int, 1>{}, fa1, fb1);
-    __builtin_amdgcn_sched_group_barrier(0x020, 4, 0);
+  auto interleave = [&]() {   // 6 x {MFMA, LDS read}, 2 more MFMAs
 #pragma unroll
     for (int q = 0; q < 6; ++q) {
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
       __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
     }
     __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
-#pragma unroll
-    for (int q = 0; q < 6; ++q) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+  };
+  // One macro stage s = 2 kb + MS (256 K, LDS slot MS), four K steps of 64.  Pieces of step j+1 are read while step j
+  // multiplies.  Before the last step: wait for this wave's loads of stage s+1 and meet the other waves -- then stage
+  // s+1 is in LDS for everyone and nobody reads this stage's slot any more (its step-3 pieces are in registers), so the
+  // loads of stage s+2 go out into it and the last step fetches the first pieces of stage s+1.
+  auto stage = [&](auto msc, int s, int kb) {
+    constexpr int MS = decltype(msc)::value;
+    mfma8(msc, std::integral_constant<int, 0>{}, fa0, fb0);
+    read_frags(MS, 1, fa1, fb1);
+    interleave();
+    __builtin_amdgcn_sched_barrier(0);
+    mfma8(msc, std::integral_constant<int, 1>{}, fa1, fb1);
+    read_frags(MS, 2, fa0, fb0);
+    interleave();
+    __builtin_amdgcn_sched_barrier(0);
+    mfma8(msc, std::integral_constant<int, 2>{}, fa0, fb0);
+    read_frags(MS, 3, fa1, fb1);
+    interleave();
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    if constexpr (MS == 0) {
+      swrite(kb + 1);          // block kb+1 -> the other scale buffer (last read at the end of block kb-1)
+      sload(kb + 2);
+      __builtin_amdgcn_sched_barrier(0);
     }
-    __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+    gload(s + 2, MS);
+    mfma8(msc, std::integral_constant<int, 3>{}, fa1, fb1);
+    read_frags(MS ^ 1, 0, fa0, fb0);
+    __builtin_amdgcn_sched_group_barrier(0x020, 16, 0);
+    interleave();
     __builtin_amdgcn_sched_barrier(0);
   };
 
-  // ---- prologue: stages 0, 1, 2 in flight into their slots; scale block 0 in LDS, block 1 in flight; then the first
-  // stage's j=0 pieces and the first block's scales in registers.  Stages beyond K load zeros and blocks beyond K load
-  // unit scales, so nothing below is conditional.
+  // ---- prologue: stage 0 and scale block 0 into LDS, stage 1 and scale block 1 in flight; then the first step's pieces
+  // and the first block's scales in registers.  Stages beyond K load zeros and blocks beyond K load unit scales, so
+  // nothing below is conditional.
   sload(0);
   gload(0, 0);
   swrite(0);
   sload(1);
   gload(1, 1);
-  gload(2, 2);
-  asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)\n\ts_barrier" ::: "memory");   // stage 0 and scale block 0 visible to all
+  asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)\n\ts_barrier" ::: "memory");   // all but stage 1's eight loads
   read_frags(0, 0, fa0, fb0);
   read_scales(reinterpret_cast<const uint8_t*>(sscale), sa, sb);
 
-  // ---- main loop: one iteration = one 512-K block = 4 stages; LDS slot = stage % 4.
+  // ---- main loop: one iteration = one 512-K block = 2 macro stages
   for (int kb = 0; kb < KB; ++kb) {
-    const int s = kb * 4;
     const uint8_t* sblock_next = reinterpret_cast<const uint8_t*>(sscale + ((kb + 1) & 1) * GT_SCALE_BUF_DW);
-    stage(std::integral_constant<int, 0>{}, s + 0);
-    stage(std::integral_constant<int, 1>{}, s + 1);
-    swrite(kb + 1);          // block kb+1 -> the other scale buffer (last read in iteration kb-1); visible after the next barrier
-    sload(kb + 2);
-    stage(std::integral_constant<int, 2>{}, s + 2);
-    stage(std::integral_constant<int, 3>{}, s + 3);
-    read_scales(sblock_next, sa, sb);   // next block's scales (written two stages ago)
+    stage(std::integral_constant<int, 0>{}, 2 * kb, kb);
+    stage(std::integral_constant<int, 1>{}, 2 * kb + 1, kb);
+    read_scales(sblock_next, sa, sb);   // next block's scales (written one macro stage ago)
   }
   // loads of the (zero-filled) stages past the end may still be landing in the ring the epilogue reuses
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -301,8 +349,8 @@ __device__ __forceinline__ void gemm_tile_store(const TileArgs& ta, TileAcc& acc
           float f0 = acc[t][u][4 * vq + 0] * ta.out_scale, f1 = acc[t][u][4 * vq + 1] * ta.out_scale;
           float f2 = acc[t][u][4 * vq + 2] * ta.out_scale, f3 = acc[t][u][4 * vq + 3] * ta.out_scale;
           uint2 o;
-          o.x = f32_to_bf16_bits(f0) | (f32_to_bf16_bits(f1) << 16);
-          o.y = f32_to_bf16_bits(f2) | (f32_to_bf16_bits(f3) << 16);
+          o.x = pack_bf16x2(f0, f1);
+          o.y = pack_bf16x2(f2, f3);
           *reinterpret_cast<uint2*>(smem + ml * 512 + ((chunk ^ (ml & 31)) << 4) + 8 * h) = o;
         }
       }

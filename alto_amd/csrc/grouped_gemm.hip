@@ -144,8 +144,11 @@ __device__ __forceinline__ void zero_rows(OutT* out, int64_t ldo, int64_t r0, in
 // The tile as a real function: inlined into the segment loop below, its address set-up competes with the loop's own
 // state for registers and spills.
 template <typename OutT, bool KTAIL>
-__device__ __noinline__ void grouped_tile_call(const TileArgs& ta, OutT* out, int64_t ldo) {
+__device__ __noinline__ void grouped_tile_call(const TileArgs& ta_mem, OutT* out_v, int64_t ldo_v) {
   extern __shared__ __align__(16) uint8_t smem[];
+  const TileArgs ta = uniform_args(ta_mem);
+  OutT* out = reinterpret_cast<OutT*>(uniform_i64(reinterpret_cast<int64_t>(out_v)));
+  const int64_t ldo = uniform_i64(ldo_v);
   gemm_tile_256x256<OutT, KTAIL>(ta, out, ldo, smem);
 }
 
