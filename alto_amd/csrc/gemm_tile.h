@@ -154,12 +154,12 @@ __device__ __forceinline__ void gemm_tile_mainloop(const TileArgs& ta, TileAcc& 
   // Direct-to-LDS load of stage s into ring slot `slot`: lane l of instruction i lands at chunk base + 16 l.
   typedef __attribute__((address_space(3))) uint8_t lds_u8;
   lds_u8* const lds = (lds_u8*)smem;
-  auto gload = [&](int s, int slot) {
+  auto gload = [&](int s, int slot, int i0, int i1) {   // instructions i0 .. i1-1 of the stage's eight (0-3: A rows, 4-7: B rows)
     const int koff = __builtin_amdgcn_readfirstlane(s * 128);   // scalar offset operand: must live in an SGPR
     // a piece beyond K gets bit 31 set in its offset: out of range for the descriptor, so zeros land in LDS
     const uint32_t oob = (koff + gpiece * 16 < kbytes) ? 0u : 0x80000000u;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
+    for (int i = i0; i < i1; ++i) {
       int row;
       uint32_t off;
       if (i < 4) {
@@ -268,15 +268,29 @@ __device__ __forceinline__ void gemm_tile_mainloop(const TileArgs& ta, TileAcc& 
     }
     __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
   };
+  auto interleave_loads = [&]() {   // the same with one global->LDS load after every second MFMA
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      if (q < 2) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    }
+    __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+  };
   // One macro stage s = 2 kb + MS (256 K, LDS slot MS), four K steps of 64.  Pieces of step j+1 are read while step j
   // multiplies.  Before the last step: wait for this wave's loads of stage s+1 and meet the other waves -- then stage
   // s+1 is in LDS for everyone and nobody reads this stage's slot any more (its step-3 pieces are in registers), so the
-  // loads of stage s+2 go out into it and the last step fetches the first pieces of stage s+1.
+  // loads of stage s+2 go out into it: half of them during the last step, half during the first step of the next
+  // stage, one load per two MFMAs.  (A wave issues in order, and the address unit takes a 1 KB load about every 16
+  // clocks per compute unit: a burst of eight loads per wave would hold the MFMAs behind it for a thousand clocks.)
   auto stage = [&](auto msc, int s, int kb) {
     constexpr int MS = decltype(msc)::value;
+    gload(s + 1, MS ^ 1, 4, 8);
     mfma8(msc, std::integral_constant<int, 0>{}, fa0, fb0);
     read_frags(MS, 1, fa1, fb1);
-    interleave();
+    interleave_loads();
     __builtin_amdgcn_sched_barrier(0);
     mfma8(msc, std::integral_constant<int, 1>{}, fa1, fb1);
     read_frags(MS, 2, fa0, fb0);
@@ -292,11 +306,10 @@ __device__ __forceinline__ void gemm_tile_mainloop(const TileArgs& ta, TileAcc& 
       sload(kb + 2);
       __builtin_amdgcn_sched_barrier(0);
     }
-    gload(s + 2, MS);
+    gload(s + 2, MS, 0, 4);
     mfma8(msc, std::integral_constant<int, 3>{}, fa1, fb1);
     read_frags(MS ^ 1, 0, fa0, fb0);
-    __builtin_amdgcn_sched_group_barrier(0x020, 16, 0);
-    interleave();
+    interleave_loads();
     __builtin_amdgcn_sched_barrier(0);
   };
 
@@ -304,11 +317,11 @@ __device__ __forceinline__ void gemm_tile_mainloop(const TileArgs& ta, TileAcc& 
   // and the first block's scales in registers.  Stages beyond K load zeros and blocks beyond K load unit scales, so
   // nothing below is conditional.
   sload(0);
-  gload(0, 0);
+  gload(0, 0, 0, 8);
   swrite(0);
   sload(1);
-  gload(1, 1);
-  asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)\n\ts_barrier" ::: "memory");   // all but stage 1's eight loads
+  gload(1, 1, 0, 4);   // the other half goes out in the first step of the loop
+  asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)\n\ts_barrier" ::: "memory");   // all but stage 1's four loads
   read_frags(0, 0, fa0, fb0);
   read_scales(reinterpret_cast<const uint8_t*>(sscale), sa, sb);
 
