@@ -41,6 +41,8 @@ struct TileArgs {
   float out_scale;
   int64_t a_bytes, b_bytes;    // extent of the code buffers in bytes (< 2^31), for the buffer descriptors
   int64_t as_bytes, bs_bytes;  // extent of the scale buffers in bytes (< 2^31)
+  int s_k0;                    // first scale byte of this reduction inside the operands' scale rows (0 unless a sub-range of K)
+  int s_row;                   // length of a whole scale row in bytes (>= 16): loads never reach past it
 };
 
 // Every field of TileArgs is the same for all lanes.  When the struct arrives through memory (a real function call) the
@@ -70,6 +72,7 @@ __device__ __forceinline__ TileArgs uniform_args(const TileArgs& t) {
   o.out_scale = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, t.out_scale)));
   o.a_bytes = uniform_i64(t.a_bytes); o.b_bytes = uniform_i64(t.b_bytes);
   o.as_bytes = uniform_i64(t.as_bytes); o.bs_bytes = uniform_i64(t.bs_bytes);
+  o.s_k0 = __builtin_amdgcn_readfirstlane(t.s_k0); o.s_row = __builtin_amdgcn_readfirstlane(t.s_row);
   return o;
 }
 
@@ -91,9 +94,9 @@ __device__ __forceinline__ void gemm_tile_zero(TileAcc& acc) {
       for (int v = 0; v < 16; ++v) acc[t][u][v] = 0.0f;
 }
 
-// K loop of one 256x256 tile: acc += A[m0.., :] . B[n0.., :]^T over G groups of 32.  KTAIL = false requires G % 4 == 0
-// (K a multiple of 128): then every scale dword of a row is either fully inside K or fully beyond it and the main loop
-// is branch-free.  KTAIL = true additionally handles a last partial dword of a scale row with byte loads.  Requirements
+// K loop of one 256x256 tile: acc += A[m0.., :] . B[n0.., :]^T over G groups of 32.  KTAIL = false requires G % 16 == 0
+// (K a multiple of 512) and s_k0 == 0: then every 16-byte scale block of a row lies inside the row.  KTAIL = true
+// handles any G and any start inside the scale rows (a reduction over a sub-range of K).  Requirements
 // checked by the host: unit-stride scale rows, operand extents below 2^31 bytes.  Every thread of the workgroup must
 // call it; it may be called again (same or other operands) to keep accumulating.
 template <bool KTAIL>
@@ -183,31 +186,43 @@ __device__ __forceinline__ void gemm_tile_mainloop(const TileArgs& ta, TileAcc& 
   auto sload = [&](int kb) {
     const int rem = ta.G - kb * 16;   // wave-uniform
     const int kb16 = __builtin_amdgcn_readfirstlane(kb * 16);
-    if constexpr (!KTAIL) {   // rows are dword-aligned and every dword is all inside or all beyond K: one 16-byte load
+    if constexpr (!KTAIL) {   // G % 4 == 0 and the whole K range: every dword is all inside or all beyond K, one 16-byte load
       v4i_t w4 = __builtin_amdgcn_raw_buffer_load_b128(rsrc_s, (int)soff, kb16, 0);
 #pragma unroll
       for (int d = 0; d < 4; ++d) sreg[d] = rem - 4 * d >= 4 ? (uint32_t)w4[d] : 0x7F7F7F7Fu;
       return;
     }
-    // K tail: the row's last dword may be partial (G % 4 bytes).  Those bytes are fetched one by one, so that nothing
-    // is trusted from beyond the row (a dword load there may cross the end of the buffer and come back as zeros).
-    // Branch-free: all selections are mask arithmetic on wave-uniform values.
-    const int tail_at = __builtin_amdgcn_readfirstlane(ta.G & ~3);
-    uint32_t t0 = __builtin_amdgcn_raw_buffer_load_b8(rsrc_s, (int)soff, tail_at, 0);
-    uint32_t t1 = __builtin_amdgcn_raw_buffer_load_b8(rsrc_s, (int)soff, tail_at + 1, 0);
-    uint32_t t2 = __builtin_amdgcn_raw_buffer_load_b8(rsrc_s, (int)soff, tail_at + 2, 0);
-    asm volatile("" : "+v"(t0), "+v"(t1), "+v"(t2));
-    const uint32_t w_tail = (t0 & 0xFFu) | ((t1 & 0xFFu) << 8) | ((t2 & 0xFFu) << 16);
+    // General case (any G, any sub-range of K): still one 16-byte load per row.  A block that would reach past the end
+    // of the scale row is loaded from the last 16 bytes of the row instead and shifted down by the difference, so no
+    // byte from beyond the row (possibly beyond the buffer) is ever used; bytes at or beyond G become 127.  All shift
+    // amounts and masks are wave-uniform and applied with mask arithmetic: no branch splits the MFMA loop.
+    const int want = ta.s_k0 + kb16;                     // where the block starts in the scale row
+    const int last = ta.s_row - 16;
+    const int off = __builtin_amdgcn_readfirstlane(want < last ? want : last);
+    int sh = want - off;                                 // bytes to shift down: 0 unless clamped
+    sh = sh > 16 ? 16 : sh;
+    const int q = sh >> 2, rb = sh & 3;
+    int valid = rem < 0 ? 0 : (rem > 16 ? 16 : rem);     // bytes of this block that lie inside K
+    v4i_t L = __builtin_amdgcn_raw_buffer_load_b128(rsrc_s, (int)soff, off, 0);
+    asm volatile("" : "+v"(L));
+    uint32_t mq[5];
+#pragma unroll
+    for (int c = 0; c < 5; ++c) mq[c] = (uint32_t)(-(int)(q == c));   // all ones for the dword shift in effect
 #pragma unroll
     for (int d = 0; d < 4; ++d) {
-      const int n = rem - 4 * d;   // valid groups from this dword's first byte
-      uint32_t w = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rsrc_s, (int)soff, kb16 + 4 * d, 0);
-      asm volatile("" : "+v"(w));   // keep the load unconditional: a branch around it would split the MFMA loop
-      const int nn = n < 1 ? 1 : (n > 3 ? 3 : n);
-      const uint32_t part = (w_tail & ~(0xFFFFFFFFu << (8 * nn))) | (0x7F7F7F7Fu << (8 * nn));
-      const uint32_t m_full = (uint32_t)((3 - n) >> 31);               // all ones iff n >= 4 (mask arithmetic, no branch)
-      const uint32_t m_part = (uint32_t)((-n) >> 31) & ~m_full;        // all ones iff 0 < n < 4
-      sreg[d] = (w & m_full) | (part & m_part) | (0x7F7F7F7Fu & ~(m_full | m_part));
+      uint32_t lo = 0, hi = 0;
+#pragma unroll
+      for (int c = 0; c < 5; ++c) {
+        const uint32_t xl = d + c < 4 ? (uint32_t)L[(d + c) & 3] : 0x7F7F7F7Fu;
+        const uint32_t xh = d + c + 1 < 4 ? (uint32_t)L[(d + c + 1) & 3] : 0x7F7F7F7Fu;
+        lo |= xl & mq[c];
+        hi |= xh & mq[c];
+      }
+      const uint32_t w = __builtin_amdgcn_alignbyte(hi, lo, (uint32_t)rb);
+      int nv = valid - 4 * d;
+      nv = nv < 0 ? 0 : (nv > 4 ? 4 : nv);
+      const uint32_t keep = (uint32_t)((1ull << (8 * nv)) - 1ull);
+      sreg[d] = (w & keep) | (0x7F7F7F7Fu & ~keep);
     }
   };
   // LDS row layout (4 dwords): [h=0: K 0..255 | h=0: K 256..511 | h=1: K 0..255 | h=1: K 256..511], where the half-wave h

@@ -32,7 +32,7 @@ __global__ __launch_bounds__(GT_THREADS) void gemm_tiled_kernel(OperandView A, O
   if (!tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn)) return;
   TileArgs ta{A, B, (int64_t)tm * GT_TM, (int64_t)tn * GT_TN, 0, M, N, G, out_scale,
               (M - 1) * A.ld + G * 16, (N - 1) * B.ld + G * 16,
-              ((A.is_2d ? M / 32 : M) - 1) * A.ss_r + G, ((B.is_2d ? N / 32 : N) - 1) * B.ss_r + G};
+              ((A.is_2d ? M / 32 : M) - 1) * A.ss_r + G, ((B.is_2d ? N / 32 : N) - 1) * B.ss_r + G, 0, G};
   gemm_tile_256x256<OutT, KTAIL>(ta, c, ldc, smem);
 }
 
@@ -56,7 +56,7 @@ int launch_tiled(const OperandView& A, const OperandView& B, int64_t M, int64_t 
 bool gemm_tiled_supported(const OperandView& A, const OperandView& B, int64_t M, int64_t N, int64_t K, const void* c, int c_dtype, int64_t ldc) {
   (void)c_dtype;
   // small problems do not fill 256x256 tiles; the direct kernel handles them
-  if (M < 128 || N < 128 || K < 128) return false;
+  if (M < 128 || N < 128 || K < 512) return false;   // (scale rows are read 16 bytes = 512 K at a time)
   // the tile kernel reads scale rows with unit stride along K and stores C in aligned 16-byte groups
   if (A.ss_k != 1 || B.ss_k != 1) return false;
   if (M * A.ld >= (1ll << 31) || N * B.ld >= (1ll << 31)) return false;   // 32-bit buffer offsets
@@ -68,7 +68,7 @@ bool gemm_tiled_supported(const OperandView& A, const OperandView& B, int64_t M,
 
 void gemm_tiled_launch(const OperandView& A, const OperandView& B, int64_t M, int64_t N, int64_t K, void* c, int c_dtype, int64_t ldc,
                        float out_scale, hipStream_t st) {
-  const bool tail = (K / 32) % 4 != 0;
+  const bool tail = (K / 32) % 16 != 0;   // K not a multiple of 512: the last scale block of a row is partial
   if (c_dtype == ALTO_DT_BF16) {
     if (tail) launch_tiled<__bf16, true>(A, B, M, N, K, c, ldc, out_scale, st);
     else launch_tiled<__bf16, false>(A, B, M, N, K, c, ldc, out_scale, st);

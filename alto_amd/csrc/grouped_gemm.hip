@@ -203,7 +203,7 @@ __global__ __launch_bounds__(GT_THREADS) void grouped_tiled_kernel(OperandView A
       OperandView B{w + e * w_stride_e, ldw, w_scales + e * ws_stride_e, ws_r, 1, w_is_2d};
       TileArgs ta{A, B, row0, n0, cur, seg_end, N, G, 1.0f,
                   (M_total - 1) * A.ld + G * 16, (N - 1) * ldw + G * 16,
-                  ((A.is_2d ? M_total / 32 : M_total) - 1) * A.ss_r + G, ((w_is_2d ? N / 32 : N) - 1) * ws_r + G};
+                  ((A.is_2d ? M_total / 32 : M_total) - 1) * A.ss_r + G, ((w_is_2d ? N / 32 : N) - 1) * ws_r + G, 0, G};
       grouped_tile_call<OutT, KTAIL>(ta, out, ldo);
       __syncthreads();   // the next segment reuses the LDS the store staged through
     }
@@ -290,16 +290,14 @@ __global__ __launch_bounds__(GT_THREADS) void grouped_dw_tiled_kernel(OperandVie
     }
     if (!have) break;
     if (t1 <= t0) continue;
-    OperandView Pv = P, Qv = Q;
+    OperandView Pv = P, Qv = Q;   // codes start at the run; the scale rows keep their base and the run's offset rides in s_k0
     Pv.codes += t0 / 2;
     Qv.codes += t0 / 2;
-    Pv.scales += t0 / 32;
-    Qv.scales += t0 / 32;
     TileArgs ta{Pv, Qv, (int64_t)tm * GT_TM, (int64_t)tn * GT_TN, 0, NP, NQ, (int)((t1 - t0) / 32), out_scale,
-                p_bytes - t0 / 2, q_bytes - t0 / 2, ps_bytes - t0 / 32, qs_bytes - t0 / 32};
+                p_bytes - t0 / 2, q_bytes - t0 / 2, ps_bytes, qs_bytes, (int)(t0 / 32), (int)(M_total / 32)};
     gemm_tile_mainloop<true>(ta, acc, smem);
   }
-  TileArgs ta{P, Q, (int64_t)tm * GT_TM, (int64_t)tn * GT_TN, 0, NP, NQ, 0, out_scale, 0, 0, 0, 0};
+  TileArgs ta{P, Q, (int64_t)tm * GT_TM, (int64_t)tn * GT_TN, 0, NP, NQ, 0, out_scale, 0, 0, 0, 0, 0, 0};
   gemm_tile_store<OutT>(ta, acc, dw + e * s_e, ld, smem);
 }
 
@@ -362,12 +360,12 @@ extern "C" int alto_mxfp4_grouped_gemm(const uint8_t* a, int64_t lda, const uint
   OperandView A{a, lda, a_scales, a_ss_r, a_ss_k, a_is_2d};
   // 256x256 tiles when the problem fills them and the layouts fit their loads (unit-stride scale rows, 32-bit buffer
   // offsets, 16-byte output chunks); otherwise the direct kernel below
-  const bool tiled = M_total >= 128 && N >= 128 && K >= 128 && a_ss_k == 1 && ws_k == 1 && N % 8 == 0 && ldo % 8 == 0 &&
+  const bool tiled = M_total >= 128 && N >= 128 && K >= 512 && a_ss_k == 1 && ws_k == 1 && N % 8 == 0 && ldo % 8 == 0 &&
                      (reinterpret_cast<uintptr_t>(out) & 15) == 0 && M_total * lda < (1ll << 31) && N * ldw < (1ll << 31) &&
                      M_total * a_ss_r < (1ll << 31) && N * ws_r < (1ll << 31) &&
                      ((M_total + GT_TM - 1) / GT_TM) * ((N + GT_TN - 1) / GT_TN) < (1ll << 28);
   if (tiled) {
-    const bool tail = (K / 32) % 4 != 0;
+    const bool tail = (K / 32) % 16 != 0;
     int rc;
     if (out_dtype == ALTO_DT_BF16)
       rc = tail ? launch_grouped_tiled<__bf16, true>(A, w, w_stride_e, ldw, w_scales, ws_stride_e, ws_r, w_is_2d, offs, group_expert, num_groups, num_experts, M_total, N, K, out, ldo, st)
@@ -421,7 +419,7 @@ extern "C" int alto_mxfp4_grouped_gemm_dw(const uint8_t* go, int64_t ld_go, cons
     const int64_t NP = n_major ? N : K, NQ = n_major ? K : N;
     const int64_t ld = n_major ? dw_stride_n : dw_stride_k;
     const bool unit = n_major || dw_stride_n == 1;
-    const bool tiled = unit && M_total >= 128 && N >= 128 && K >= 128 && gs_k == 1 && xs_k == 1 && NQ % 8 == 0 && ld % 8 == 0 && dw_stride_e % 8 == 0 &&
+    const bool tiled = unit && M_total >= 512 && N >= 128 && K >= 128 && gs_k == 1 && xs_k == 1 && NQ % 8 == 0 && ld % 8 == 0 && dw_stride_e % 8 == 0 &&
                        (reinterpret_cast<uintptr_t>(dw) & 15) == 0 && N * ld_go < (1ll << 31) && K * ld_xq < (1ll << 31) &&
                        N * gs_r < (1ll << 31) && K * xs_r < (1ll << 31) && num_groups <= GT_DW_MAX_GROUPS && num_experts <= 65535 &&
                        ((NP + GT_TM - 1) / GT_TM) * ((NQ + GT_TN - 1) / GT_TN) < (1ll << 28);

@@ -48,7 +48,8 @@ def test_gemm_matches_dequant_matmul(m, shape, use_2dblock_a, use_2dblock_b, tra
     assert O.rel_frobenius(c.cpu(), ref) < TOL[out_dtype]
 
 
-@pytest.mark.parametrize("shape", [(64, 96, 160), (100, 72, 96), (33, 40, 32), (256, 256, 2880)])
+@pytest.mark.parametrize("shape", [(64, 96, 160), (100, 72, 96), (33, 40, 32), (256, 256, 2880), (200, 136, 544), (128, 128, 992),
+                                   (300, 264, 512), (136, 256, 1312)])
 def test_gemm_ragged_shapes_and_kpack_false(m, shape):
     M, N, K = shape
     a = randn_outliers((M, K), torch.bfloat16, seed=3)
