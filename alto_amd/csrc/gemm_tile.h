@@ -94,52 +94,39 @@ __device__ __forceinline__ void gemm_tile_zero(TileAcc& acc) {
       for (int v = 0; v < 16; ++v) acc[t][u][v] = 0.0f;
 }
 
-// K loop of one 256x256 tile: acc += A[m0.., :] . B[n0.., :]^T over G groups of 32.  KTAIL = false requires G % 16 == 0
-// (K a multiple of 512) and s_k0 == 0: then every 16-byte scale block of a row lies inside the row.  KTAIL = true
-// handles any G and any start inside the scale rows (a reduction over a sub-range of K).  Requirements
-// checked by the host: unit-stride scale rows, operand extents below 2^31 bytes.  Every thread of the workgroup must
-// call it; it may be called again (same or other operands) to keep accumulating.
-template <bool KTAIL>
-__device__ __forceinline__ void gemm_tile_mainloop(const TileArgs& ta, TileAcc& acc, uint8_t* smem) {
-  __syncthreads();   // the LDS ring may still be read by a previous call
-  const int tid = threadIdx.x;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;   // the wave index lives in a scalar register
-  const int wm = wave >> 2, wn = wave & 3;
-  const int r = lane & 31, h = lane >> 5;
-  uint32_t* sscale = reinterpret_cast<uint32_t*>(smem + GT_NSTAGE * GT_STAGE_BYTES);
-  const int KB = (ta.G + 15) / 16;       // loop iterations: blocks of 512 K = 2 macro stages
-  const int kbytes = ta.G * 16;
+// Per-thread state of the global -> LDS operand loads and the scale loads of one tile.
+//   Operands: instruction i (0..7) of a wave moves chunk q = 8 i + wave = 8 tile rows x 128 bytes (whole cache lines).
+//   Chunks 0..31 are A rows, 32..63 B rows.  Lane l holds row 8 q + l / 8, slot l % 8, which stores global piece
+//   (l % 8) ^ ((row / 2) % 8) of that row.  Raw buffer loads: 32-bit per-lane byte offsets, the K offset of the stage
+//   rides in the scalar offset, and a piece beyond the end of K gets an out-of-range offset, for which the hardware
+//   returns zeros.  (Per-load offsets are recomputed at every stage rather than kept in 8 registers.)
+//   Scales: thread t owns tile row t of A (t < 256) or tile row t - 256 of B (unit stride along K, any alignment).
+struct TileLoader {
+  __amdgpu_buffer_rsrc_t rsrc_a, rsrc_b, rsrc_s;
+  int wave, gpiece, arow0, brow0, a_last, a_first, b_last, kbytes, G, s_k0, s_row;
+  uint32_t ld_a, ld_b, soff;
 
-  // ---- global -> LDS: instruction i (0..7) of this wave moves chunk q = 8 i + wave = 8 tile rows x 128 bytes (whole
-  // cache lines).  Chunks 0..31 are A rows, 32..63 B rows.  Lane l holds row 8 q + l / 8, slot l % 8, which stores
-  // global piece (l % 8) ^ ((row / 2) % 8) of that row.  Raw buffer loads: 32-bit per-lane byte offsets, the K offset
-  // of the stage rides in the scalar offset, and a piece beyond the end of K gets an out-of-range offset, for which the
-  // hardware returns zeros.
-  const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(ta.A.codes), 0, (int)ta.a_bytes, 0x00020000);
-  const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(ta.B.codes), 0, (int)ta.b_bytes, 0x00020000);
-  // (per-load offsets are recomputed at every stage rather than kept in 8 registers: three VALU ops per 1 KB load)
-  const int gpiece = (lane & 7) ^ ((4 * (wave & 1) + (lane >> 4)) & 7);
-  const int arow0 = (int)ta.m0 + 8 * wave + (lane >> 3), brow0 = (int)ta.n0 + 8 * wave + (lane >> 3);
-  const int a_last = (int)ta.m_hi - 1, a_first = (int)ta.m_lo, b_last = (int)ta.n_hi - 1;
-  const uint32_t ld_a = (uint32_t)ta.A.ld, ld_b = (uint32_t)ta.B.ld;
-  // ---- fragment read offsets (bytes inside a stage): row * 128 + ((2 j + h) ^ ((row / 2) % 8)) * 16; the j-dependent
-  // part is an XOR with 32 j
-  uint32_t a_off, b_off;   // for j = 0
-  {
-    const int c0 = (h ^ ((r >> 1) & 7)) << 4;
-    a_off = (uint32_t)(128 * wm + r) * 128 + c0;
-    b_off = GT_TM * 128 + (uint32_t)(64 * wn + r) * 128 + c0;
-  }
-  // scale read offsets (bytes): row * 20 + 8h within a block buffer
-  const uint32_t sa_off = (uint32_t)(128 * wm + r) * (GT_SCALE_PITCH * 4) + 8 * h;
-  const uint32_t sb_off = (uint32_t)(GT_TM + 64 * wn + r) * (GT_SCALE_PITCH * 4) + 8 * h;
-
-  // scale staging: thread t owns tile row t of A (t < 256) or tile row t - 256 of B (unit stride along K, any alignment)
-  const bool s_is_a = wave < GT_TM / 64;   // scalar: the descriptor choice below must be provably wave-uniform
-  const __amdgpu_buffer_rsrc_t rsrc_s = __builtin_amdgcn_make_buffer_rsrc(
-      const_cast<uint8_t*>(s_is_a ? ta.A.scales : ta.B.scales), 0, (int)(s_is_a ? ta.as_bytes : ta.bs_bytes), 0x00020000);
-  uint32_t soff;
-  {
+  __device__ __forceinline__ void init(const TileArgs& ta) {
+    const int tid = threadIdx.x;
+    wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // the wave index lives in a scalar register
+    const int lane = tid & 63;
+    rsrc_a = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(ta.A.codes), 0, (int)ta.a_bytes, 0x00020000);
+    rsrc_b = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(ta.B.codes), 0, (int)ta.b_bytes, 0x00020000);
+    gpiece = (lane & 7) ^ ((4 * (wave & 1) + (lane >> 4)) & 7);
+    arow0 = (int)ta.m0 + 8 * wave + (lane >> 3);
+    brow0 = (int)ta.n0 + 8 * wave + (lane >> 3);
+    a_last = (int)ta.m_hi - 1;
+    a_first = (int)ta.m_lo;
+    b_last = (int)ta.n_hi - 1;
+    ld_a = (uint32_t)ta.A.ld;
+    ld_b = (uint32_t)ta.B.ld;
+    kbytes = ta.G * 16;
+    G = ta.G;
+    s_k0 = ta.s_k0;
+    s_row = ta.s_row;
+    const bool s_is_a = wave < GT_TM / 64;   // scalar: the descriptor choice below must be provably wave-uniform
+    rsrc_s = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(s_is_a ? ta.A.scales : ta.B.scales), 0,
+                                               (int)(s_is_a ? ta.as_bytes : ta.bs_bytes), 0x00020000);
     int64_t row;
     if (s_is_a) {
       row = ta.m0 + tid;
@@ -152,12 +139,12 @@ __device__ __forceinline__ void gemm_tile_mainloop(const TileArgs& ta, TileAcc& 
       soff = (uint32_t)((ta.B.is_2d ? (row >> 5) : row) * ta.B.ss_r);
     }
   }
-  uint32_t sreg[4];
 
-  // Direct-to-LDS load of stage s into ring slot `slot`: lane l of instruction i lands at chunk base + 16 l.
-  typedef __attribute__((address_space(3))) uint8_t lds_u8;
-  lds_u8* const lds = (lds_u8*)smem;
-  auto gload = [&](int s, int slot, int i0, int i1) {   // instructions i0 .. i1-1 of the stage's eight (0-3: A rows, 4-7: B rows)
+  // Direct-to-LDS load of stage s into ring slot `slot`, instructions i0 .. i1-1 of the stage's eight (0-3: A rows,
+  // 4-7: B rows): lane l of instruction i lands at chunk base + 16 l.
+  __device__ __forceinline__ void gload(uint8_t* smem, int s, int slot, int i0, int i1) const {
+    typedef __attribute__((address_space(3))) uint8_t lds_u8;
+    lds_u8* const lds = (lds_u8*)smem;
     const int koff = __builtin_amdgcn_readfirstlane(s * 128);   // scalar offset operand: must live in an SGPR
     // a piece beyond K gets bit 31 set in its offset: out of range for the descriptor, so zeros land in LDS
     const uint32_t oob = (koff + gpiece * 16 < kbytes) ? 0u : 0x80000000u;
@@ -180,11 +167,13 @@ __device__ __forceinline__ void gemm_tile_mainloop(const TileArgs& ta, TileAcc& 
                                                (__attribute__((address_space(3))) void*)(lds + slot * GT_STAGE_BYTES + (8 * i + wave) * 1024),
                                                16, (int)off, koff, 0, 0);
     }
-  };
+  }
+
   // 16 scale bytes of K block kb for this thread's row; groups at or beyond G read as 127 (scale 1.0) so that the zero
   // codes of a K tail never meet a NaN scale byte.
-  auto sload = [&](int kb) {
-    const int rem = ta.G - kb * 16;   // wave-uniform
+  template <bool KTAIL>
+  __device__ __forceinline__ void sload(int kb, uint32_t (&sreg)[4]) const {
+    const int rem = G - kb * 16;   // wave-uniform
     const int kb16 = __builtin_amdgcn_readfirstlane(kb * 16);
     if constexpr (!KTAIL) {   // G % 4 == 0 and the whole K range: every dword is all inside or all beyond K, one 16-byte load
       v4i_t w4 = __builtin_amdgcn_raw_buffer_load_b128(rsrc_s, (int)soff, kb16, 0);
@@ -196,8 +185,8 @@ __device__ __forceinline__ void gemm_tile_mainloop(const TileArgs& ta, TileAcc& 
     // of the scale row is loaded from the last 16 bytes of the row instead and shifted down by the difference, so no
     // byte from beyond the row (possibly beyond the buffer) is ever used; bytes at or beyond G become 127.  All shift
     // amounts and masks are wave-uniform and applied with mask arithmetic: no branch splits the MFMA loop.
-    const int want = ta.s_k0 + kb16;                     // where the block starts in the scale row
-    const int last = ta.s_row - 16;
+    const int want = s_k0 + kb16;                     // where the block starts in the scale row
+    const int last = s_row - 16;
     const int off = __builtin_amdgcn_readfirstlane(want < last ? want : last);
     int sh = want - off;                                 // bytes to shift down: 0 unless clamped
     sh = sh > 16 ? 16 : sh;
@@ -224,7 +213,38 @@ __device__ __forceinline__ void gemm_tile_mainloop(const TileArgs& ta, TileAcc& 
       const uint32_t keep = (uint32_t)((1ull << (8 * nv)) - 1ull);
       sreg[d] = (w & keep) | (0x7F7F7F7Fu & ~keep);
     }
-  };
+  }
+};
+
+// K loop of one 256x256 tile: acc += A[m0.., :] . B[n0.., :]^T over G groups of 32.  KTAIL = false requires G % 16 == 0
+// (K a multiple of 512) and s_k0 == 0: then every 16-byte scale block of a row lies inside the row.  KTAIL = true
+// handles any G and any start inside the scale rows (a reduction over a sub-range of K).  Requirements
+// checked by the host: unit-stride scale rows, operand extents below 2^31 bytes.  Every thread of the workgroup must
+// call it; it may be called again (same or other operands) to keep accumulating.
+template <bool KTAIL>
+__device__ __forceinline__ void gemm_tile_mainloop(const TileArgs& ta, TileAcc& acc, uint8_t* smem) {
+  TileLoader ld;
+  uint32_t sreg[4];
+  __syncthreads();   // the LDS ring may still be read by a previous call
+  const int tid = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;   // the wave index lives in a scalar register
+  const int wm = wave >> 2, wn = wave & 3;
+  const int r = lane & 31, h = lane >> 5;
+  uint32_t* sscale = reinterpret_cast<uint32_t*>(smem + GT_NSTAGE * GT_STAGE_BYTES);
+  const int KB = (ta.G + 15) / 16;       // loop iterations: blocks of 512 K = 2 macro stages
+
+  // ---- fragment read offsets (bytes inside a stage): row * 128 + ((2 j + h) ^ ((row / 2) % 8)) * 16; the j-dependent
+  // part is an XOR with 32 j
+  uint32_t a_off, b_off;   // for j = 0
+  {
+    const int c0 = (h ^ ((r >> 1) & 7)) << 4;
+    a_off = (uint32_t)(128 * wm + r) * 128 + c0;
+    b_off = GT_TM * 128 + (uint32_t)(64 * wn + r) * 128 + c0;
+  }
+  // scale read offsets (bytes): row * 20 + 8h within a block buffer
+  const uint32_t sa_off = (uint32_t)(128 * wm + r) * (GT_SCALE_PITCH * 4) + 8 * h;
+  const uint32_t sb_off = (uint32_t)(GT_TM + 64 * wn + r) * (GT_SCALE_PITCH * 4) + 8 * h;
+
   // LDS row layout (4 dwords): [h=0: K 0..255 | h=0: K 256..511 | h=1: K 0..255 | h=1: K 256..511], where the half-wave h
   // of the MFMA uses group 8 ms + 2 j + h at K step j of macro stage ms: byte j of dword 2 h + ms.
   auto swrite = [&](int kb) {
@@ -238,7 +258,7 @@ __device__ __forceinline__ void gemm_tile_mainloop(const TileArgs& ta, TileAcc& 
   // Fragment / scale registers: F0 = pieces of K step j = 0 of the current stage (read during the previous stage),
   // F1 = pieces of step j = 1, S = this block's scale bytes (8 per lane and sub-tile, selected by op_sel).
   v8i_t fa0[4], fb0[2], fa1[4], fb1[2];
-  int sa[4][2], sb[2][2];
+  int sa[4][2], sb[2][2], sa_next[4][2], sb_next[2][2];
   auto read_frags = [&](int slot, int j, v8i_t (&fa)[4], v8i_t (&fb)[2]) {
     const uint8_t* base = smem + slot * GT_STAGE_BYTES;
 #pragma unroll
@@ -302,7 +322,7 @@ __device__ __forceinline__ void gemm_tile_mainloop(const TileArgs& ta, TileAcc& 
   // clocks per compute unit: a burst of eight loads per wave would hold the MFMAs behind it for a thousand clocks.)
   auto stage = [&](auto msc, int s, int kb) {
     constexpr int MS = decltype(msc)::value;
-    gload(s + 1, MS ^ 1, 4, 8);
+    ld.gload(smem, s + 1, MS ^ 1, 4, 8);
     mfma8(msc, std::integral_constant<int, 0>{}, fa0, fb0);
     read_frags(MS, 1, fa1, fb1);
     interleave_loads();
@@ -318,10 +338,12 @@ __device__ __forceinline__ void gemm_tile_mainloop(const TileArgs& ta, TileAcc& 
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
     if constexpr (MS == 0) {
       swrite(kb + 1);          // block kb+1 -> the other scale buffer (last read at the end of block kb-1)
-      sload(kb + 2);
+      ld.template sload<KTAIL>(kb + 2, sreg);
       __builtin_amdgcn_sched_barrier(0);
     }
-    gload(s + 2, MS, 0, 4);
+    ld.gload(smem, s + 2, MS, 0, 4);
+    if constexpr (MS == 1)   // the next block's scales (in LDS since this stage's barrier) ride along with the last step
+      read_scales(reinterpret_cast<const uint8_t*>(sscale + ((kb + 1) & 1) * GT_SCALE_BUF_DW), sa_next, sb_next);
     mfma8(msc, std::integral_constant<int, 3>{}, fa1, fb1);
     read_frags(MS ^ 1, 0, fa0, fb0);
     interleave_loads();
@@ -331,21 +353,24 @@ __device__ __forceinline__ void gemm_tile_mainloop(const TileArgs& ta, TileAcc& 
   // ---- prologue: stage 0 and scale block 0 into LDS, stage 1 and scale block 1 in flight; then the first step's pieces
   // and the first block's scales in registers.  Stages beyond K load zeros and blocks beyond K load unit scales, so
   // nothing below is conditional.
-  sload(0);
-  gload(0, 0, 0, 8);
+  ld.init(ta);
+  ld.template sload<KTAIL>(0, sreg);
+  ld.gload(smem, 0, 0, 0, 8);
   swrite(0);
-  sload(1);
-  gload(1, 1, 0, 4);   // the other half goes out in the first step of the loop
+  ld.template sload<KTAIL>(1, sreg);
+  ld.gload(smem, 1, 1, 0, 4);   // the other half goes out in the first step of the loop
   asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)\n\ts_barrier" ::: "memory");   // all but stage 1's four loads
   read_frags(0, 0, fa0, fb0);
   read_scales(reinterpret_cast<const uint8_t*>(sscale), sa, sb);
 
   // ---- main loop: one iteration = one 512-K block = 2 macro stages
   for (int kb = 0; kb < KB; ++kb) {
-    const uint8_t* sblock_next = reinterpret_cast<const uint8_t*>(sscale + ((kb + 1) & 1) * GT_SCALE_BUF_DW);
     stage(std::integral_constant<int, 0>{}, 2 * kb, kb);
     stage(std::integral_constant<int, 1>{}, 2 * kb + 1, kb);
-    read_scales(sblock_next, sa, sb);   // next block's scales (written one macro stage ago)
+#pragma unroll
+    for (int t = 0; t < 4; ++t) { sa[t][0] = sa_next[t][0]; sa[t][1] = sa_next[t][1]; }
+#pragma unroll
+    for (int u = 0; u < 2; ++u) { sb[u][0] = sb_next[u][0]; sb[u][1] = sb_next[u][1]; }
   }
   // loads of the (zero-filled) stages past the end may still be landing in the ring the epilogue reuses
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
