@@ -64,7 +64,10 @@ __device__ __forceinline__ float div_sqrt32_signed(float z, uint32_t flip) {
 
 template <typename T>
 __device__ __forceinline__ float round_to_T(float v) {
-  if constexpr (sizeof(T) == 2) return u2f(f32_to_bf16_bits(v) << 16);
+  if constexpr (sizeof(T) == 2) {   // float -> bf16 (round to nearest even, one v_cvt_pk_bf16_f32 per pair) -> float
+    const __bf16 b = (__bf16)v;
+    return u2f((uint32_t)__builtin_bit_cast(unsigned short, b) << 16);
+  }
   return v;
 }
 
@@ -91,8 +94,16 @@ __global__ __launch_bounds__(256) void quant_kernel(const QuantParams p) {
     __syncthreads();
   }
 
-  const T* xb = reinterpret_cast<const T*>(p.x) + b * p.bs_x;
-  const uint32_t* rb = SR ? p.rand + b * p.bs_r : nullptr;
+  // Tile-relative addressing: the descriptors start at the tile's first row, per-lane offsets are 32-bit, and the row
+  // step of each load is a scalar offset, so no load needs 64-bit address arithmetic.  (The host bounds ld_x / ld_rand.)
+  const int rows_here = M - row0 < 32 ? M - row0 : 32;
+  const T* xt = reinterpret_cast<const T*>(p.x) + b * p.bs_x + (int64_t)row0 * p.ld_x;
+  const __amdgpu_buffer_rsrc_t rsrc_x = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<T*>(xt), 0, (int)(((int64_t)(rows_here - 1) * p.ld_x + C) * (int64_t)sizeof(T)), 0x00020000);
+  const uint32_t* rt_ = SR ? p.rand + b * p.bs_r + (int64_t)row0 * p.ld_r : nullptr;
+  const __amdgpu_buffer_rsrc_t rsrc_r = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<uint32_t*>(rt_), 0, SR ? (int)(((int64_t)(rows_here - 1) * p.ld_r + C) * 4) : 0, 0x00020000);
+  const int ldx_b = (int)p.ld_x * (int)sizeof(T), ldr_b = (int)p.ld_r * 4;   // row pitches in bytes
 
   // ------------------------------------------------------------------ row phase
   const int chunk = tid & 31;
@@ -104,17 +115,15 @@ __global__ __launch_bounds__(256) void quant_kernel(const QuantParams p) {
   for (int i = 0; i < 4; ++i) {
     const int r = (tid >> 5) + 8 * i;
     valid[i] = (row0 + r < M) && (c < C);
-    if (valid[i]) {
-      const uint4* src = reinterpret_cast<const uint4*>(xb + (int64_t)(row0 + r) * p.ld_x + c);
-      uint4 v0 = src[0];
-      w[i][0] = v0.x; w[i][1] = v0.y; w[i][2] = v0.z; w[i][3] = v0.w;
+    {
+      // rows past M are out of the descriptor's range and read as zeros; columns past C get an out-of-range offset
+      const int voff = valid[i] ? (tid >> 5) * ldx_b + c * (int)sizeof(T) : (int)0x80000000;
+      const v4i_t v0 = __builtin_amdgcn_raw_buffer_load_b128(rsrc_x, voff, 8 * i * ldx_b, 0);
+      w[i][0] = v0[0]; w[i][1] = v0[1]; w[i][2] = v0[2]; w[i][3] = v0[3];
       if constexpr (!BF) {
-        uint4 v1 = src[1];
-        w[i][4] = v1.x; w[i][5] = v1.y; w[i][6] = v1.z; w[i][7] = v1.w;
+        const v4i_t v1 = __builtin_amdgcn_raw_buffer_load_b128(rsrc_x, voff, 8 * i * ldx_b + 16, 0);
+        w[i][4] = v1[0]; w[i][5] = v1[1]; w[i][6] = v1[2]; w[i][7] = v1[3];
       }
-    } else {
-#pragma unroll
-      for (int e = 0; e < (BF ? 4 : 8); ++e) w[i][e] = 0;
     }
     if (DO_COL) {
       const int pos = RHT ? sperm[r] : r;
@@ -178,9 +187,11 @@ __global__ __launch_bounds__(256) void quant_kernel(const QuantParams p) {
         out = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(out, v[6], v[7], scale_f, 3);
       } else {
         const float inv = u2f((254u - s) << 23);
-        const uint4* rs = reinterpret_cast<const uint4*>(rb + row * p.ld_r + c);
-        uint4 r0 = rs[0], r1 = rs[1];
-        uint32_t rr[8] = {r0.x, r0.y, r0.z, r0.w, r1.x, r1.y, r1.z, r1.w};
+        const int roff = (tid >> 5) * ldr_b + c * 4;
+        const v4i_t r0 = __builtin_amdgcn_raw_buffer_load_b128(rsrc_r, roff, 8 * i * ldr_b, 0);
+        const v4i_t r1 = __builtin_amdgcn_raw_buffer_load_b128(rsrc_r, roff, 8 * i * ldr_b + 16, 0);
+        uint32_t rr[8] = {(uint32_t)r0[0], (uint32_t)r0[1], (uint32_t)r0[2], (uint32_t)r0[3],
+                          (uint32_t)r1[0], (uint32_t)r1[1], (uint32_t)r1[2], (uint32_t)r1[3]};
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
           float q = v[e] * inv;
@@ -241,7 +252,7 @@ __global__ __launch_bounds__(256) void quant_kernel(const QuantParams p) {
         codes[k] = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(0u, v, 0.0f, scale_f, 0) & 0xFu;
       } else {
         const int row = RHT ? p.perm_inv[k] : k;
-        uint32_t r = rb[(int64_t)(row0 + row) * p.ld_r + cc];
+        const uint32_t r = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rsrc_r, tid * 4 + col0 * 4, __builtin_amdgcn_readfirstlane(row * ldr_b), 0);
         float q = v * inv;
         codes[k] = e2m1_sr_mag(__builtin_fabsf(q), r) | ((f2u(q) >> 28) & 8u);
       }
@@ -387,6 +398,7 @@ extern "C" int alto_mxfp4_quantize(const void* x, int dtype, int64_t batch, int6
   const int64_t vec = dtype == ALTO_DT_BF16 ? 8 : 4;
   ALTO_REQUIRE(ld_x >= C && ld_x % vec == 0 && bs_x % vec == 0, "quantize: ld_x/bs_x must be >= C and multiples of %lld elements", (long long)vec);
   ALTO_REQUIRE((reinterpret_cast<uintptr_t>(x) & 15) == 0, "quantize: x must be 16-byte aligned");
+  ALTO_REQUIRE(ld_x < (1ll << 24) && ld_rand < (1ll << 24), "quantize: row strides of 2^24 elements or more are not supported");
   ALTO_REQUIRE(rounding == ALTO_ROUND_RNE || rounding == ALTO_ROUND_SR, "quantize: bad rounding mode %d", rounding);
   if (rounding == ALTO_ROUND_SR) {
     ALTO_REQUIRE(rand_bits != nullptr, "quantize: stochastic rounding needs rand_bits");
