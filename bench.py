@@ -263,6 +263,32 @@ class CopyCalibration(Workload):
         return (lambda: dst.copy_(src)), self.work, "the same 256 MiB copy on the host"
 
 
+class MfmaProbe(Workload):
+    """Register-only loop of FP4 scaled-MFMA instructions (no memory traffic): the rate the matrix pipe itself sustains
+    on this part, with constant or pseudo-random FP4 operands.  A diagnostic next to the published peak, not a product path."""
+    bound = "mfma"
+    kernel = "mfma_probe_kernel"
+
+    def __init__(self, random_operands):
+        self.random = int(random_operands)
+        self.name = f"mfma_pipe_probe[{'random' if self.random else 'constant'} operands]"
+
+    def setup(self, dev, gen):
+        import torch
+        from alto_amd.mxfp4 import _runtime as rt
+        self.rt, self.stream = rt, rt.stream_ptr(dev)
+        self.sink = torch.zeros(512, dtype=torch.float32, device=dev)
+        self.iters, self.wgs = 4000, torch.cuda.get_device_properties(dev).multi_processor_count
+        self.work = 2.0 * 32 * 32 * 64 * 8 * self.iters * 8 * self.wgs
+
+    def step(self):
+        code = self.rt.lib().alto_mxfp4_probe_mfma(self.random, self.iters, self.wgs, self.sink.data_ptr(), self.stream)
+        assert code == 0, code
+
+    def cpu_sample(self):
+        raise NotImplementedError("the probe has no CPU counterpart")
+
+
 def load_traffic(key):
     """HBM bytes per launch of the workload's dominant kernel, from the committed rocprofv3 counter summaries (or None)."""
     try:
@@ -282,6 +308,8 @@ def make_workloads():
         "cfg4_wgrad": Gemm("cfg4_wgrad_gemm[4096x14336x8192]", 4096, 14336, 8192, False, False, "grad", "act"),
         "cfg5_grouped": GroupedGemm(),
         "copy_calib": CopyCalibration(),
+        "mfma_probe_const": MfmaProbe(False),
+        "mfma_probe_random": MfmaProbe(True),
     }
 
 
@@ -353,6 +381,11 @@ def main():
     if not args.only:
         for key, w in wl.items():
             if key == args.workload or key == "copy_calib":
+                continue
+            if key.startswith("mfma_probe"):   # the pipe's own rate, reported beside the published peak
+                r = measure(w, dev, gen, 3, 1)
+                others[key] = {"workload": r["workload"], "ms": round(r["ms"], 4), "achieved": round(r["achieved"], 2), "unit": r["unit"],
+                               "bound": r["bound"], "frac": round(r["frac"], 4)}
                 continue
             primary_mem_release = None  # noqa: F841
             try:

@@ -173,6 +173,15 @@ int alto_mxfp4_grouped_gemm_dw(const uint8_t* go, int64_t ld_go, const uint8_t* 
                                void* dw, int dw_dtype, int64_t dw_stride_e, int64_t dw_stride_n, int64_t dw_stride_k,
                                float out_scale, void* stream);
 
+/*
+ * Diagnostic, no counterpart in the reference: a register-only loop of FP4 scaled-MFMA instructions
+ * (8 per iteration and wave, 8 waves per workgroup, `workgroups` workgroups; 2*32*32*64 FLOP each),
+ * with constant (random_operands = 0) or pseudo-random FP4 operands.  bench.py times it to report
+ * the rate the matrix pipe itself sustains on this part next to the published peak.
+ * `sink` is device memory for 512 floats (practically never written).
+ */
+int alto_mxfp4_probe_mfma(int random_operands, int iters, int workgroups, float* sink, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
