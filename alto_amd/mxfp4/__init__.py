@@ -7,6 +7,7 @@ from .hadamard import HadamardFactory, HadamardTransform
 from .linear import MXFP4LinearFunction, _to_mxfp4_then_scaled_mm, blockwise_mxfp4_gemm, transpose_codes
 from .quantization import BLOCK_SIZE_DEFAULT, convert_from_mxfp4, convert_to_mxfp4, hadamard_left, quantize_rowcol
 from ._runtime import set_rand_bits_source
+from .tensor import MXFP4TrainingWeightWrapperTensor, TrainingWeightWrapperBaseTensor, swap_params
 
 __all__ = (
     "_quantize_then_mxfp_scaled_grouped_mm",
@@ -30,4 +31,7 @@ __all__ = (
     "hadamard_left",
     "transpose_codes",
     "set_rand_bits_source",
+    "MXFP4TrainingWeightWrapperTensor",
+    "TrainingWeightWrapperBaseTensor",
+    "swap_params",
 )

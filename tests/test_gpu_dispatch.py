@@ -1,0 +1,80 @@
+"""The weight-wrapper tensor routes linear-like ops and torch._grouped_mm to the MXFP4 path
+(alto/kernels/dispatch/tensor.py:214-303): results and gradients equal the direct calls."""
+import pytest
+import torch
+
+from tests.helpers import rand_bits, randn_outliers
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+@pytest.fixture(scope="module")
+def m():
+    import alto_amd.mxfp4 as mod
+    return mod
+
+
+def _fixed_randomness(m, shape_seed):
+    m.HadamardFactory.configure(seed=1234)
+    m.set_rand_bits_source(lambda shp, d: rand_bits(tuple(shp), seed=shape_seed).to(d))
+
+
+def test_linear_module_through_wrapper(m):
+    cfg = m.TrainingOpConfig()   # production recipe: 1D x, 2D w, Hadamard, stochastic gradient rounding
+    lin = torch.nn.Linear(256, 384, bias=True, dtype=torch.bfloat16, device=DEV)
+    with torch.no_grad():
+        lin.weight.copy_(randn_outliers((384, 256), torch.bfloat16, seed=1).to(DEV) * 0.02)
+    w_plain = lin.weight.detach().clone().requires_grad_(True)
+    x = randn_outliers((4, 64, 256), torch.bfloat16, seed=2).to(DEV)
+    go = randn_outliers((4, 64, 384), torch.bfloat16, seed=3).to(DEV) / 1000
+    try:
+        _fixed_randomness(m, 7)
+        x1 = x.clone().requires_grad_(True)
+        y_ref = m._to_mxfp4_then_scaled_mm(x1, w_plain, cfg.use_2dblock_x, cfg.use_2dblock_w, cfg.use_sr_grad, cfg.use_dge,
+                                           cfg.clip_mode, cfg.use_hadamard) + lin.bias
+        y_ref.backward(go)
+        m.swap_params(lin, config=cfg)
+        assert isinstance(lin.weight.data, m.MXFP4TrainingWeightWrapperTensor)
+        _fixed_randomness(m, 7)
+        x2 = x.clone().requires_grad_(True)
+        y = lin(x2)
+        y.backward(go)
+    finally:
+        m.set_rand_bits_source(None)
+    assert type(y) is torch.Tensor
+    assert torch.equal(y, y_ref)
+    assert torch.equal(x2.grad, x1.grad)
+    assert lin.weight.grad is not None and torch.equal(lin.weight.grad, w_plain.grad)
+    assert lin.bias.grad is not None
+
+
+def test_mm_with_wrapped_second_operand(m):
+    cfg = m.TrainingOpConfig(use_hadamard=False, use_sr_grad=False)
+    w = (randn_outliers((256, 128), torch.bfloat16, seed=4) * 0.02).to(DEV)      # [K, N]: mm(x, w)
+    x = randn_outliers((96, 256), torch.bfloat16, seed=5).to(DEV)
+    ww = m.MXFP4TrainingWeightWrapperTensor(w, cfg)
+    y = torch.mm(x, ww)
+    y_ref = m._to_mxfp4_then_scaled_mm(x, w.T, False, True, False, False, "none", False)
+    assert torch.equal(y, y_ref)
+    y2 = torch.addmm(torch.ones(128, dtype=torch.bfloat16, device=DEV), x, ww)
+    assert torch.equal(y2, y_ref + 1)
+
+
+def test_grouped_mm_through_wrapper(m):
+    cfg = m.TrainingOpConfig(use_hadamard=False, use_sr_grad=False)
+    E, K, N = 4, 256, 384
+    w = (randn_outliers((E, K, N), torch.bfloat16, seed=6) * 0.02).to(DEV)       # torch._grouped_mm layout [E, K, N]
+    a = randn_outliers((512, K), torch.bfloat16, seed=7).to(DEV)
+    offs = torch.tensor([128, 128, 384, 512], dtype=torch.int32, device=DEV)
+    wp = torch.nn.Parameter(m.MXFP4TrainingWeightWrapperTensor(w.clone(), cfg))
+    a1 = a.clone().requires_grad_(True)
+    y = torch._grouped_mm(a1, wp, offs=offs)
+    y.float().square().mean().backward()
+    w2 = w.clone().requires_grad_(True)
+    a2 = a.clone().requires_grad_(True)
+    y_ref = m._quantize_then_mxfp_scaled_grouped_mm(a2, w2, offs, False, True, False, False, False, "none", False)
+    y_ref.float().square().mean().backward()
+    assert torch.equal(y, y_ref)
+    assert torch.equal(a1.grad, a2.grad)
+    assert torch.equal(wp.grad, w2.grad)

@@ -94,3 +94,32 @@ def test_group_helpers():
     assert g.n == 4 and g.offs.tolist() == [0, 128, 256, 384, 512] and g.expert.tolist() == [0, 2, 2, 3]
     off = G.offsets_from_ends(ends)
     assert off.tolist() == [0, 128, 128, 384, 512] and G.groups_from_offsets(off).n == 4
+
+
+# ----------------------------------------------------------------------------------------------- weight wrapper (CPU)
+def test_weight_wrapper_passes_other_ops_through():
+    """Non-GEMM ops see the plain payload; view-like ops keep the wrapper (alto/kernels/dispatch/tensor.py:33-47,101-137)."""
+    import alto_amd.mxfp4 as m
+    cfg = m.TrainingOpConfig()
+    w = torch.randn(64, 32)
+    ww = m.MXFP4TrainingWeightWrapperTensor(w, cfg)
+    assert ww.shape == w.shape and ww.dtype == w.dtype and ww._data is w
+    assert isinstance(ww.detach(), m.MXFP4TrainingWeightWrapperTensor)
+    t = ww.t()
+    assert isinstance(t, m.MXFP4TrainingWeightWrapperTensor) and t.shape == (32, 64) and t.config == cfg
+    assert isinstance(ww.clone(), m.MXFP4TrainingWeightWrapperTensor)
+    s = ww + 1.0
+    assert type(s) is torch.Tensor and torch.equal(s, w + 1.0)
+    assert torch.equal(m.linear.unwrap_weight_wrapper(ww), w)
+
+
+def test_swap_params_wraps_weights_not_biases():
+    import alto_amd.mxfp4 as m
+    cfg = m.TrainingOpConfig()
+    model = torch.nn.Sequential(torch.nn.Linear(32, 64), torch.nn.ReLU(), torch.nn.Linear(64, 32))
+    m.swap_params(model, config=cfg, module_filter_fn=lambda mod, fqn: isinstance(mod, torch.nn.Linear) and fqn == "2")
+    assert type(model[0].weight.data) is torch.Tensor
+    assert isinstance(model[2].weight.data, m.MXFP4TrainingWeightWrapperTensor) and model[2].weight.requires_grad
+    assert type(model[2].bias.data) is torch.Tensor
+    with pytest.raises(ValueError):
+        m.swap_params(model, config=None)
