@@ -83,6 +83,14 @@ __device__ __forceinline__ uint32_t e2m1_rne_mag(float m) {
   return m < 1.0f ? den : n;
 }
 
+// E2M1 code (sign in bit 3) -> value: 0, 0.5, then (1 + m/2) * 2^(e-1)
+__device__ __forceinline__ float e2m1_decode(uint32_t code) {
+  uint32_t c = code & 7u;
+  uint32_t bits = (((c >> 1) + 126u) << 23) | ((c & 1u) << 22);
+  bits = c == 0u ? 0u : (c == 1u ? 0x3F000000u : bits);
+  return u2f(bits | ((code & 8u) << 28));
+}
+
 // ----------------------------------------------------------------------------- device: cross-lane
 template <int CTRL>
 __device__ __forceinline__ uint32_t dpp_u32(uint32_t v) {

@@ -4,14 +4,6 @@
 namespace alto {
 namespace {
 
-__device__ __forceinline__ float e2m1_decode(uint32_t code) {
-  // 0, 0.5, then (1 + m/2) * 2^(e-1); sign in bit 3
-  uint32_t c = code & 7u;
-  uint32_t bits = (((c >> 1) + 126u) << 23) | ((c & 1u) << 22);
-  bits = c == 0u ? 0u : (c == 1u ? 0x3F000000u : bits);
-  return u2f(bits | ((code & 8u) << 28));
-}
-
 // one thread: 8 codes (one dword of packed data) of one row
 template <typename OutT>
 __global__ __launch_bounds__(256) void dequant_kernel(const uint8_t* __restrict__ codes, const uint8_t* __restrict__ scales,

@@ -4,7 +4,9 @@ from .grouped_gemm import (ALIGN_SIZE_M, MXFP4GroupedGEMM, _quantize_then_mxfp_s
                            create_indices_from_offsets_nosync, mxfp4_grouped_gemm, mxfp4_grouped_gemm_backward_inputs,
                            mxfp4_grouped_gemm_backward_weights, mxfp4_grouped_gemm_forward)
 from .hadamard import HadamardFactory, HadamardTransform
-from .linear import MXFP4LinearFunction, _to_mxfp4_then_scaled_mm, blockwise_mxfp4_gemm, transpose_codes
+from .linear import (MXFP4LinearFunction, _to_mxfp4_then_scaled_mm, blockwise_mxfp4_gemm, clear_weight_cache, enable_weight_cache,
+                     transpose_codes, weight_cache_stats)
+from .qdq import _make_qdq_fn_for, quantize_dequantize
 from .quantization import BLOCK_SIZE_DEFAULT, convert_from_mxfp4, convert_to_mxfp4, hadamard_left, quantize_rowcol
 from ._runtime import set_rand_bits_source
 from .tensor import MXFP4TrainingWeightWrapperTensor, TrainingWeightWrapperBaseTensor, swap_params
@@ -34,4 +36,9 @@ __all__ = (
     "MXFP4TrainingWeightWrapperTensor",
     "TrainingWeightWrapperBaseTensor",
     "swap_params",
+    "enable_weight_cache",
+    "clear_weight_cache",
+    "weight_cache_stats",
+    "quantize_dequantize",
+    "_make_qdq_fn_for",
 )

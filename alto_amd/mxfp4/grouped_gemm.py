@@ -18,7 +18,7 @@ import torch
 from . import _runtime as rt
 from .._lib import check
 from .hadamard import HadamardFactory, HadamardTransform
-from .linear import transpose_codes, unwrap_weight_wrapper
+from .linear import cached_weight_quantisation, transpose_codes, unwrap_weight_wrapper
 from .quantization import convert_to_mxfp4, quantize_rowcol
 
 ALIGN_SIZE_M = 128
@@ -218,9 +218,8 @@ def _quantize_experts(w: torch.Tensor, use_uos: bool):
     """w [E, R, C] (unit stride along C) -> codes packed along C [E,R,C/2], 2D scales [E,R/32,C/32], codes packed along R
     [E,C,R/2] and the same scales stored transposed [E,C/32,R/32] (each operand of a GEMM wants unit stride along its K)."""
     from .quantization import _prep, _quantize_call
-    E, R, C = w.shape
-    w3 = _prep(w)
-    return _quantize_call(w3, True, True, True, False, None, None, 0, use_uos)
+    return cached_weight_quantisation(w, ("experts2d", bool(use_uos)),
+                                      lambda: _quantize_call(_prep(w), True, True, True, False, None, None, 0, use_uos))
 
 
 def mxfp4_grouped_gemm(inputs, expert_weights, expert_indices, *, trans_weights=True, use_2dblock_x=False, use_2dblock_w=True,

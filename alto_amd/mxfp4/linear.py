@@ -24,6 +24,54 @@ def unwrap_weight_wrapper(weight: torch.Tensor) -> torch.Tensor:
     return weight.as_subclass(torch.Tensor)
 
 
+# ----------------------------------------------------------------------------------------------- quantized-weight cache
+# The reference re-quantizes the weight in every forward (mxfp_linear.py:317-322).  Between two optimizer steps the
+# weight does not change (gradient accumulation, activation recomputation), so the four tensors of its 2D-block
+# quantisation can be kept.  An entry is valid while the weight's storage, shape and autograd version counter are the
+# ones it was made from: any in-place update (optimizer step, copy_) bumps the counter and the entry is rebuilt.
+_WEIGHT_CACHE_ENABLED = False
+_WEIGHT_CACHE: dict = {}
+_WEIGHT_CACHE_STATS = {"hits": 0, "misses": 0}
+
+
+def enable_weight_cache(enabled: bool = True) -> None:
+    """Keep the quantized form of 2D-block weights across forwards until the weight is modified in place."""
+    global _WEIGHT_CACHE_ENABLED
+    _WEIGHT_CACHE_ENABLED = bool(enabled)
+    if not enabled:
+        clear_weight_cache()
+
+
+def clear_weight_cache() -> None:
+    _WEIGHT_CACHE.clear()
+    _WEIGHT_CACHE_STATS["hits"] = _WEIGHT_CACHE_STATS["misses"] = 0
+
+
+def weight_cache_stats() -> dict:
+    return dict(_WEIGHT_CACHE_STATS, entries=len(_WEIGHT_CACHE))
+
+
+def cached_weight_quantisation(weight: torch.Tensor, tag, make):
+    """``make()`` or, with the cache enabled and the weight unchanged since, the tensors it returned last time."""
+    if not _WEIGHT_CACHE_ENABLED:
+        return make()
+    key = (weight.data_ptr(), weight.device.index, tag)
+    stamp = (weight._version, tuple(weight.shape), tuple(weight.stride()), weight.dtype)
+    hit = _WEIGHT_CACHE.get(key)
+    if hit is not None and hit[0] == stamp:
+        _WEIGHT_CACHE_STATS["hits"] += 1
+        return hit[1]
+    _WEIGHT_CACHE_STATS["misses"] += 1
+    out = make()
+    _WEIGHT_CACHE[key] = (stamp, out)
+    return out
+
+
+def _quantize_weight_2d(weight: torch.Tensor, use_uos: bool):
+    """(w_q, w_s, w_qt, w_st) of a 2D-block quantisation, from the cache when the weight is unchanged."""
+    return cached_weight_quantisation(weight, ("linear2d", bool(use_uos)), lambda: quantize_rowcol(weight, True, use_uos=use_uos))
+
+
 def transpose_codes(codes: torch.Tensor) -> torch.Tensor:
     """[R, C/2] bytes packed along C -> [C, R/2] bytes packed along R (same 4-bit codes)."""
     assert codes.dim() == 2 and codes.dtype == torch.uint8
@@ -148,7 +196,7 @@ class MXFP4LinearFunction(torch.autograd.Function):
                 x_qm, x_sm = convert_to_mxfp4(x2, axis=0, clip_mode=clip_mode, use_uos=use_uos, hadamard=hadamard_transform)
 
         if use_2dblock_w:
-            w_q, w_s, w_qt, w_st = quantize_rowcol(weight, True, use_uos=use_uos)
+            w_q, w_s, w_qt, w_st = _quantize_weight_2d(weight, use_uos)
             # [N/2, K] view over [K][N/2] memory; scales [N/32, K/32] as a view over [K/32][N/32] memory (same values as
             # w_s, stored so that the dgrad GEMM reads them with unit stride along its reduction dim N)
             w_bwd, w_bwd_s = w_qt, w_st

@@ -174,6 +174,17 @@ int alto_mxfp4_grouped_gemm_dw(const uint8_t* go, int64_t ld_go, const uint8_t* 
                                float out_scale, void* stream);
 
 /*
+ * Fused quantize -> dequantize: y = convert_from_mxfp4(convert_to_mxfp4(x, axis=-1, is_2d_block), output_dtype = dtype
+ * of x), round to nearest even, no clipping, in one pass (no codes or scales are written).  Replaces the pair of
+ * launches in the weight de-oscillation hook (alto/components/optimizer.py:123-158, which calls
+ * mxfp_quantization.py:410-484 then :487-545).  x, y: `batch` row-major matrices [M][C] of bf16 or f32 with row
+ * strides ld_x / ld_y and matrix strides bs_x / bs_y (elements).  With 2D blocks the result does not depend on the
+ * quantisation axis; a 1D quantisation along the row dim is not offered here.
+ */
+int alto_mxfp4_qdq(const void* x, int dtype, int64_t batch, int64_t M, int64_t C, int64_t ld_x, int64_t bs_x,
+                   void* y, int64_t ld_y, int64_t bs_y, int is_2d, int use_uos, void* stream);
+
+/*
  * Diagnostic, no counterpart in the reference: a register-only loop of FP4 scaled-MFMA instructions
  * (8 per iteration and wave, 8 waves per workgroup, `workgroups` workgroups; 2*32*32*64 FLOP each),
  * with constant (random_operands = 0) or pseudo-random FP4 operands.  bench.py times it to report

@@ -78,3 +78,49 @@ def test_grouped_mm_through_wrapper(m):
     assert torch.equal(y, y_ref)
     assert torch.equal(a1.grad, a2.grad)
     assert torch.equal(wp.grad, w2.grad)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("is_2d", [True, False])
+@pytest.mark.parametrize("use_uos", [False, True])
+def test_fused_qdq_equals_quantize_then_dequantize(m, dtype, is_2d, use_uos):
+    """One launch == convert_from_mxfp4(convert_to_mxfp4(w)) bit for bit (the de-oscillation hook, optimizer.py:123-168)."""
+    w = (randn_outliers((3, 96, 320), dtype, seed=11) * 0.02).to(DEV)
+    for axis in (-1, -2):
+        q, s = m.convert_to_mxfp4(w, axis=axis, is_2d_block=is_2d, use_uos=use_uos)
+        ref = m.convert_from_mxfp4(q, s, output_dtype=dtype, axis=axis, is_2d_block=is_2d)
+        got = m.quantize_dequantize(w, axis=axis, is_2d_block=is_2d, use_uos=use_uos)
+        assert got.dtype == dtype and got.shape == w.shape
+        assert torch.equal(got.view(torch.int16 if dtype == torch.bfloat16 else torch.int32),
+                           ref.contiguous().view(torch.int16 if dtype == torch.bfloat16 else torch.int32)), (axis, is_2d)
+    # the recipe-level closure, with a row count that is not a multiple of 32 (padded as the reference does)
+    cfg = m.TrainingOpConfig(use_2dblock_w=is_2d, use_uos=use_uos)
+    w2 = (randn_outliers((100, 256), dtype, seed=12) * 0.02).to(DEV)
+    got = m._make_qdq_fn_for(cfg)(w2, -1)
+    wp = torch.nn.functional.pad(w2, (0, 0, 0, 28))
+    q, s = m.convert_to_mxfp4(wp, axis=-1, is_2d_block=is_2d, use_uos=use_uos)
+    ref = m.convert_from_mxfp4(q, s, output_dtype=dtype, axis=-1, is_2d_block=is_2d)[:100]
+    assert got.shape == (100, 256) and torch.equal(got, ref)
+
+
+def test_weight_cache_reuses_until_weight_changes(m):
+    x = randn_outliers((64, 256), torch.bfloat16, seed=13).to(DEV)
+    w = (randn_outliers((128, 256), torch.bfloat16, seed=14) * 0.02).to(DEV).requires_grad_(True)
+    args = (False, True, False, False, "none", False)
+    y0 = m._to_mxfp4_then_scaled_mm(x, w, *args)
+    m.enable_weight_cache(True)
+    try:
+        y1 = m._to_mxfp4_then_scaled_mm(x, w, *args)
+        y2 = m._to_mxfp4_then_scaled_mm(x, w, *args)
+        assert m.weight_cache_stats() == {"hits": 1, "misses": 1, "entries": 1}
+        assert torch.equal(y1, y0) and torch.equal(y2, y0)
+        y2.float().sum().backward()          # backward of a cached forward still works
+        assert w.grad is not None
+        with torch.no_grad():
+            w.mul_(2.0)                       # an optimizer-style in-place update invalidates the entry
+        y3 = m._to_mxfp4_then_scaled_mm(x, w, *args)
+        assert m.weight_cache_stats()["misses"] == 2
+        m.enable_weight_cache(False)
+        assert torch.equal(y3, m._to_mxfp4_then_scaled_mm(x, w, *args))
+    finally:
+        m.enable_weight_cache(False)
