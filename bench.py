@@ -3,7 +3,7 @@
 
 ``python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]`` prints ONE JSON line.
 
-The default workload is the MXFP4 fprop GEMM at the Llama-3-8B MLP up-projection shape (config 3 of BASELINE.json):
+The default workload is the MXFP4 fprop GEMM at the Llama-3-8B MLP up-projection shape (M=8192, N=14336, K=4096):
 a "step" is one GEMM launch on operands already quantized and resident in HBM; ``value`` is TFLOP/s.  The same line
 carries the fused RHT+SR gradient quantizer (config 2, GB/s) and the other GEMM shapes under ``"others"``, a
 ``roofline`` object for the dominant kernel of the selected workload (duration measured live with HIP events on the
@@ -355,7 +355,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     args = ap.parse_args()
     if args.gpus != 1:
-        print("bench.py measures one GPU: this build has no multi-GPU path (every kernel is per-shard; see DESIGN.md). "
+        print("bench.py measures one GPU: this build has no multi-GPU path (every kernel works on one GPU's shard). "
               "Run with --gpus 1.", file=sys.stderr)
         sys.exit(2)
 

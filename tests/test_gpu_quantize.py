@@ -155,7 +155,7 @@ def test_fused_2d_weight_gives_both_packings(m):
 
 
 def test_config1_roundtrip_full_size(m):
-    """BASELINE config 1: bf16 [4096, 4096] ~ N(0,1) with 1% entries x50, 1D blocks, RNE, no Hadamard."""
+    """Benchmark configuration 1: bf16 [4096, 4096] ~ N(0,1) with 1% entries x50, 1D blocks, RNE, no Hadamard."""
     g = torch.Generator().manual_seed(0)
     x = torch.randn(4096, 4096, generator=g)
     x = torch.where(torch.rand(4096, 4096, generator=g) < 0.01, x * 50, x).bfloat16()
@@ -172,7 +172,7 @@ def test_config1_roundtrip_full_size(m):
 
 
 def test_config2_fused_gradient_quantizer_full_size(m):
-    """BASELINE config 2: bf16 [8192, 4096] ~ Laplace(0, 1e-3), row copy + Hadamard column copy, SR with supplied bits."""
+    """Benchmark configuration 2: bf16 [8192, 4096] ~ Laplace(0, 1e-3), row copy + Hadamard column copy, SR with supplied bits."""
     M, C = 8192, 4096
     x = laplace((M, C), 1e-3, torch.bfloat16, seed=21)
     r = rand_bits((M, C), seed=22)
