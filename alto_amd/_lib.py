@@ -26,6 +26,10 @@ SIGNATURES = {
                                     c_vp, c_vp, c_vp, c_vp,
                                     c_int, c_int, c_vp, c_i64, c_i64,
                                     c_int, c_vp, c_vp, c_int, c_int, c_vp]),
+    "alto_mxfp4_quantize_pitched": (c_int, [c_vp, c_int, c_i64, c_i64, c_i64, c_i64, c_i64,
+                                            c_vp, c_vp, c_vp, c_vp, c_i64, c_i64,
+                                            c_int, c_int, c_vp, c_i64, c_i64,
+                                            c_int, c_vp, c_vp, c_int, c_int, c_vp]),
     "alto_mxfp4_hadamard": (c_int, [c_vp, c_int, c_i64, c_i64, c_i64, c_vp, c_i64, c_vp, c_vp, c_vp]),
     "alto_mxfp4_dequantize": (c_int, [c_vp, c_vp, c_i64, c_i64, c_int, c_vp, c_int, c_i64, c_i64, c_int, c_vp]),
     "alto_mxfp4_transpose_codes": (c_int, [c_vp, c_i64, c_i64, c_vp, c_vp]),

@@ -29,6 +29,7 @@ struct QuantParams {
   uint8_t* row_scales;
   uint8_t* col_codes;
   uint8_t* col_scales;
+  int64_t ld_rc, ld_cc;  // row pitch in bytes of the row / column code outputs (>= C/2, M/2)
   uint32_t sign_mask;    // bit k set: Q[k] == -1 (k = position after the permutation)
   uint8_t perm[32];      // row j of a block -> position perm[j]
   uint8_t perm_inv[32];  // position k -> row
@@ -199,7 +200,7 @@ __global__ __launch_bounds__(256) void quant_kernel(const QuantParams p) {
           out |= code << (4 * e);
         }
       }
-      *reinterpret_cast<uint32_t*>(p.row_codes + (b * M + row) * (C / 2) + (c >> 1)) = out;
+      *reinterpret_cast<uint32_t*>(p.row_codes + (b * M + row) * p.ld_rc + (c >> 1)) = out;
     }
   }
 
@@ -282,7 +283,7 @@ __global__ __launch_bounds__(256) void quant_kernel(const QuantParams p) {
         out[j] = o;
       }
     }
-    *reinterpret_cast<uint4*>(p.col_codes + (b * C + cc) * (M / 2) + blockIdx.y * 16) = make_uint4(out[0], out[1], out[2], out[3]);
+    *reinterpret_cast<uint4*>(p.col_codes + (b * C + cc) * p.ld_cc + blockIdx.y * 16) = make_uint4(out[0], out[1], out[2], out[3]);
   }
 }
 
@@ -382,7 +383,21 @@ extern "C" int alto_mxfp4_quantize(const void* x, int dtype, int64_t batch, int6
                                    int is_2d, int rounding, const uint32_t* rand_bits, int64_t ld_rand, int64_t bs_rand,
                                    int hadamard, const int8_t* signs, const uint8_t* perm,
                                    int clip_mode, int use_uos, void* stream) {
+  return alto_mxfp4_quantize_pitched(x, dtype, batch, M, C, ld_x, bs_x, row_codes, row_scales, col_codes, col_scales, 0, 0, is_2d, rounding,
+                                     rand_bits, ld_rand, bs_rand, hadamard, signs, perm, clip_mode, use_uos, stream);
+}
+
+extern "C" int alto_mxfp4_quantize_pitched(const void* x, int dtype, int64_t batch, int64_t M, int64_t C, int64_t ld_x, int64_t bs_x,
+                                           uint8_t* row_codes, uint8_t* row_scales, uint8_t* col_codes, uint8_t* col_scales,
+                                           int64_t ld_row_codes, int64_t ld_col_codes,
+                                           int is_2d, int rounding, const uint32_t* rand_bits, int64_t ld_rand, int64_t bs_rand,
+                                           int hadamard, const int8_t* signs, const uint8_t* perm,
+                                           int clip_mode, int use_uos, void* stream) {
   using namespace alto;
+  if (ld_row_codes == 0) ld_row_codes = C / 2;
+  if (ld_col_codes == 0) ld_col_codes = M / 2;
+  ALTO_REQUIRE(row_codes == nullptr || (ld_row_codes >= C / 2 && ld_row_codes % 4 == 0), "quantize: ld_row_codes must be >= C/2 and a multiple of 4 bytes");
+  ALTO_REQUIRE(col_codes == nullptr || (ld_col_codes >= M / 2 && ld_col_codes % 16 == 0), "quantize: ld_col_codes must be >= M/2 and a multiple of 16 bytes");
   const bool do_row = row_codes != nullptr, do_col = col_codes != nullptr;
   ALTO_REQUIRE(x != nullptr, "quantize: x is NULL");
   ALTO_REQUIRE(dtype == ALTO_DT_BF16 || dtype == ALTO_DT_F32, "quantize: dtype %d is neither bf16 (0) nor f32 (1)", dtype);
@@ -417,6 +432,7 @@ extern "C" int alto_mxfp4_quantize(const void* x, int dtype, int64_t batch, int6
   p.x = x; p.ld_x = ld_x; p.bs_x = bs_x; p.M = (int)M; p.C = (int)C;
   p.rand = rand_bits; p.ld_r = ld_rand; p.bs_r = bs_rand;
   p.row_codes = row_codes; p.row_scales = row_scales; p.col_codes = col_codes; p.col_scales = col_scales;
+  p.ld_rc = ld_row_codes; p.ld_cc = ld_col_codes;
   p.sign_mask = 0;
   for (int k = 0; k < 32; ++k) { p.perm[k] = (uint8_t)k; p.perm_inv[k] = (uint8_t)k; }
   if (hadamard) {

@@ -179,7 +179,7 @@ class MXFP4GroupedGEMM(torch.autograd.Function):
             groups = groups_from_offsets(offsets)
         torch._check(M_buf % 32 == 0)
         x = inputs if inputs.is_contiguous() else inputs.contiguous()
-        a_q, a_s, a_qm, a_sm = quantize_rowcol(x, False, hadamard=hadamard_transform, clip_mode=clip_mode, use_uos=use_uos)
+        a_q, a_s, a_qm, a_sm = quantize_rowcol(x, False, hadamard=hadamard_transform, clip_mode=clip_mode, use_uos=use_uos, pad_codes=True)
         # weights: one pass gives the K-packed codes (forward) and the N-packed codes (dX)
         w = expert_weights if trans_weights else expert_weights.transpose(1, 2)   # logical [E, N, K]
         if w.stride(2) == 1:
@@ -206,7 +206,7 @@ class MXFP4GroupedGEMM(torch.autograd.Function):
         sr = bool(ctx.use_sr_grad)
         rand = rt.draw_rand_bits(go.shape, go.device) if sr else None
         go_q, go_s, go_qm, go_sm = quantize_rowcol(go, False, use_sr=sr, rand_bits=rand, hadamard=ctx.hadamard_transform,
-                                                   clip_mode=ctx.clip_mode, use_uos=ctx.use_uos)
+                                                   clip_mode=ctx.clip_mode, use_uos=ctx.use_uos, pad_codes=True)
         grad_inputs = grouped_forward(go_q, go_s, wq_kn, ws_kn, groups, False, True, ctx.original_dtype)
         grad_weights = grouped_dw(go_qm.transpose(0, 1), go_sm.transpose(0, 1), a_qm.transpose(0, 1), a_sm.transpose(0, 1),
                                   groups, ctx.num_experts, ctx.original_dtype, ctx.trans_weights,
@@ -219,7 +219,7 @@ def _quantize_experts(w: torch.Tensor, use_uos: bool):
     [E,C,R/2] and the same scales stored transposed [E,C/32,R/32] (each operand of a GEMM wants unit stride along its K)."""
     from .quantization import _prep, _quantize_call
     return cached_weight_quantisation(w, ("experts2d", bool(use_uos)),
-                                      lambda: _quantize_call(_prep(w), True, True, True, False, None, None, 0, use_uos))
+                                      lambda: _quantize_call(_prep(w), True, True, True, False, None, None, 0, use_uos, True))
 
 
 def mxfp4_grouped_gemm(inputs, expert_weights, expert_indices, *, trans_weights=True, use_2dblock_x=False, use_2dblock_w=True,

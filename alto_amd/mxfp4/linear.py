@@ -69,7 +69,7 @@ def cached_weight_quantisation(weight: torch.Tensor, tag, make):
 
 def _quantize_weight_2d(weight: torch.Tensor, use_uos: bool):
     """(w_q, w_s, w_qt, w_st) of a 2D-block quantisation, from the cache when the weight is unchanged."""
-    return cached_weight_quantisation(weight, ("linear2d", bool(use_uos)), lambda: quantize_rowcol(weight, True, use_uos=use_uos))
+    return cached_weight_quantisation(weight, ("linear2d", bool(use_uos)), lambda: quantize_rowcol(weight, True, use_uos=use_uos, pad_codes=True))
 
 
 def transpose_codes(codes: torch.Tensor) -> torch.Tensor:
@@ -187,7 +187,7 @@ class MXFP4LinearFunction(torch.autograd.Function):
 
         fuse_x = (not use_2dblock_x) and M % 32 == 0
         if fuse_x:
-            x_q, x_s, x_qm, x_sm = quantize_rowcol(x2, False, hadamard=hadamard_transform, clip_mode=clip_mode, use_uos=use_uos)
+            x_q, x_s, x_qm, x_sm = quantize_rowcol(x2, False, hadamard=hadamard_transform, clip_mode=clip_mode, use_uos=use_uos, pad_codes=True)
         else:
             x_q, x_s = convert_to_mxfp4(x2, axis=-1, is_2d_block=use_2dblock_x, use_uos=use_uos)
             if use_2dblock_x:
@@ -228,7 +228,7 @@ class MXFP4LinearFunction(torch.autograd.Function):
             go_qm, go_sm = go_q, go_s
         else:
             go_q, go_s, go_qm, go_sm = quantize_rowcol(go, False, use_sr=sr, rand_bits=rand, hadamard=ctx.hadamard_transform,
-                                                       clip_mode=ctx.clip_mode, use_uos=ctx.use_uos)
+                                                       clip_mode=ctx.clip_mode, use_uos=ctx.use_uos, pad_codes=True)
         # dgrad: reduction over N.  The saved weight operand is already packed along N (both layouts of a 2D-block
         # quantisation hold the same codes), so no k_pack=False repack is needed here.
         grad_inputs = blockwise_mxfp4_gemm(go_q, go_s, w_bwd, w_bwd_s, use_2dblock_a=ctx.use_2dblock_x,

@@ -39,17 +39,27 @@ def _signs_perm_ptrs(h: Optional[HadamardTransform]):
     return 1, h.signs.data_ptr(), (None if h.perm is None else h.perm.data_ptr())
 
 
+def _code_buffer(B: int, R: int, nbytes: int, dev, pad: bool) -> torch.Tensor:
+    """[B, R, nbytes] code tensor; with ``pad`` its rows start on 128-byte boundaries (a view over padded storage)."""
+    pitch = (nbytes + 127) // 128 * 128 if pad else nbytes
+    if pitch == nbytes:
+        return torch.empty((B, R, nbytes), dtype=torch.uint8, device=dev)
+    return torch.empty((B, R, pitch), dtype=torch.uint8, device=dev)[:, :, :nbytes]
+
+
 def _quantize_call(x3: torch.Tensor, want_row: bool, want_col: bool, is_2d: bool, use_sr: bool,
-                   rand3: Optional[torch.Tensor], hadamard: Optional[HadamardTransform], clip: int, use_uos: bool):
-    """x3: [B, M, C] with unit stride along C and uniform row / batch strides. Returns dense outputs (or None)."""
+                   rand3: Optional[torch.Tensor], hadamard: Optional[HadamardTransform], clip: int, use_uos: bool,
+                   pad_codes: bool = False):
+    """x3: [B, M, C] with unit stride along C and uniform row / batch strides. Returns the outputs (or None): dense, or
+    with ``pad_codes`` code tensors whose rows are padded to whole 128-byte cache lines (for GEMM operands)."""
     B, M, C = x3.shape
     dev = x3.device
     row_codes = row_scales = col_codes = col_scales = None
     if want_row:
-        row_codes = torch.empty((B, M, C // 2), dtype=torch.uint8, device=dev)
+        row_codes = _code_buffer(B, M, C // 2, dev, pad_codes)
         row_scales = torch.empty((B, M // 32, C // 32) if is_2d else (B, M, C // 32), dtype=torch.uint8, device=dev)
     if want_col:
-        col_codes = torch.empty((B, C, M // 2), dtype=torch.uint8, device=dev)
+        col_codes = _code_buffer(B, C, M // 2, dev, pad_codes)
         col_scales = torch.empty((B, C // 32, M // 32) if is_2d else (B, C, M // 32), dtype=torch.uint8, device=dev)
     had, sp, pp = _signs_perm_ptrs(hadamard)
     ld_x = x3.stride(1) if M > 1 else C
@@ -58,12 +68,13 @@ def _quantize_call(x3: torch.Tensor, want_row: bool, want_col: bool, is_2d: bool
     if use_sr:
         ld_r = rand3.stride(1) if M > 1 else C
         bs_r = rand3.stride(0) if B > 1 else M * ld_r
-    rc = rt.lib().alto_mxfp4_quantize(
+    rc = rt.lib().alto_mxfp4_quantize_pitched(
         x3.data_ptr(), rt.dtype_code(x3.dtype), B, M, C, ld_x, bs_x,
         rt.ptr(row_codes), rt.ptr(row_scales), rt.ptr(col_codes), rt.ptr(col_scales),
+        row_codes.stride(1) if want_row else 0, col_codes.stride(1) if want_col else 0,
         int(is_2d), rt.ROUND_SR if use_sr else rt.ROUND_RNE, rt.ptr(rand3), ld_r, bs_r,
         had, sp, pp, clip, int(use_uos), rt.stream_ptr(dev))
-    check(rc, "alto_mxfp4_quantize")
+    check(rc, "alto_mxfp4_quantize_pitched")
     return row_codes, row_scales, col_codes, col_scales
 
 
@@ -191,6 +202,7 @@ def quantize_rowcol(
     hadamard: Optional[HadamardTransform] = None,
     clip_mode: str = "none",
     use_uos: bool = False,
+    pad_codes: bool = False,
 ):
     """One pass over a 2D ``x [M, C]`` producing BOTH quantisations the linear layer needs.
 
@@ -213,7 +225,7 @@ def quantize_rowcol(
         assert rand_bits.shape == x.shape
         r3 = _as_i32(rand_bits)
         r3 = _batched_view(r3 if r3.stride(-1) == 1 and r3.stride(0) % 4 == 0 and r3.data_ptr() % 16 == 0 else r3.contiguous())
-    rc, rs, cc, cs = _quantize_call(x3, True, True, is_2d_block, use_sr, r3, hadamard, clip, use_uos)
+    rc, rs, cc, cs = _quantize_call(x3, True, True, is_2d_block, use_sr, r3, hadamard, clip, use_uos, pad_codes)
     return rc[0], rs[0], cc[0].transpose(0, 1), cs[0].transpose(0, 1)
 
 

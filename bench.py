@@ -105,7 +105,7 @@ class FusedGradQuant(Workload):
 
     def cpu_sample(self):
         import oracle as O
-        rows = 512
+        rows = 2048
         x = self.x[:rows].cpu()
         r = self.r[:rows].cpu()
         signs, perm = self.h.signs, self.h.perm.long()
@@ -184,7 +184,7 @@ class Gemm(Workload):
     def cpu_sample(self):
         import torch
         import oracle as O
-        rows = 256
+        rows = min(4096, self.M)   # about 10 s of host work per repetition at the Llama shapes
         aq, as_ = self.aq[:rows].cpu(), (self.as_[:rows // 32] if self.a_2d else self.as_[:rows]).cpu()
         bq, bs = self.bq.cpu(), self.bs.cpu()
 
@@ -212,11 +212,15 @@ class GroupedGemm(Workload):
         counts = torch.bincount(top, minlength=self.E)
         offs = torch.cat([torch.zeros(1, dtype=torch.int64, device=dev), counts.cumsum(0)]).to(torch.int32)
         self.groups = G.groups_from_offsets(offs)
+        # operands as the autograd function holds them: code rows padded to whole 128-byte cache lines (K/2 = 1440 bytes
+        # is not a multiple of 128), scales dense
+        from alto_amd.mxfp4.quantization import _prep, _quantize_call
         a = torch.randn(rows, self.K, device=dev, generator=gen).bfloat16()
-        self.aq, self.as_ = m.convert_to_mxfp4(a)
+        aq, as_, _, _ = _quantize_call(_prep(a), True, False, False, False, None, None, 0, False, True)
+        self.aq, self.as_ = aq[0], as_[0]
         del a
         w = (torch.randn(self.E, self.N, self.K, device=dev, generator=gen) * 0.02).bfloat16()
-        self.wq, self.ws = m.convert_to_mxfp4(w, is_2d_block=True)
+        self.wq, self.ws, _, _ = _quantize_call(_prep(w), True, False, True, False, None, None, 0, False, True)
         del w
         self.rows = rows
         self.work = 2.0 * rows * self.N * self.K

@@ -88,6 +88,19 @@ int alto_mxfp4_quantize(const void* x, int dtype, int64_t batch, int64_t M, int6
                         int clip_mode, int use_uos, void* stream);
 
 /*
+ * The same quantizer with a row pitch for the code outputs: row_codes[b][M][ld_row_codes] and
+ * col_codes[b][C][ld_col_codes] (bytes; 0 = dense, i.e. C/2 and M/2).  A GEMM operand whose rows start on
+ * 128-byte boundaries loads whole cache lines; the host layer pads K = 2880-like shapes this way for its own
+ * intermediate operands.  No counterpart in the reference (its outputs are always dense).
+ */
+int alto_mxfp4_quantize_pitched(const void* x, int dtype, int64_t batch, int64_t M, int64_t C, int64_t ld_x, int64_t bs_x,
+                                uint8_t* row_codes, uint8_t* row_scales, uint8_t* col_codes, uint8_t* col_scales,
+                                int64_t ld_row_codes, int64_t ld_col_codes,
+                                int is_2d, int rounding, const uint32_t* rand_bits, int64_t ld_rand, int64_t bs_rand,
+                                int hadamard, const int8_t* signs, const uint8_t* perm,
+                                int clip_mode, int use_uos, void* stream);
+
+/*
  * Standalone randomized Hadamard transform along M in blocks of 32 rows:
  *   y[32b + i][c] = cast((sum_j W[i][j] * fp32(x[32b + j][c])) / float32(sqrt(32)))
  * with W built from signs/perm as in alto_mxfp4_quantize (same summation order, so

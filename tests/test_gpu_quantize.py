@@ -218,3 +218,14 @@ def test_edge_cases(m):
         m.convert_to_mxfp4(torch.zeros(32, 48, device=DEV))
     with pytest.raises(NotImplementedError):
         m.convert_to_mxfp4(torch.zeros(32, 64, device=DEV), clip_mode="dynamic")
+
+
+def test_padded_code_rows_hold_the_same_bytes(m):
+    """Code outputs with rows padded to whole cache lines (what the autograd functions keep as GEMM operands) are views
+    with the dense results' bytes; shape with C/2 and M/2 not multiples of 128."""
+    x = randn_outliers((96, 2880), torch.bfloat16, seed=91).to(DEV)
+    dense = m.quantize_rowcol(x, False)
+    padded = m.quantize_rowcol(x, False, pad_codes=True)
+    assert padded[0].stride(0) == 1536 and padded[2].transpose(0, 1).stride(0) == 128
+    for d, p_ in zip(dense, padded):
+        assert d.shape == p_.shape and torch.equal(d, p_)
