@@ -18,7 +18,7 @@ import torch
 from . import _runtime as rt
 from .._lib import check
 from .hadamard import HadamardFactory, HadamardTransform
-from .linear import cached_weight_quantisation, transpose_codes, unwrap_weight_wrapper
+from .linear import _wgrad_scale, cached_weight_quantisation, transpose_codes, unwrap_weight_wrapper
 from .quantization import convert_to_mxfp4, quantize_rowcol
 
 ALIGN_SIZE_M = 128
@@ -161,8 +161,6 @@ class MXFP4GroupedGEMM(torch.autograd.Function):
     def forward(ctx, inputs, expert_weights, expert_indices, trans_weights=True, use_2dblock_x=False, use_2dblock_w=True,
                 use_sr_grad=False, use_dge=False, clip_mode="none", use_macro_block_scaling=False,
                 hadamard_transform: Optional[HadamardTransform] = None, use_uos: bool = False, offsets: Optional[torch.Tensor] = None):
-        if use_dge:
-            raise NotImplementedError("use_dge is not part of the MXFP4 hot path this build covers")
         assert not use_macro_block_scaling, "Macro block scaling is not supported in real MXFP4 kernels"
         if use_2dblock_x or not use_2dblock_w:
             raise NotImplementedError("grouped MXFP4 GEMM: only use_2dblock_x=False, use_2dblock_w=True is implemented")
@@ -196,6 +194,7 @@ class MXFP4GroupedGEMM(torch.autograd.Function):
         ctx.clip_mode = clip_mode
         ctx.use_uos = use_uos
         ctx.num_experts = E
+        ctx.use_dge = bool(use_dge)
         return out
 
     @staticmethod
@@ -210,7 +209,7 @@ class MXFP4GroupedGEMM(torch.autograd.Function):
         grad_inputs = grouped_forward(go_q, go_s, wq_kn, ws_kn, groups, False, True, ctx.original_dtype)
         grad_weights = grouped_dw(go_qm.transpose(0, 1), go_sm.transpose(0, 1), a_qm.transpose(0, 1), a_sm.transpose(0, 1),
                                   groups, ctx.num_experts, ctx.original_dtype, ctx.trans_weights,
-                                  16.0 / 9.0 if ctx.clip_mode == "static" else 1.0)
+                                  _wgrad_scale(ctx.clip_mode, ctx.use_dge))
         return (grad_inputs, grad_weights) + (None,) * 11
 
 

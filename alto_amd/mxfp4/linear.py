@@ -11,6 +11,7 @@ import torch
 
 from . import _runtime as rt
 from .._lib import check
+from .dge import DGE_FACTOR
 from .hadamard import HadamardFactory, HadamardTransform
 from .quantization import BLOCK_SIZE_DEFAULT, convert_to_mxfp4, quantize_rowcol
 
@@ -163,6 +164,13 @@ def blockwise_mxfp4_gemm(
     return c
 
 
+def _wgrad_scale(clip_mode: str, use_dge: bool) -> float:
+    """Constant multiplier of dW: 16/9 undoes the two 3/4 clips (mxfp_linear.py:543-544), the estimator's factor follows
+    mxfp_linear.py:549-568 (constant on the E2M1 grid, see dge.py)."""
+    s = 16.0 / 9.0 if clip_mode == "static" else 1.0
+    return s * DGE_FACTOR if use_dge else s
+
+
 class MXFP4LinearFunction(torch.autograd.Function):
     """``y = x @ W^T`` with MXFP4 operands in forward and in both backward GEMMs (mxfp_linear.py:258-570).
 
@@ -176,8 +184,6 @@ class MXFP4LinearFunction(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x, weight, use_2dblock_x, use_2dblock_w, use_sr_grad, use_dge, clip_mode,
                 use_macro_block_scaling, hadamard_transform: Optional[HadamardTransform] = None, use_uos: bool = False):
-        if use_dge:
-            raise NotImplementedError("use_dge is not part of the MXFP4 hot path this build covers")
         assert not use_macro_block_scaling, "Macro block scaling is not supported in real MXFP4 kernels"
         weight = unwrap_weight_wrapper(weight)
         original_shape = x.shape
@@ -214,6 +220,7 @@ class MXFP4LinearFunction(torch.autograd.Function):
         ctx.hadamard_transform = hadamard_transform
         ctx.clip_mode = clip_mode
         ctx.use_uos = use_uos
+        ctx.use_dge = bool(use_dge)
         return y.view(*original_shape[:-1], -1)
 
     @staticmethod
@@ -238,7 +245,7 @@ class MXFP4LinearFunction(torch.autograd.Function):
                                             use_2dblock_b=ctx.use_2dblock_x, trans_a=True,
                                             k_pack_a=not ctx.use_2dblock_x, k_pack_b=not ctx.use_2dblock_x,
                                             output_dtype=ctx.original_dtype,
-                                            out_scale=16.0 / 9.0 if ctx.clip_mode == "static" else 1.0)
+                                            out_scale=_wgrad_scale(ctx.clip_mode, ctx.use_dge))
         return grad_inputs.view(*original_shape[:-1], -1), grad_weights, None, None, None, None, None, None, None, None
 
 

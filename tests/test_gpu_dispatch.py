@@ -124,3 +124,42 @@ def test_weight_cache_reuses_until_weight_changes(m):
         assert torch.equal(y3, m._to_mxfp4_then_scaled_mm(x, w, *args))
     finally:
         m.enable_weight_cache(False)
+
+
+@pytest.mark.parametrize("clip_mode", ["none", "static"])
+def test_dge_scales_the_weight_gradient(m, clip_mode):
+    """use_dge multiplies dW by dge_bwd at the quantised weight's grid values (mxfp_linear.py:549-568), which is the
+    constant fp32(1/5) on the E2M1 grid; dX and the forward result are untouched.  fp32 tensors: the reference's
+    searchsorted needs the fp32 dtype of its break points."""
+    x = randn_outliers((128, 256), torch.float32, seed=11).to(DEV)
+    w = (randn_outliers((192, 256), torch.float32, seed=12) * 0.02).to(DEV)
+    go = randn_outliers((128, 192), torch.float32, seed=13).to(DEV) / 1000
+    grads = {}
+    for dge in (False, True):
+        xi, wi = x.clone().requires_grad_(True), w.clone().requires_grad_(True)
+        y = m._to_mxfp4_then_scaled_mm(xi, wi, False, True, False, dge, clip_mode, False)
+        y.backward(go)
+        grads[dge] = (y.detach(), xi.grad, wi.grad)
+    assert torch.equal(grads[True][0], grads[False][0])
+    assert torch.equal(grads[True][1], grads[False][1])
+    f = torch.tensor(0.2, dtype=torch.float32)
+    # one rounding in the GEMM epilogue (acc * (16/9 * 0.2)) versus the reference's two: within a few fp32 ulps
+    torch.testing.assert_close(grads[True][2], grads[False][2] * f, rtol=4e-7, atol=0)
+    assert grads[False][2].abs().max() > 0
+
+
+def test_dge_grouped_weight_gradient(m):
+    E, N, K, M = 2, 128, 256, 256
+    x = randn_outliers((M, K), torch.float32, seed=21).to(DEV)
+    w = (randn_outliers((E, N, K), torch.float32, seed=22) * 0.02).to(DEV)
+    go = randn_outliers((M, N), torch.float32, seed=23).to(DEV) / 1000
+    idx = torch.arange(M, device=DEV, dtype=torch.int32) // 128
+    grads = {}
+    for dge in (False, True):
+        xi, wi = x.clone().requires_grad_(True), w.clone().requires_grad_(True)
+        y = m.mxfp4_grouped_gemm(xi, wi, idx, use_dge=dge)
+        y.backward(go)
+        grads[dge] = (xi.grad, wi.grad)
+    assert torch.equal(grads[True][0], grads[False][0])
+    torch.testing.assert_close(grads[True][1], grads[False][1] * 0.2, rtol=4e-7, atol=0)
+    assert grads[False][1].abs().max() > 0

@@ -123,3 +123,18 @@ def test_swap_params_wraps_weights_not_biases():
     assert type(model[2].bias.data) is torch.Tensor
     with pytest.raises(ValueError):
         m.swap_params(model, config=None)
+
+
+def test_dge_factor_is_one_fifth_on_the_e2m1_grid():
+    """dge_bwd (alto/kernels/dge/dge.py:80-93) at a break point: |x - mid| = half_delta, so the factor is 1/k."""
+    import numpy as np
+    from alto_amd.mxfp4.dge import DGE_FACTOR, DGE_K, dge_bwd_e2m1_grid
+    t = dge_bwd_e2m1_grid()
+    assert t.shape == (16,) and t.dtype == np.float32
+    assert np.float32(DGE_FACTOR) == np.float32(1.0 / DGE_K)
+    assert np.all(np.abs(t - np.float32(0.2)) <= 2 * np.spacing(np.float32(0.2)))
+    # an off-grid point does not give 1/k: the constant is a property of the grid, not of the formula
+    bp = np.array([1.0, 1.5], dtype=np.float32)
+    half, mid, x = np.float32(0.25), np.float32(1.25), np.float32(1.3)
+    off = half ** np.float32(0.8) * np.abs(x - mid) ** np.float32(-0.8) / np.float32(5)
+    assert abs(off - 0.2) > 0.1
