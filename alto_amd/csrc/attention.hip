@@ -1,0 +1,231 @@
+// MXFP4 flash-attention forward for gfx950: S = Q K^T and O = P V both on v_mfma_scale_f32_32x32x64_f8f6f4, with the
+// probabilities re-quantised to MXFP4 in registers and the row sums taken from the SAME quantised probabilities
+// (the recurrence of alto/kernels/fp4/mxfp4/triton_flash_attention_mxfp4.py:168-400,640-890, key blocks of 64).
+//
+// One wave owns 32 query rows of one head.  The MFMA is issued as (first = rows that land in registers, second = rows
+// that land in lanes): S tiles and O tiles keep the query row in the lane (lane % 32) and spread keys / value columns
+// over the 16 accumulator registers, so the per-row softmax state (running max, rescale factor) is one scalar per lane
+// and the only cross-lane traffic is between the two lanes (l, l ^ 32) that share a row.
+#include "common.h"
+
+namespace alto {
+
+struct AttnArgs {
+  const uint8_t* q;  const uint8_t* qs;    // [B, Hq, Sq, D/2],  [B, Hq, Sq/32, D/32]
+  const uint8_t* k;  const uint8_t* ks;    // [B, Hk, Sk, D/2],  [B, Hk, Sk/32, D/32]
+  const uint8_t* vt; const uint8_t* vs;    // [B, Hk, Dv, Sk/2] packed along keys, [B, Hk, Dv/32, Sk/32]
+  void* out; float* lse;                   // [B, Hq, Sq, Dv] bf16, [B, Hq, Sq] fp32
+  int Hq, Hk, Sq, Sk;
+  float sm_scale;
+  int causal;
+};
+
+constexpr float ATTN_RCP_LN2 = 1.4426950408889634f;
+constexpr float ATTN_LN2 = 0.6931471824645996f;
+
+__device__ __forceinline__ v8i_t frag16(const uint8_t* p) {
+  const uint4 w = *reinterpret_cast<const uint4*>(p);
+  return v8i_t{(int)w.x, (int)w.y, (int)w.z, (int)w.w, 0, 0, 0, 0};
+}
+__device__ __forceinline__ float xor32(float v) { return __shfl_xor(v, 32, 64); }
+__device__ __forceinline__ uint32_t xor32(uint32_t v) { return (uint32_t)__shfl_xor((int)v, 32, 64); }
+
+// NK = D / 64 (MFMA K steps of Q K^T), ND = Dv / 32 (output tiles).
+template <int NK, int ND>
+__global__ __launch_bounds__(256) void attn_fwd_kernel(AttnArgs a) {
+  constexpr int D = NK * 64, DV = ND * 32;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r = lane & 31, h = lane >> 5;
+  const int q0 = (blockIdx.x * 4 + wave) * 32;
+  if (q0 >= a.Sq) return;                         // no workgroup-wide synchronisation below
+  const int hq = blockIdx.y, b = blockIdx.z;
+  const int hk = hq / (a.Hq / a.Hk);
+  const int64_t bhq = (int64_t)b * a.Hq + hq, bhk = (int64_t)b * a.Hk + hk;
+  const int qrow = q0 + r;
+  const int shift = a.Sk - a.Sq;                  // causal mask is aligned to the bottom-right corner
+
+  // ---- Q pieces: row qrow, K step ks, half h -> 16 bytes; one scale byte per (32-row block, 32-column block)
+  v8i_t qf[NK];
+  int qsc[NK];
+#pragma unroll
+  for (int s = 0; s < NK; ++s) {
+    qf[s] = frag16(a.q + (bhq * a.Sq + qrow) * (D / 2) + s * 32 + h * 16);
+    qsc[s] = a.qs[(bhq * (a.Sq / 32) + q0 / 32) * (D / 32) + 2 * s + h];
+  }
+
+  v16f_t acc_o[ND], acc_l;
+#pragma unroll
+  for (int d = 0; d < ND; ++d)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc_o[d][v] = 0.0f;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) acc_l[v] = 0.0f;
+  float m_i = -__builtin_inff();
+
+  // byte selectors that interleave my 4-key groups with the partner lane's into natural key order
+  const uint32_t sel_lo = h ? 0x01000504u : 0x05040100u;
+  const uint32_t sel_hi = h ? 0x03020706u : 0x07060302u;
+  const v8i_t ones = v8i_t{0x22222222, 0x22222222, 0x22222222, 0x22222222, 0, 0, 0, 0};   // E2M1 code 2 = 1.0
+
+  int nblk = a.Sk / 64;
+  if (a.causal) {
+    const int lim = (q0 + 32 + shift + 63) / 64;  // blocks holding a key some row of this wave may see
+    nblk = lim < nblk ? lim : nblk;
+  }
+
+  for (int kb = 0; kb < nblk; ++kb) {
+    const int key0 = kb * 64;
+    // ---- S = Q K^T for two 32-key tiles
+    v16f_t S[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) S[t][v] = 0.0f;
+      const uint8_t* krow = a.k + (bhk * a.Sk + key0 + 32 * t + r) * (D / 2) + h * 16;
+      const uint8_t* ksrow = a.ks + (bhk * (a.Sk / 32) + key0 / 32 + t) * (D / 32) + h;
+#pragma unroll
+      for (int s = 0; s < NK; ++s) {
+        const v8i_t kf = frag16(krow + s * 32);
+        const int ksc = ksrow[2 * s];
+        S[t] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(kf, qf[s], S[t], 4, 4, 0, ksc, 0, qsc[s]);
+      }
+    }
+    // ---- scale, mask, running max
+    const bool diag = a.causal && (key0 + 63 > q0 + shift);
+    float mx = -__builtin_inff();
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        float s = S[t][v] * a.sm_scale;
+        if (diag) {
+          const int key = key0 + 32 * t + 8 * (v >> 2) + 4 * h + (v & 3);
+          if (key > qrow + shift) s = -__builtin_inff();
+        }
+        S[t][v] = s;
+        mx = fmaxf(mx, s);
+      }
+    mx = fmaxf(mx, xor32(mx));
+    const float m_new = fmaxf(m_i, mx);
+    const float alpha = __builtin_amdgcn_exp2f((m_i - m_new) * ATTN_RCP_LN2);
+    m_i = m_new;
+
+    // ---- probabilities, one E8M0 scale per (row, 32 keys), E2M1 codes (round to nearest even)
+    uint32_t c[2][2];
+    int psc[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      float p[16];
+      float am = 0.0f;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        p[v] = __builtin_amdgcn_exp2f((S[t][v] - m_new) * ATTN_RCP_LN2);
+        am = fmaxf(am, p[v]);
+      }
+      am = fmaxf(am, xor32(am));
+      const uint32_t e = e8m0_from_f32_bits(f2u(am));
+      psc[t] = (int)e;
+      const float scale_f = u2f(e << 23);
+#pragma unroll
+      for (int w = 0; w < 2; ++w) {
+        uint32_t o = 0;
+        o = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(o, p[8 * w + 0], p[8 * w + 1], scale_f, 0);
+        o = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(o, p[8 * w + 2], p[8 * w + 3], scale_f, 1);
+        o = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(o, p[8 * w + 4], p[8 * w + 5], scale_f, 2);
+        o = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(o, p[8 * w + 6], p[8 * w + 7], scale_f, 3);
+        c[t][w] = o;
+      }
+    }
+    // Lane (r, h) multiplies tile h of this block: it keeps its half of tile h and gets the other half from lane
+    // (r, 1 - h), which in turn needs this lane's half of tile 1 - h.
+    uint32_t keep[2], recv[2];
+#pragma unroll
+    for (int w = 0; w < 2; ++w) {
+      keep[w] = h ? c[1][w] : c[0][w];
+      recv[w] = xor32(h ? c[0][w] : c[1][w]);
+    }
+    const v8i_t pf = v8i_t{(int)__builtin_amdgcn_perm(recv[0], keep[0], sel_lo), (int)__builtin_amdgcn_perm(recv[0], keep[0], sel_hi),
+                           (int)__builtin_amdgcn_perm(recv[1], keep[1], sel_lo), (int)__builtin_amdgcn_perm(recv[1], keep[1], sel_hi),
+                           0, 0, 0, 0};
+    const int pscale = h ? psc[1] : psc[0];
+
+    // ---- row sums of the quantised probabilities (a column of ones) and O += P V
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc_l[v] *= alpha;
+    acc_l = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ones, pf, acc_l, 4, 4, 0, 127, 0, pscale);
+#pragma unroll
+    for (int d = 0; d < ND; ++d) {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc_o[d][v] *= alpha;
+      const v8i_t vf = frag16(a.vt + ((bhk * DV + 32 * d + r) * (int64_t)(a.Sk / 2)) + (key0 + 32 * h) / 2);
+      const int vsc = a.vs[(bhk * (DV / 32) + d) * (a.Sk / 32) + key0 / 32 + h];
+      acc_o[d] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(vf, pf, acc_o[d], 4, 4, 0, vsc, 0, pscale);
+    }
+  }
+
+  // ---- O = acc / l, bf16; log-sum-exp
+  const float l = acc_l[0];
+  const float rl = 1.0f / l;
+  __bf16* orow = reinterpret_cast<__bf16*>(a.out) + (bhq * a.Sq + qrow) * DV;
+#pragma unroll
+  for (int d = 0; d < ND; ++d)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      bf16x2_t lo, hi;
+      lo[0] = (__bf16)(acc_o[d][4 * g + 0] * rl);
+      lo[1] = (__bf16)(acc_o[d][4 * g + 1] * rl);
+      hi[0] = (__bf16)(acc_o[d][4 * g + 2] * rl);
+      hi[1] = (__bf16)(acc_o[d][4 * g + 3] * rl);
+      uint2 w;
+      w.x = __builtin_bit_cast(uint32_t, lo);
+      w.y = __builtin_bit_cast(uint32_t, hi);
+      *reinterpret_cast<uint2*>(orow + 32 * d + 8 * g + 4 * h) = w;
+    }
+  if (h == 0) a.lse[bhq * a.Sq + qrow] = (m_i * ATTN_RCP_LN2 + log2f(l)) * ATTN_LN2;
+}
+
+template <int NK, int ND>
+static int launch_attn(const AttnArgs& a, int B, hipStream_t st) {
+  dim3 grid((unsigned)((a.Sq + 127) / 128), (unsigned)a.Hq, (unsigned)B);
+  hipLaunchKernelGGL((attn_fwd_kernel<NK, ND>), grid, dim3(256), 0, st, a);
+  return check_launch("attention_fwd");
+}
+
+template <int NK>
+static int launch_attn_nd(const AttnArgs& a, int B, int Dv, hipStream_t st) {
+  switch (Dv) {
+    case 64: return launch_attn<NK, 2>(a, B, st);
+    case 128: return launch_attn<NK, 4>(a, B, st);
+  }
+  return ALTO_MXFP4_EINVAL;
+}
+
+}  // namespace alto
+
+extern "C" int alto_mxfp4_attention_fwd(const void* q_codes, const void* q_scales, const void* k_codes, const void* k_scales,
+                                        const void* vt_codes, const void* v_scales, void* out, float* lse, int64_t B, int64_t Hq,
+                                        int64_t Hk, int64_t Sq, int64_t Sk, int64_t D, int64_t Dv, float sm_scale, int causal,
+                                        void* stream) {
+  using namespace alto;
+  ALTO_REQUIRE(q_codes && q_scales && k_codes && k_scales && vt_codes && v_scales && out && lse, "attention_fwd: null pointer");
+  ALTO_REQUIRE(B > 0 && Hq > 0 && Hk > 0 && Hq % Hk == 0, "attention_fwd: Hq=%lld must be a positive multiple of Hk=%lld", (long long)Hq, (long long)Hk);
+  ALTO_REQUIRE(Sq > 0 && Sq % 32 == 0, "attention_fwd: Sq=%lld must be a positive multiple of 32", (long long)Sq);
+  ALTO_REQUIRE(Sk > 0 && Sk % 64 == 0, "attention_fwd: Sk=%lld must be a positive multiple of 64", (long long)Sk);
+  ALTO_REQUIRE(D == 64 || D == 128 || D == 192 || D == 256, "attention_fwd: head dim D=%lld must be 64, 128, 192 or 256", (long long)D);
+  ALTO_REQUIRE(Dv == 64 || Dv == 128, "attention_fwd: value dim Dv=%lld must be 64 or 128", (long long)Dv);
+  ALTO_REQUIRE(!causal || Sq <= Sk, "attention_fwd: causal attention needs Sq <= Sk (got %lld > %lld)", (long long)Sq, (long long)Sk);
+  ALTO_REQUIRE(B <= 65535 && Hq <= 65535, "attention_fwd: B and Hq must fit a grid dimension");
+  ALTO_REQUIRE(B * Hq * Sq * (D > Dv ? D : Dv) < (1ll << 40), "attention_fwd: tensor too large");
+  ALTO_REQUIRE(((uintptr_t)q_codes | (uintptr_t)k_codes | (uintptr_t)vt_codes) % 16 == 0 && (uintptr_t)out % 8 == 0,
+               "attention_fwd: code pointers must be 16-byte aligned, out 8-byte aligned");
+  AttnArgs a{(const uint8_t*)q_codes, (const uint8_t*)q_scales, (const uint8_t*)k_codes, (const uint8_t*)k_scales,
+             (const uint8_t*)vt_codes, (const uint8_t*)v_scales, out, lse, (int)Hq, (int)Hk, (int)Sq, (int)Sk, sm_scale, causal ? 1 : 0};
+  hipStream_t st = (hipStream_t)stream;
+  switch (D) {
+    case 64: return launch_attn_nd<1>(a, (int)B, (int)Dv, st);
+    case 128: return launch_attn_nd<2>(a, (int)B, (int)Dv, st);
+    case 192: return launch_attn_nd<3>(a, (int)B, (int)Dv, st);
+    case 256: return launch_attn_nd<4>(a, (int)B, (int)Dv, st);
+  }
+  return ALTO_MXFP4_EINVAL;
+}

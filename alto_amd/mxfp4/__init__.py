@@ -1,4 +1,5 @@
 """Entry points of the MXFP4 hot path, named as in ``alto/kernels/fp4/mxfp4/__init__.py:5-26``."""
+from .attention import LPScaledDotProductAttention, attention_mxfp4_forward, quantize_qkv, triton_attention_mxfp4
 from .config import TrainingOpConfig
 from .grouped_gemm import (ALIGN_SIZE_M, MXFP4GroupedGEMM, _quantize_then_mxfp_scaled_grouped_mm,
                            create_indices_from_offsets_nosync, mxfp4_grouped_gemm, mxfp4_grouped_gemm_backward_inputs,
@@ -41,4 +42,8 @@ __all__ = (
     "weight_cache_stats",
     "quantize_dequantize",
     "_make_qdq_fn_for",
+    "triton_attention_mxfp4",
+    "attention_mxfp4_forward",
+    "quantize_qkv",
+    "LPScaledDotProductAttention",
 )

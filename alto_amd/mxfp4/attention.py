@@ -1,0 +1,109 @@
+"""MXFP4 flash-attention forward, named as in ``alto/kernels/fp4/mxfp4/triton_flash_attention_mxfp4.py``.
+
+``triton_attention_mxfp4`` keeps the reference's name and argument list (:1206-1239) so that
+``alto/kernels/dispatch/attention.py:22`` can point at it; here it quantises Q, K, V with the fused HIP quantizer
+(2D blocks along the head dim, :1105-1107; V also packed along the keys by the same pass) and runs one HIP kernel.
+Like the reference (:1143-1145) it has no backward.  Options outside the path ALTO's dispatch layer uses
+(``alto/kernels/dispatch/attention.py:61-77``: layout "bhsd", no bias, no alibi, no dropout, fixed lengths) raise.
+"""
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+
+from . import _runtime as rt
+from .._lib import check
+from .config import TrainingOpConfig
+from .quantization import _prep, _quantize_call
+
+
+def attention_mxfp4_forward(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, q_scale: torch.Tensor, k_scale: torch.Tensor,
+                            v_scale: torch.Tensor, sm_scale: float, causal: bool) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Pre-quantised operands -> (out bf16 [B,Hq,Sq,Dv], lse fp32 [B,Hq,Sq]).
+
+    q [B,Hq,Sq,D/2], q_scale [B,Hq,Sq/32,D/32]; k [B,Hk,Sk,D/2], k_scale [B,Hk,Sk/32,D/32]; v packed along the keys:
+    [B,Hk,Dv,Sk/2] with v_scale [B,Hk,Dv/32,Sk/32] (the reference's kernel takes V packed along Dv and unpacks it inside
+    ``tl.dot_scaled(..., rhs_k_pack=False)``, :393; same codes, other byte order).
+    """
+    rt.require_gpu(q, k, v, q_scale, k_scale, v_scale)
+    for t in (q, k, v, q_scale, k_scale, v_scale):
+        assert t.is_contiguous() and t.dtype == torch.uint8
+    B, Hq, Sq, D = q.shape[0], q.shape[1], q.shape[2], q.shape[3] * 2
+    Hk, Sk = k.shape[1], k.shape[2]
+    Dv = v.shape[2]
+    assert k.shape == (B, Hk, Sk, D // 2) and v.shape == (B, Hk, Dv, Sk // 2)
+    assert q_scale.shape == (B, Hq, Sq // 32, D // 32) and k_scale.shape == (B, Hk, Sk // 32, D // 32)
+    assert v_scale.shape == (B, Hk, Dv // 32, Sk // 32)
+    out = torch.empty((B, Hq, Sq, Dv), dtype=torch.bfloat16, device=q.device)
+    lse = torch.empty((B, Hq, Sq), dtype=torch.float32, device=q.device)
+    check(rt.lib().alto_mxfp4_attention_fwd(q.data_ptr(), q_scale.data_ptr(), k.data_ptr(), k_scale.data_ptr(), v.data_ptr(),
+                                            v_scale.data_ptr(), out.data_ptr(), lse.data_ptr(), B, Hq, Hk, Sq, Sk, D, Dv,
+                                            float(sm_scale), int(bool(causal)), rt.stream_ptr(q.device)), "alto_mxfp4_attention_fwd")
+    return out, lse
+
+
+def quantize_qkv(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor):
+    """bf16/fp32 [B,H,S,D] tensors -> (q, q_scale, k, k_scale, v packed along keys, v_scale): three quantizer launches."""
+    def rows(t):
+        t3 = _prep(t.reshape(-1, t.shape[-2], t.shape[-1]))
+        codes, scales, _, _ = _quantize_call(t3, True, False, True, False, None, None, 0, False)
+        return codes.view(*t.shape[:-1], t.shape[-1] // 2), scales.view(*t.shape[:-2], t.shape[-2] // 32, t.shape[-1] // 32)
+
+    def cols(t):
+        t3 = _prep(t.reshape(-1, t.shape[-2], t.shape[-1]))
+        _, _, codes, scales = _quantize_call(t3, False, True, True, False, None, None, 0, False)
+        return codes.view(*t.shape[:-2], t.shape[-1], t.shape[-2] // 2), scales.view(*t.shape[:-2], t.shape[-1] // 32, t.shape[-2] // 32)
+
+    qq, qs = rows(q)
+    kq, ks = rows(k)
+    vq, vs = cols(v)
+    return qq, qs, kq, ks, vq, vs
+
+
+def triton_attention_mxfp4(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, alibi_slopes: Optional[torch.Tensor] = None,
+                           bias: Optional[torch.Tensor] = None, sm_scale: Optional[float] = None, dropout_p: float = 0.0,
+                           cu_seqlens_q=0, cu_seqlens_k=0, max_seqlens_q: Optional[int] = None, max_seqlens_k: Optional[int] = None,
+                           causal: bool = True, return_scores: bool = False, use_exp2: bool = True, layout: str = "bhsd"):
+    """(q, k, v) [B,H,S,D] -> (out bf16, softmax_lse fp32, exp_scores placeholder), as :1206-1239.
+
+    ``use_exp2`` is accepted either way: both settings evaluate exp(x) as exp2(x * log2 e) on the GPU's exp unit.
+    """
+    if layout != "bhsd":
+        raise NotImplementedError(f"layout {layout!r}: only 'bhsd' is implemented (the layout ALTO's dispatch layer passes)")
+    if alibi_slopes is not None or bias is not None:
+        raise NotImplementedError("alibi slopes and bias are not implemented")
+    if dropout_p != 0.0:
+        raise NotImplementedError("dropout is not implemented (the reference's own dropout is a no-op after PNQ, :357-360)")
+    if return_scores:
+        raise NotImplementedError("return_scores is a debugging output of the reference and is not implemented")
+    rt.require_gpu(q, k, v)
+    assert q.dim() == 4 and k.dim() == 4 and v.dim() == 4
+    assert max_seqlens_q in (None, q.shape[2]) and max_seqlens_k in (None, k.shape[2]), "variable lengths are not implemented"
+    if sm_scale is None:
+        sm_scale = q.shape[-1] ** -0.5
+    qq, qs, kq, ks, vq, vs = quantize_qkv(q, k, v)
+    out, lse = attention_mxfp4_forward(qq, kq, vq, qs, ks, vs, sm_scale=sm_scale, causal=causal)
+    return out, lse, torch.empty([], device=q.device, dtype=torch.float32)
+
+
+class LPScaledDotProductAttention(torch.nn.Module):
+    """Module form used by ALTO's model converter (``alto/kernels/dispatch/attention.py:14-80``): inputs [B, L, N, H]."""
+
+    def __init__(self, config: TrainingOpConfig):
+        super().__init__()
+        if not (isinstance(config, TrainingOpConfig) and config.precision == "mxfp4"):
+            raise ValueError(f"Unsupported SDPA config: {config}")
+        self.config = config
+
+    def forward(self, q_BLNH, k_BLNH, v_BLNH, *, attention_masks=None, scale: Optional[float] = None, enable_gqa: bool = False,
+                is_causal: bool = True, **kwargs):
+        if attention_masks is not None:
+            raise ValueError("ScaledDotProductAttention does not support attention_masks; it only supports causal/non-causal "
+                             "attention via is_causal.")
+        q, k, v = (t.transpose(1, 2).contiguous() for t in (q_BLNH, k_BLNH, v_BLNH))
+        assert q.shape[0] == k.shape[0] == v.shape[0] and k.shape[1] == v.shape[1]
+        assert q.shape[3] == k.shape[3] and k.shape[2] == v.shape[2]
+        sm_scale = q.shape[3] ** -0.5 if scale is None else scale
+        o = triton_attention_mxfp4(q, k, v, sm_scale=sm_scale, causal=is_causal, max_seqlens_q=q.shape[2], max_seqlens_k=k.shape[2])[0]
+        return o.transpose(1, 2)

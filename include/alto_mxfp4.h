@@ -198,6 +198,24 @@ int alto_mxfp4_qdq(const void* x, int dtype, int64_t batch, int64_t M, int64_t C
                    void* y, int64_t ld_y, int64_t bs_y, int is_2d, int use_uos, void* stream);
 
 /*
+ * MXFP4 flash-attention forward (alto/kernels/fp4/mxfp4/triton_flash_attention_mxfp4.py:425-897, launched at :1031-1080
+ * with BLOCK_N = 64, layout "bhsd", no bias / alibi / dropout / varlen): per key block of 64,
+ *   S = (Q K^T) * sm_scale (FP4 x FP4, 2D-block scales), causal mask aligned bottom-right, m = running row max,
+ *   P = exp2((S - m) * log2(e)) quantised to MXFP4 with one E8M0 scale per (row, 32 keys), round to nearest even,
+ *   l = l * alpha + rowsum(dequantised P),  O = O * alpha + P V   (alpha = exp2((m_old - m) * log2(e))),
+ * out = O / l as bf16 [B][Hq][Sq][Dv], lse = m + ln(l) as f32 [B][Hq][Sq].
+ * q_codes [B][Hq][Sq][D/2], q_scales [B][Hq][Sq/32][D/32]; k_codes [B][Hk][Sk][D/2], k_scales [B][Hk][Sk/32][D/32]:
+ * 2D-block quantisations of Q and K along D (mxfp_quantization.py:410-484, is_2d_block=True).  V is the same 2D-block
+ * quantisation of [Sk][Dv], handed over packed along the keys: vt_codes [B][Hk][Dv][Sk/2], v_scales [B][Hk][Dv/32][Sk/32]
+ * (the column outputs of alto_mxfp4_quantize).  Hq % Hk == 0 (grouped-query heads), D in {64,128,192,256},
+ * Dv in {64,128}, Sq % 32 == 0, Sk % 64 == 0, causal needs Sq <= Sk.  All tensors dense.
+ */
+int alto_mxfp4_attention_fwd(const void* q_codes, const void* q_scales, const void* k_codes, const void* k_scales,
+                             const void* vt_codes, const void* v_scales, void* out, float* lse, int64_t B, int64_t Hq,
+                             int64_t Hk, int64_t Sq, int64_t Sk, int64_t D, int64_t Dv, float sm_scale, int causal,
+                             void* stream);
+
+/*
  * Diagnostic, no counterpart in the reference: a register-only loop of FP4 scaled-MFMA instructions
  * (8 per iteration and wave, 8 waves per workgroup, `workgroups` workgroups; 2*32*32*64 FLOP each),
  * with constant (random_operands = 0) or pseudo-random FP4 operands.  bench.py times it to report

@@ -1,0 +1,133 @@
+"""HIP MXFP4 flash attention (through the C ABI) against the CPU model of
+alto/kernels/fp4/mxfp4/triton_flash_attention_mxfp4.py.
+
+Tolerance: Q/K/V operands are compared bit for bit; the output is floating point and passes through v_exp_f32 on the GPU
+and libm on the CPU, so a probability can land on the other side of an E2M1 rounding boundary now and then.  Bound used:
+relative L2 error <= 2e-3 of the bf16 output (observed: 0 to 2e-8), log-sum-exp within 1e-4 absolute.
+"""
+import pytest
+import torch
+
+from oracle import mxfp4_oracle as O
+from oracle.attention_oracle import attention_fp32_ref, attention_fwd_ref
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+REL_L2 = 2e-3
+
+
+@pytest.fixture(scope="module")
+def m():
+    import alto_amd.mxfp4 as mod
+    return mod
+
+
+def _qkv(B, Hq, Hk, Sq, Sk, D, Dv, seed, v_mode="randn"):
+    g = torch.Generator().manual_seed(seed)
+    q = torch.randn(B, Hq, Sq, D, generator=g).to(torch.bfloat16)
+    k = torch.randn(B, Hk, Sk, D, generator=g).to(torch.bfloat16)
+    v = torch.randn(B, Hk, Sk, Dv, generator=g).to(torch.bfloat16)
+    if v_mode == "ones":
+        v = torch.ones_like(v)
+    elif v_mode == "biased":
+        v = v + 2.0
+    return q, k, v
+
+
+def _rel(a, b):
+    return float((a.float() - b.float()).norm() / b.float().norm().clamp_min(1e-12))
+
+
+CASES = [
+    # B, Hq, Hk, Sq, Sk, D, Dv, causal
+    (1, 4, 2, 128, 128, 64, 64, True),
+    (2, 4, 4, 256, 256, 128, 128, True),
+    (1, 8, 1, 256, 256, 128, 128, False),
+    (1, 2, 1, 128, 256, 128, 64, True),       # Sq < Sk: mask aligned to the bottom-right corner
+    (1, 2, 2, 96, 128, 192, 128, False),      # Sq not a multiple of the 128 rows a workgroup covers
+    (1, 2, 1, 64, 192, 256, 128, False),
+    (1, 2, 1, 32, 64, 64, 128, True),
+    (1, 3, 3, 160, 320, 192, 64, True),
+]
+
+
+@pytest.mark.parametrize("case", CASES, ids=lambda c: "x".join(map(str, c)))
+def test_attention_matches_cpu_model(m, case):
+    B, Hq, Hk, Sq, Sk, D, Dv, causal = case
+    q, k, v = _qkv(B, Hq, Hk, Sq, Sk, D, Dv, seed=sum(case))
+    out, lse, _ = m.triton_attention_mxfp4(q.to(DEV), k.to(DEV), v.to(DEV), None, None, D ** -0.5, 0.0, 0, 0, Sq, Sk, causal, False, True, "bhsd")
+    ref, ref_lse = attention_fwd_ref(q, k, v, causal=causal)
+    assert out.dtype == torch.bfloat16 and out.shape == (B, Hq, Sq, Dv) and lse.shape == (B, Hq, Sq)
+    assert _rel(out.cpu(), ref) <= REL_L2
+    assert float((lse.cpu() - ref_lse).abs().max()) <= 1e-4
+    # and it is attention: close to the fp32 result within what 4-bit operands allow
+    assert _rel(out.cpu(), attention_fp32_ref(q, k, v, causal=causal)) < 0.35
+
+
+def test_operands_are_the_reference_quantisations(m):
+    """Q, K: 2D-block codes/scales along the head dim; V: the same 2D-block quantisation, packed along the keys."""
+    q, k, v = _qkv(2, 2, 1, 64, 128, 128, 64, seed=3)
+    qq, qs, kq, ks, vq, vs = m.quantize_qkv(q.to(DEV), k.to(DEV), v.to(DEV))
+    for got, got_s, src in ((qq, qs, q), (kq, ks, k)):
+        c, s = O.quantize(src, axis=-1, is_2d_block=True)
+        assert torch.equal(got.cpu(), c) and torch.equal(got_s.cpu(), s)
+    c, s = O.quantize(v.transpose(-1, -2).contiguous(), axis=-1, is_2d_block=True)
+    assert torch.equal(vq.cpu(), c) and torch.equal(vs.cpu(), s)
+    # same codes as quantising V along Dv (2D blocks are symmetric), only packed the other way
+    c2, s2 = O.quantize(v, axis=-1, is_2d_block=True)
+    assert torch.equal(O.unpack_nibbles(c.reshape(-1, c.shape[-1])).reshape(2, 1, 64, 128).transpose(-1, -2),
+                       O.unpack_nibbles(c2.reshape(-1, c2.shape[-1])).reshape(2, 1, 128, 64))
+    assert torch.equal(s.transpose(-1, -2), s2)
+
+
+@pytest.mark.parametrize("v_mode", ["ones", "biased"])
+def test_constant_value_attention(m, v_mode):
+    """test_mxfp_pnq.py:163-174 on the GPU: with V = 1 the output is exactly 1 (row sums come from the quantised P)."""
+    torch.manual_seed(1234)
+    q = torch.randn(1, 32, 64, 64, dtype=torch.bfloat16)
+    k = torch.randn(1, 8, 64, 64, dtype=torch.bfloat16)
+    v = torch.ones(1, 8, 64, 64, dtype=torch.bfloat16)
+    if v_mode == "biased":
+        v = torch.randn(1, 8, 64, 64, dtype=torch.bfloat16) + 2.0
+    out, lse, _ = m.triton_attention_mxfp4(q.to(DEV), k.to(DEV), v.to(DEV), causal=True)
+    if v_mode == "ones":
+        assert torch.equal(out.cpu(), torch.ones_like(out.cpu()))
+    else:
+        ref, _ = attention_fwd_ref(q, k, v, causal=True)
+        assert _rel(out.cpu(), ref) <= REL_L2
+
+
+def test_module_form_and_prequantised_entry(m):
+    cfg = m.TrainingOpConfig()
+    B, L, Hq, Hk, D = 1, 128, 4, 2, 128
+    q, k, v = _qkv(B, Hq, Hk, L, L, D, D, seed=9)
+    attn = m.LPScaledDotProductAttention(cfg)
+    o = attn(q.transpose(1, 2).to(DEV), k.transpose(1, 2).to(DEV), v.transpose(1, 2).to(DEV), is_causal=True)   # [B, L, N, H]
+    assert o.shape == (B, L, Hq, D)
+    ref, _ = attention_fwd_ref(q, k, v, causal=True)
+    assert _rel(o.transpose(1, 2).cpu(), ref) <= REL_L2
+    qq, qs, kq, ks, vq, vs = m.quantize_qkv(q.to(DEV), k.to(DEV), v.to(DEV))
+    o2, _ = m.attention_mxfp4_forward(qq, kq, vq, qs, ks, vs, D ** -0.5, True)
+    assert torch.equal(o2, o.transpose(1, 2))
+    with pytest.raises(ValueError):
+        attn(q.to(DEV), k.to(DEV), v.to(DEV), attention_masks=object())
+
+
+def test_rejected_arguments(m):
+    q, k, v = (t.to(DEV) for t in _qkv(1, 2, 2, 64, 64, 64, 64, seed=1))
+    with pytest.raises(NotImplementedError):
+        m.triton_attention_mxfp4(q, k, v, layout="bshd")
+    with pytest.raises(NotImplementedError):
+        m.triton_attention_mxfp4(q, k, v, dropout_p=0.1)
+    with pytest.raises(NotImplementedError):
+        m.triton_attention_mxfp4(q, k, v, bias=torch.zeros(1, device=DEV))
+    with pytest.raises(AssertionError, match="Sq <= Sk"):
+        m.triton_attention_mxfp4(q.repeat(1, 1, 2, 1), k, v, causal=True)
+    qb, kb, vb = (t.to(DEV) for t in _qkv(1, 2, 2, 64, 96, 64, 64, seed=1))
+    with pytest.raises(AssertionError, match="multiple of 64"):
+        m.triton_attention_mxfp4(qb, kb, vb, causal=False)
+    q3, k3, v3 = (t.to(DEV) for t in _qkv(1, 2, 2, 64, 64, 96, 64, seed=1))
+    with pytest.raises(AssertionError, match="head dim"):
+        m.triton_attention_mxfp4(q3, k3, v3, causal=False)
+    with pytest.raises(RuntimeError):
+        m.triton_attention_mxfp4(q.cpu(), k.cpu(), v.cpu())
