@@ -20,6 +20,9 @@ struct AttnArgs {
   int causal;
 };
 
+#ifndef ATTN_WG_PER_CU
+#define ATTN_WG_PER_CU 3
+#endif
 constexpr float ATTN_RCP_LN2 = 1.4426950408889634f;
 constexpr float ATTN_LN2 = 0.6931471824645996f;
 
@@ -31,17 +34,29 @@ __device__ __forceinline__ float xor32(float v) { return __shfl_xor(v, 32, 64); 
 __device__ __forceinline__ uint32_t xor32(uint32_t v) { return (uint32_t)__shfl_xor((int)v, 32, 64); }
 
 // NK = D / 64 (MFMA K steps of Q K^T), ND = Dv / 32 (output tiles).
+// The four waves of a workgroup own 128 consecutive query rows of one head and walk the key blocks together: a block's
+// K codes (64 rows x D/2 bytes) and V codes (Dv rows x 32 bytes) are fetched once per workgroup with coalesced 16-byte
+// loads one block ahead, parked in registers during the softmax and written to the other half of a two-slot LDS ring;
+// one barrier per block.  (Fetching the pieces per wave straight from global memory made the vector-memory path the
+// bound: 8 KB per wave and block in scattered 16-byte accesses.)
 template <int NK, int ND>
-__global__ __launch_bounds__(256) void attn_fwd_kernel(AttnArgs a) {
+__global__ __launch_bounds__(256, ATTN_WG_PER_CU) void attn_fwd_kernel(AttnArgs a) {
   constexpr int D = NK * 64, DV = ND * 32;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  constexpr int K_BYTES = 64 * (D / 2), V_BYTES = DV * 32;       // one block of K codes, of V codes
+  constexpr int K_PIECES = K_BYTES / 16, V_PIECES = V_BYTES / 16;
+  constexpr int K_PER_THREAD = (K_PIECES + 255) / 256, V_PER_THREAD = (V_PIECES + 255) / 256;
+  __shared__ __attribute__((aligned(16))) uint8_t ring[2][K_BYTES + V_BYTES];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r = lane & 31, h = lane >> 5;
-  const int q0 = (blockIdx.x * 4 + wave) * 32;
-  if (q0 >= a.Sq) return;                         // no workgroup-wide synchronisation below
+  const int qblk = a.causal ? (int)(gridDim.x - 1 - blockIdx.x) : (int)blockIdx.x;   // causal: long rows are dispatched first
+  const int q0 = (qblk * 4 + wave) * 32;
+  const bool live = q0 < a.Sq;                    // a wave past the last row still helps with loads and barriers
   const int hq = blockIdx.y, b = blockIdx.z;
   const int hk = hq / (a.Hq / a.Hk);
   const int64_t bhq = (int64_t)b * a.Hq + hq, bhk = (int64_t)b * a.Hk + hk;
-  const int qrow = q0 + r;
+  const int qrow = live ? q0 + r : 0;
   const int shift = a.Sk - a.Sq;                  // causal mask is aligned to the bottom-right corner
 
   // ---- Q pieces: row qrow, K step ks, half h -> 16 bytes; one scale byte per (32-row block, 32-column block)
@@ -50,7 +65,7 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(AttnArgs a) {
 #pragma unroll
   for (int s = 0; s < NK; ++s) {
     qf[s] = frag16(a.q + (bhq * a.Sq + qrow) * (D / 2) + s * 32 + h * 16);
-    qsc[s] = a.qs[(bhq * (a.Sq / 32) + q0 / 32) * (D / 32) + 2 * s + h];
+    qsc[s] = a.qs[(bhq * (a.Sq / 32) + qrow / 32) * (D / 32) + 2 * s + h];
   }
 
   v16f_t acc_o[ND], acc_l;
@@ -60,108 +75,162 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(AttnArgs a) {
     for (int v = 0; v < 16; ++v) acc_o[d][v] = 0.0f;
 #pragma unroll
   for (int v = 0; v < 16; ++v) acc_l[v] = 0.0f;
-  float m_i = -__builtin_inff();
+  float m_i = -__builtin_inff();                   // running row max of S * sm_scale * log2(e)
+  const float c2 = a.sm_scale * ATTN_RCP_LN2;
 
   // byte selectors that interleave my 4-key groups with the partner lane's into natural key order
   const uint32_t sel_lo = h ? 0x01000504u : 0x05040100u;
   const uint32_t sel_hi = h ? 0x03020706u : 0x07060302u;
   const v8i_t ones = v8i_t{0x22222222, 0x22222222, 0x22222222, 0x22222222, 0, 0, 0, 0};   // E2M1 code 2 = 1.0
 
-  int nblk = a.Sk / 64;
+  // blocks this wave needs, and the most any wave of the workgroup needs (the last wave's rows reach furthest)
+  const int all_blk = a.Sk / 64;
+  int nblk = all_blk, wg_blk = all_blk;
   if (a.causal) {
-    const int lim = (q0 + 32 + shift + 63) / 64;  // blocks holding a key some row of this wave may see
-    nblk = lim < nblk ? lim : nblk;
+    const int lim = (q0 + 32 + shift + 63) / 64;
+    nblk = lim < all_blk ? lim : all_blk;
+    int q_end = qblk * 128 + 128;
+    q_end = q_end < a.Sq ? q_end : a.Sq;
+    const int wlim = (q_end + shift + 63) / 64;
+    wg_blk = wlim < all_blk ? wlim : all_blk;
   }
+  if (!live) nblk = 0;
 
-  for (int kb = 0; kb < nblk; ++kb) {
-    const int key0 = kb * 64;
-    // ---- S = Q K^T for two 32-key tiles
-    v16f_t S[2];
+  // ---- cooperative fetch of one block: thread -> 16-byte pieces (K is contiguous; V is DV rows of 32 bytes)
+  uint4 kreg[K_PER_THREAD], vreg[V_PER_THREAD];
+  auto fetch = [&](int kb) {
+    const uint8_t* kblk = a.k + (bhk * a.Sk + kb * 64) * (D / 2);
+    const uint8_t* vblk = a.vt + bhk * DV * (int64_t)(a.Sk / 2) + kb * 32;
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
-#pragma unroll
-      for (int v = 0; v < 16; ++v) S[t][v] = 0.0f;
-      const uint8_t* krow = a.k + (bhk * a.Sk + key0 + 32 * t + r) * (D / 2) + h * 16;
-      const uint8_t* ksrow = a.ks + (bhk * (a.Sk / 32) + key0 / 32 + t) * (D / 32) + h;
-#pragma unroll
-      for (int s = 0; s < NK; ++s) {
-        const v8i_t kf = frag16(krow + s * 32);
-        const int ksc = ksrow[2 * s];
-        S[t] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(kf, qf[s], S[t], 4, 4, 0, ksc, 0, qsc[s]);
-      }
+    for (int i = 0; i < K_PER_THREAD; ++i) {
+      const int piece = tid + 256 * i;
+      if (K_PIECES % 256 == 0 || piece < K_PIECES) kreg[i] = *reinterpret_cast<const uint4*>(kblk + (uint32_t)piece * 16);
     }
-    // ---- scale, mask, running max
-    const bool diag = a.causal && (key0 + 63 > q0 + shift);
-    float mx = -__builtin_inff();
 #pragma unroll
-    for (int t = 0; t < 2; ++t)
+    for (int i = 0; i < V_PER_THREAD; ++i) {
+      const int piece = tid + 256 * i;
+      if (V_PIECES % 256 == 0 || piece < V_PIECES)
+        vreg[i] = *reinterpret_cast<const uint4*>(vblk + (uint32_t)(piece >> 1) * (uint32_t)(a.Sk / 2) + (piece & 1) * 16);
+    }
+  };
+  auto park = [&](int slot) {
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        float s = S[t][v] * a.sm_scale;
-        if (diag) {
-          const int key = key0 + 32 * t + 8 * (v >> 2) + 4 * h + (v & 3);
-          if (key > qrow + shift) s = -__builtin_inff();
-        }
-        S[t][v] = s;
-        mx = fmaxf(mx, s);
-      }
-    mx = fmaxf(mx, xor32(mx));
-    const float m_new = fmaxf(m_i, mx);
-    const float alpha = __builtin_amdgcn_exp2f((m_i - m_new) * ATTN_RCP_LN2);
-    m_i = m_new;
+    for (int i = 0; i < K_PER_THREAD; ++i) {
+      const int piece = tid + 256 * i;
+      if (K_PIECES % 256 == 0 || piece < K_PIECES) *reinterpret_cast<uint4*>(&ring[slot][piece * 16]) = kreg[i];
+    }
+#pragma unroll
+    for (int i = 0; i < V_PER_THREAD; ++i) {
+      const int piece = tid + 256 * i;
+      if (V_PIECES % 256 == 0 || piece < V_PIECES) *reinterpret_cast<uint4*>(&ring[slot][K_BYTES + piece * 16]) = vreg[i];
+    }
+  };
+  if (wg_blk > 0) {
+    fetch(0);
+    park(0);
+  }
+  __syncthreads();
 
-    // ---- probabilities, one E8M0 scale per (row, 32 keys), E2M1 codes (round to nearest even)
-    uint32_t c[2][2];
-    int psc[2];
+  for (int kb = 0; kb < wg_blk; ++kb) {
+    const int key0 = kb * 64;
+    const uint8_t* tile = ring[kb & 1];
+    if (kb + 1 < wg_blk) fetch(kb + 1);            // travels during this block's arithmetic
+    if (kb < nblk) {
+      // scale bytes of the block: uniform addresses; the lane half picks its byte
+      const uint8_t* ksblk = a.ks + (bhk * (a.Sk / 32) + kb * 2) * (D / 32);
+      const uint8_t* vsblk = a.vs + bhk * (DV / 32) * (a.Sk / 32) + kb * 2;
+      // ---- S = Q K^T for two 32-key tiles
+      v16f_t S[2];
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
-      float p[16];
-      float am = 0.0f;
+      for (int t = 0; t < 2; ++t) {
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        p[v] = __builtin_amdgcn_exp2f((S[t][v] - m_new) * ATTN_RCP_LN2);
-        am = fmaxf(am, p[v]);
+        for (int v = 0; v < 16; ++v) S[t][v] = 0.0f;
+#pragma unroll
+        for (int s = 0; s < NK; ++s) {
+          const v8i_t kf = frag16(tile + (32 * t + r) * (D / 2) + 32 * s + 16 * h);
+          const int ksc = h ? ksblk[t * (D / 32) + 2 * s + 1] : ksblk[t * (D / 32) + 2 * s];
+          S[t] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(kf, qf[s], S[t], 4, 4, 0, ksc, 0, qsc[s]);
+        }
       }
-      am = fmaxf(am, xor32(am));
-      const uint32_t e = e8m0_from_f32_bits(f2u(am));
-      psc[t] = (int)e;
-      const float scale_f = u2f(e << 23);
+      // ---- mask (only blocks the diagonal crosses), running max kept in the base-2 domain: m = max(S) * sm_scale * log2(e)
+      if (a.causal && key0 + 63 > q0 + shift) {
+        asm volatile("" ::: "memory");   // keep this a branch: most blocks skip it
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int v = 0; v < 16; ++v) {
+            const int key = key0 + 32 * t + 8 * (v >> 2) + 4 * h + (v & 3);
+            if (key > qrow + shift) S[t][v] = -__builtin_inff();
+          }
+      }
+      float mx = -__builtin_inff();
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) mx = fmaxf(mx, S[t][v]);
+      mx = fmaxf(mx, xor32(mx));
+      const float m_new = fmaxf(m_i, mx * c2);
+      const float alpha = __builtin_amdgcn_exp2f(m_i - m_new);
+      m_i = m_new;
+
+      // ---- probabilities, one E8M0 scale per (row, 32 keys), E2M1 codes (round to nearest even)
+      uint32_t c[2][2];
+      int psc[2];
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        float am = 0.0f;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          S[t][v] = __builtin_amdgcn_exp2f(__builtin_fmaf(S[t][v], c2, -m_new));
+          am = fmaxf(am, S[t][v]);
+        }
+        am = fmaxf(am, xor32(am));
+        const uint32_t e = e8m0_from_f32_bits(f2u(am));
+        psc[t] = (int)e;
+        const float scale_f = u2f(e << 23);
+#pragma unroll
+        for (int w = 0; w < 2; ++w) {
+          uint32_t o = 0;
+          o = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(o, S[t][8 * w + 0], S[t][8 * w + 1], scale_f, 0);
+          o = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(o, S[t][8 * w + 2], S[t][8 * w + 3], scale_f, 1);
+          o = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(o, S[t][8 * w + 4], S[t][8 * w + 5], scale_f, 2);
+          o = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(o, S[t][8 * w + 6], S[t][8 * w + 7], scale_f, 3);
+          c[t][w] = o;
+        }
+      }
+      // Lane (r, h) multiplies tile h of this block: it keeps its half of tile h and gets the other half from lane
+      // (r, 1 - h), which in turn needs this lane's half of tile 1 - h.
+      uint32_t keep[2], recv[2];
 #pragma unroll
       for (int w = 0; w < 2; ++w) {
-        uint32_t o = 0;
-        o = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(o, p[8 * w + 0], p[8 * w + 1], scale_f, 0);
-        o = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(o, p[8 * w + 2], p[8 * w + 3], scale_f, 1);
-        o = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(o, p[8 * w + 4], p[8 * w + 5], scale_f, 2);
-        o = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(o, p[8 * w + 6], p[8 * w + 7], scale_f, 3);
-        c[t][w] = o;
+        keep[w] = h ? c[1][w] : c[0][w];
+        recv[w] = xor32(h ? c[0][w] : c[1][w]);
+      }
+      const v8i_t pf = v8i_t{(int)__builtin_amdgcn_perm(recv[0], keep[0], sel_lo), (int)__builtin_amdgcn_perm(recv[0], keep[0], sel_hi),
+                             (int)__builtin_amdgcn_perm(recv[1], keep[1], sel_lo), (int)__builtin_amdgcn_perm(recv[1], keep[1], sel_hi),
+                             0, 0, 0, 0};
+      const int pscale = h ? psc[1] : psc[0];
+
+      // ---- row sums of the quantised probabilities (a column of ones) and O += P V
+      if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {   // the row maxima settle after a few blocks
+        acc_l[0] *= alpha;                                     // all 16 registers hold the row sum; only [0] is read
+#pragma unroll
+        for (int d = 0; d < ND; ++d)
+#pragma unroll
+          for (int v = 0; v < 16; ++v) acc_o[d][v] *= alpha;
+      }
+      acc_l = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ones, pf, acc_l, 4, 4, 0, 127, 0, pscale);
+#pragma unroll
+      for (int d = 0; d < ND; ++d) {
+        const v8i_t vf = frag16(tile + K_BYTES + (32 * d + r) * 32 + 16 * h);
+        const int vsc = h ? vsblk[d * (a.Sk / 32) + 1] : vsblk[d * (a.Sk / 32)];
+        acc_o[d] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(vf, pf, acc_o[d], 4, 4, 0, vsc, 0, pscale);
       }
     }
-    // Lane (r, h) multiplies tile h of this block: it keeps its half of tile h and gets the other half from lane
-    // (r, 1 - h), which in turn needs this lane's half of tile 1 - h.
-    uint32_t keep[2], recv[2];
-#pragma unroll
-    for (int w = 0; w < 2; ++w) {
-      keep[w] = h ? c[1][w] : c[0][w];
-      recv[w] = xor32(h ? c[0][w] : c[1][w]);
-    }
-    const v8i_t pf = v8i_t{(int)__builtin_amdgcn_perm(recv[0], keep[0], sel_lo), (int)__builtin_amdgcn_perm(recv[0], keep[0], sel_hi),
-                           (int)__builtin_amdgcn_perm(recv[1], keep[1], sel_lo), (int)__builtin_amdgcn_perm(recv[1], keep[1], sel_hi),
-                           0, 0, 0, 0};
-    const int pscale = h ? psc[1] : psc[0];
-
-    // ---- row sums of the quantised probabilities (a column of ones) and O += P V
-#pragma unroll
-    for (int v = 0; v < 16; ++v) acc_l[v] *= alpha;
-    acc_l = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ones, pf, acc_l, 4, 4, 0, 127, 0, pscale);
-#pragma unroll
-    for (int d = 0; d < ND; ++d) {
-#pragma unroll
-      for (int v = 0; v < 16; ++v) acc_o[d][v] *= alpha;
-      const v8i_t vf = frag16(a.vt + ((bhk * DV + 32 * d + r) * (int64_t)(a.Sk / 2)) + (key0 + 32 * h) / 2);
-      const int vsc = a.vs[(bhk * (DV / 32) + d) * (a.Sk / 32) + key0 / 32 + h];
-      acc_o[d] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(vf, pf, acc_o[d], 4, 4, 0, vsc, 0, pscale);
-    }
+    if (kb + 1 < wg_blk) park((kb + 1) & 1);
+    __syncthreads();
   }
+  if (!live) return;
 
   // ---- O = acc / l, bf16; log-sum-exp
   const float l = acc_l[0];
@@ -181,7 +250,7 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(AttnArgs a) {
       w.y = __builtin_bit_cast(uint32_t, hi);
       *reinterpret_cast<uint2*>(orow + 32 * d + 8 * g + 4 * h) = w;
     }
-  if (h == 0) a.lse[bhq * a.Sq + qrow] = (m_i * ATTN_RCP_LN2 + log2f(l)) * ATTN_LN2;
+  if (h == 0) a.lse[bhq * a.Sq + qrow] = (m_i + log2f(l)) * ATTN_LN2;
 }
 
 template <int NK, int ND>

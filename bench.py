@@ -244,6 +244,39 @@ class GroupedGemm(Workload):
         return run, 2.0 * rows * self.N * self.K, f"{rows} rows of the largest expert, dequantize + fp32 matmul"
 
 
+class AttentionFwd(Workload):
+    """MXFP4 flash-attention forward on pre-quantised Q, K, V: the largest case of the reference's own test list
+    (tests/unittest/mxfp4/test_mxfp_attention.py:64: batch 4, 2048 tokens, 64 query / 8 KV heads, head dim 128, causal)."""
+    name = "attn_fwd[b4,s2048,hq64,hk8,d128,causal]"
+    bound = "mfma"
+    kernel = "attention"
+    B, S, HQ, HK, D = 4, 2048, 64, 8, 128
+
+    def setup(self, dev, gen):
+        import torch
+        import alto_amd.mxfp4 as m
+        self.m = m
+        q = torch.randn(self.B, self.HQ, self.S, self.D, device=dev, generator=gen).bfloat16()
+        k = torch.randn(self.B, self.HK, self.S, self.D, device=dev, generator=gen).bfloat16()
+        v = torch.randn(self.B, self.HK, self.S, self.D, device=dev, generator=gen).bfloat16()
+        self.q, self.k, self.v = q, k, v
+        self.ops = m.quantize_qkv(q, k, v)
+        # algorithmic FLOPs: the unmasked (query, key) pairs, each 2 D (QK^T) + 2 Dv (PV)
+        self.work = 4.0 * self.D * self.B * self.HQ * (self.S * (self.S + 1) / 2)
+
+    def step(self):
+        qq, qs, kq, ks, vq, vs = self.ops
+        return self.m.attention_mxfp4_forward(qq, kq, vq, qs, ks, vs, self.D ** -0.5, True)
+
+    def cpu_sample(self):
+        from oracle.attention_oracle import attention_fwd_ref
+        q, k, v = self.q[:1, :4].cpu(), self.k[:1, :1].cpu(), self.v[:1, :1].cpu()   # 4 query heads that share one KV head
+
+        def run():
+            attention_fwd_ref(q, k, v, causal=True)
+        return run, self.work * 4 / (self.B * self.HQ), "4 of 256 (batch, head) pairs at full sequence length"
+
+
 class CopyCalibration(Workload):
     """Plain device copy of 256 MiB (torch's elementwise copy kernel): the known-size launch against which the
     FETCH_SIZE / WRITE_SIZE counters of the other kernels are scaled.  Not part of the product path."""
@@ -311,6 +344,7 @@ def make_workloads():
         "cfg4_dgrad": Gemm("cfg4_dgrad_gemm[8192x14336x4096]", 8192, 14336, 4096, False, True, "grad", "weight"),
         "cfg4_wgrad": Gemm("cfg4_wgrad_gemm[4096x14336x8192]", 4096, 14336, 8192, False, False, "grad", "act"),
         "cfg5_grouped": GroupedGemm(),
+        "attn_fwd": AttentionFwd(),
         "copy_calib": CopyCalibration(),
         "mfma_probe_const": MfmaProbe(False),
         "mfma_probe_random": MfmaProbe(True),
