@@ -391,31 +391,53 @@ __device__ __forceinline__ void gemm_tile_store(const TileArgs& ta, TileAcc& acc
     // (conflict-free for the 8-byte writes of 32 different rows and for the row-wise 16-byte reads), then stored as
     // whole rows: 32 lanes x 16 bytes = one 512-byte row segment per half-wave.
     __syncthreads();   // every wave is done reading operand pieces
+    // LDS byte offset of this lane's 8 bytes of (u, vq): row r of the 32-row band, chunk (8 wn + 4 u + vq) ^ r
+    auto stage_out = [&](auto scaled) {
 #pragma unroll
-    for (int t = 0; t < 4; ++t) {
-      const int ml = 128 * wm + 32 * t + r;
-#pragma unroll
-      for (int u = 0; u < 2; ++u) {
+      for (int u = 0; u < 2; ++u)
 #pragma unroll
         for (int vq = 0; vq < 4; ++vq) {
-          const int chunk = 8 * wn + 4 * u + vq;
-          float f0 = acc[t][u][4 * vq + 0] * ta.out_scale, f1 = acc[t][u][4 * vq + 1] * ta.out_scale;
-          float f2 = acc[t][u][4 * vq + 2] * ta.out_scale, f3 = acc[t][u][4 * vq + 3] * ta.out_scale;
-          uint2 o;
-          o.x = pack_bf16x2(f0, f1);
-          o.y = pack_bf16x2(f2, f3);
-          *reinterpret_cast<uint2*>(smem + ml * 512 + ((chunk ^ (ml & 31)) << 4) + 8 * h) = o;
-        }
-      }
-    }
-    __syncthreads();
+          const uint32_t off = (uint32_t)(128 * wm + r) * 512 + (((8 * wn + 4 * u + vq) ^ r) << 4) + 8 * h;
 #pragma unroll
-    for (int it = 0; it < 16; ++it) {
-      const int id = it * GT_THREADS + tid;
-      const int row = id >> 5, ch = id & 31;
-      const uint4 v = *reinterpret_cast<const uint4*>(smem + row * 512 + ((ch ^ (row & 31)) << 4));
-      const int64_t m = ta.m0 + row, n = ta.n0 + 8 * ch;
-      if (m >= ta.m_lo && m < ta.m_hi && n + 8 <= ta.n_hi) *reinterpret_cast<uint4*>(c + m * ldc + n) = v;
+          for (int t = 0; t < 4; ++t) {
+            float f0 = acc[t][u][4 * vq + 0], f1 = acc[t][u][4 * vq + 1], f2 = acc[t][u][4 * vq + 2], f3 = acc[t][u][4 * vq + 3];
+            if constexpr (decltype(scaled)::value) {
+              f0 *= ta.out_scale; f1 *= ta.out_scale; f2 *= ta.out_scale; f3 *= ta.out_scale;
+            }
+            uint2 o;
+            o.x = pack_bf16x2(f0, f1);
+            o.y = pack_bf16x2(f2, f3);
+            *reinterpret_cast<uint2*>(smem + off + t * (32 * 512)) = o;
+          }
+        }
+    };
+    if (ta.out_scale == 1.0f) stage_out(std::false_type{});
+    else stage_out(std::true_type{});
+    __syncthreads();
+    // thread -> chunk ch of rows row0 + 16 it: the XOR term alternates between two values
+    const int row0 = tid >> 5, ch = tid & 31;
+    const uint32_t rd_even = (uint32_t)row0 * 512 + ((ch ^ row0) << 4), rd_odd = (uint32_t)(row0 + 16) * 512 + ((ch ^ (row0 + 16)) << 4);
+    const bool full = ta.m0 >= ta.m_lo && ta.m0 + GT_TM <= ta.m_hi && ta.n0 + GT_TN <= ta.n_hi && ldc < (1 << 22);
+    if (full) {   // no bounds to check; one 64-bit tile origin plus 32-bit offsets
+      OutT* origin = c + ta.m0 * ldc + ta.n0;
+      const uint32_t step = (uint32_t)ldc * 16;
+      uint32_t eoff = (uint32_t)row0 * (uint32_t)ldc + 8 * ch;
+#pragma unroll
+      for (int it = 0; it < 16; it += 2) {
+        const uint4 v0 = *reinterpret_cast<const uint4*>(smem + rd_even + (it / 2) * (32 * 512));
+        const uint4 v1 = *reinterpret_cast<const uint4*>(smem + rd_odd + (it / 2) * (32 * 512));
+        *reinterpret_cast<uint4*>(origin + eoff) = v0;
+        *reinterpret_cast<uint4*>(origin + (eoff + step)) = v1;
+        eoff += 2 * step;
+      }
+    } else {
+#pragma unroll
+      for (int it = 0; it < 16; ++it) {
+        const int row = row0 + 16 * it;
+        const uint4 v = *reinterpret_cast<const uint4*>(smem + ((it & 1) ? rd_odd : rd_even) + (it / 2) * (32 * 512));
+        const int64_t m = ta.m0 + row, n = ta.n0 + 8 * ch;
+        if (m >= ta.m_lo && m < ta.m_hi && n + 8 <= ta.n_hi) *reinterpret_cast<uint4*>(c + m * ldc + n) = v;
+      }
     }
   } else {
 #pragma unroll
