@@ -64,6 +64,22 @@ def test_attention_matches_cpu_model(m, case):
     assert _rel(out.cpu(), attention_fp32_ref(q, k, v, causal=causal)) < 0.35
 
 
+def test_long_sequence_matches_cpu_model(m):
+    """The bench shape per (batch, KV head): 2048 tokens, 8 query heads on one KV head, head dim 128, causal."""
+    q, k, v = _qkv(1, 8, 1, 2048, 2048, 128, 128, seed=77)
+    out, lse, _ = m.triton_attention_mxfp4(q.to(DEV), k.to(DEV), v.to(DEV), causal=True)
+    ref, ref_lse = attention_fwd_ref(q, k, v, causal=True)
+    assert _rel(out.cpu(), ref) <= REL_L2
+    assert float((lse.cpu() - ref_lse).abs().max()) <= 1e-4
+    # size-independent property: every output row is a convex combination of the (quantised) value rows it may see
+    vq = O.dequantize(*O.quantize(v, axis=-1, is_2d_block=True), torch.float32, axis=-1, is_2d_block=True)[0, 0]
+    hi = torch.cummax(vq, dim=0).values
+    lo = -torch.cummax(-vq, dim=0).values
+    o = out.cpu().float()[0]                                   # [8, 2048, 128]; row i sees keys 0..i
+    tol = 2 ** -7 * vq.abs().max()
+    assert bool(((o <= hi[None] + tol) & (o >= lo[None] - tol)).all())
+
+
 def test_operands_are_the_reference_quantisations(m):
     """Q, K: 2D-block codes/scales along the head dim; V: the same 2D-block quantisation, packed along the keys."""
     q, k, v = _qkv(2, 2, 1, 64, 128, 128, 64, seed=3)
