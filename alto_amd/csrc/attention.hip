@@ -6,6 +6,9 @@
 // that land in lanes): S tiles and O tiles keep the query row in the lane (lane % 32) and spread keys / value columns
 // over the 16 accumulator registers, so the per-row softmax state (running max, rescale factor) is one scalar per lane
 // and the only cross-lane traffic is between the two lanes (l, l ^ 32) that share a row.
+#include <type_traits>
+#include <utility>
+
 #include "common.h"
 
 namespace alto {
@@ -13,7 +16,7 @@ namespace alto {
 struct AttnArgs {
   const uint8_t* q;  const uint8_t* qs;    // [B, Hq, Sq, D/2],  [B, Hq, Sq/32, D/32]
   const uint8_t* k;  const uint8_t* ks;    // [B, Hk, Sk, D/2],  [B, Hk, Sk/32, D/32]
-  const uint8_t* vt; const uint8_t* vs;    // [B, Hk, Dv, Sk/2] packed along keys, [B, Hk, Dv/32, Sk/32]
+  const uint8_t* vt; const uint8_t* vs;    // [B, Hk, Dv, Sk/2] packed along keys, [B, Hk, Sk/32, Dv/32]
   void* out; float* lse;                   // [B, Hq, Sq, Dv] bf16, [B, Hq, Sq] fp32
   int Hq, Hk, Sq, Sk;
   float sm_scale;
@@ -30,8 +33,18 @@ __device__ __forceinline__ v8i_t frag16(const uint8_t* p) {
   const uint4 w = *reinterpret_cast<const uint4*>(p);
   return v8i_t{(int)w.x, (int)w.y, (int)w.z, (int)w.w, 0, 0, 0, 0};
 }
-__device__ __forceinline__ float xor32(float v) { return __shfl_xor(v, 32, 64); }
-__device__ __forceinline__ uint32_t xor32(uint32_t v) { return (uint32_t)__shfl_xor((int)v, 32, 64); }
+template <int N, typename F, int... I>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, I...>) { (f(std::integral_constant<int, I>{}), ...); }
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) { static_for_impl<N>(static_cast<F&&>(f), std::make_integer_sequence<int, N>{}); }
+
+typedef unsigned v2u_t __attribute__((ext_vector_type(2)));
+// v_permlane32_swap(a, b) returns {a of lanes 0..31 | b of lanes 0..31,  a of lanes 32..63 | b of lanes 32..63}
+// (first | second half of the wave): a value and its copy come back as the low half's and the high half's values.
+__device__ __forceinline__ float pair_max(float v) {   // max over the two lanes l and l ^ 32
+  const v2u_t p = __builtin_amdgcn_permlane32_swap(f2u(v), f2u(v), false, false);
+  return fmaxf(u2f(p[0]), u2f(p[1]));
+}
 
 // NK = D / 64 (MFMA K steps of Q K^T), ND = Dv / 32 (output tiles).
 // The four waves of a workgroup own 128 consecutive query rows of one head and walk the key blocks together: a block's
@@ -78,9 +91,6 @@ __global__ __launch_bounds__(256, ATTN_WG_PER_CU) void attn_fwd_kernel(AttnArgs 
   float m_i = -__builtin_inff();                   // running row max of S * sm_scale * log2(e)
   const float c2 = a.sm_scale * ATTN_RCP_LN2;
 
-  // byte selectors that interleave my 4-key groups with the partner lane's into natural key order
-  const uint32_t sel_lo = h ? 0x01000504u : 0x05040100u;
-  const uint32_t sel_hi = h ? 0x03020706u : 0x07060302u;
   const v8i_t ones = v8i_t{0x22222222, 0x22222222, 0x22222222, 0x22222222, 0, 0, 0, 0};   // E2M1 code 2 = 1.0
 
   // blocks this wave needs, and the most any wave of the workgroup needs (the last wave's rows reach furthest)
@@ -125,8 +135,22 @@ __global__ __launch_bounds__(256, ATTN_WG_PER_CU) void attn_fwd_kernel(AttnArgs 
       if (V_PIECES % 256 == 0 || piece < V_PIECES) *reinterpret_cast<uint4*>(&ring[slot][K_BYTES + piece * 16]) = vreg[i];
     }
   };
+  // Scale bytes of a block: 2 D/32 bytes of K (key tile t, 32-column block j at byte t D/32 + j) and 2 Dv/32 bytes of V
+  // (key tile t, column block d at byte t Dv/32 + d) sit at wave-uniform, 4-byte aligned addresses: whole dwords, one
+  // block ahead; the MFMA picks a byte of a dword with op_sel, the lane half h shifts its byte into place.
+  constexpr int KS_DW = 2 * (D / 32) / 4, VS_DW = (2 * (DV / 32) + 3) / 4;
+  uint32_t ksw[KS_DW], vsw[VS_DW], ksw_next[KS_DW], vsw_next[VS_DW];
+  auto fetch_scales = [&](int kb, uint32_t (&kw)[KS_DW], uint32_t (&vw)[VS_DW]) {
+    const uint32_t* kp = reinterpret_cast<const uint32_t*>(a.ks + (bhk * (a.Sk / 32) + kb * 2) * (D / 32));
+    const uint32_t* vp = reinterpret_cast<const uint32_t*>(a.vs + (bhk * (a.Sk / 32) + kb * 2) * (DV / 32));
+#pragma unroll
+    for (int i = 0; i < KS_DW; ++i) kw[i] = kp[i];
+#pragma unroll
+    for (int i = 0; i < VS_DW; ++i) vw[i] = vp[i];
+  };
   if (wg_blk > 0) {
     fetch(0);
+    fetch_scales(0, ksw_next, vsw_next);
     park(0);
   }
   __syncthreads();
@@ -134,24 +158,31 @@ __global__ __launch_bounds__(256, ATTN_WG_PER_CU) void attn_fwd_kernel(AttnArgs 
   for (int kb = 0; kb < wg_blk; ++kb) {
     const int key0 = kb * 64;
     const uint8_t* tile = ring[kb & 1];
-    if (kb + 1 < wg_blk) fetch(kb + 1);            // travels during this block's arithmetic
-    if (kb < nblk) {
-      // scale bytes of the block: uniform addresses; the lane half picks its byte
-      const uint8_t* ksblk = a.ks + (bhk * (a.Sk / 32) + kb * 2) * (D / 32);
-      const uint8_t* vsblk = a.vs + bhk * (DV / 32) * (a.Sk / 32) + kb * 2;
-      // ---- S = Q K^T for two 32-key tiles
-      v16f_t S[2];
 #pragma unroll
-      for (int t = 0; t < 2; ++t) {
+    for (int i = 0; i < KS_DW; ++i) ksw[i] = ksw_next[i];
+#pragma unroll
+    for (int i = 0; i < VS_DW; ++i) vsw[i] = vsw_next[i];
+    if (kb + 1 < wg_blk) {                         // travels during this block's arithmetic
+      fetch(kb + 1);
+      fetch_scales(kb + 1, ksw_next, vsw_next);
+    }
+    if (kb < nblk) {
+      // ---- S = Q K^T for two 32-key tiles; K scale of (tile t, step s, half h) = byte t D/32 + 2 s + h
+      v16f_t S[2];
+      int ksh[KS_DW];
+#pragma unroll
+      for (int i = 0; i < KS_DW; ++i) ksh[i] = (int)(ksw[i] >> (8 * h));
+      static_for<2>([&](auto tc) {
+        constexpr int t = decltype(tc)::value;
 #pragma unroll
         for (int v = 0; v < 16; ++v) S[t][v] = 0.0f;
-#pragma unroll
-        for (int s = 0; s < NK; ++s) {
+        static_for<NK>([&](auto sc) {
+          constexpr int s = decltype(sc)::value;
+          constexpr int byte = t * (D / 32) + 2 * s;
           const v8i_t kf = frag16(tile + (32 * t + r) * (D / 2) + 32 * s + 16 * h);
-          const int ksc = h ? ksblk[t * (D / 32) + 2 * s + 1] : ksblk[t * (D / 32) + 2 * s];
-          S[t] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(kf, qf[s], S[t], 4, 4, 0, ksc, 0, qsc[s]);
-        }
-      }
+          S[t] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(kf, qf[s], S[t], 4, 4, byte % 4, ksh[byte / 4], 0, qsc[s]);
+        });
+      });
       // ---- mask (only blocks the diagonal crosses), running max kept in the base-2 domain: m = max(S) * sm_scale * log2(e)
       if (a.causal && key0 + 63 > q0 + shift) {
         asm volatile("" ::: "memory");   // keep this a branch: most blocks skip it
@@ -168,7 +199,7 @@ __global__ __launch_bounds__(256, ATTN_WG_PER_CU) void attn_fwd_kernel(AttnArgs 
       for (int t = 0; t < 2; ++t)
 #pragma unroll
         for (int v = 0; v < 16; ++v) mx = fmaxf(mx, S[t][v]);
-      mx = fmaxf(mx, xor32(mx));
+      mx = pair_max(mx);
       const float m_new = fmaxf(m_i, mx * c2);
       const float alpha = __builtin_amdgcn_exp2f(m_i - m_new);
       m_i = m_new;
@@ -184,7 +215,7 @@ __global__ __launch_bounds__(256, ATTN_WG_PER_CU) void attn_fwd_kernel(AttnArgs 
           S[t][v] = __builtin_amdgcn_exp2f(__builtin_fmaf(S[t][v], c2, -m_new));
           am = fmaxf(am, S[t][v]);
         }
-        am = fmaxf(am, xor32(am));
+        am = pair_max(am);
         const uint32_t e = e8m0_from_f32_bits(f2u(am));
         psc[t] = (int)e;
         const float scale_f = u2f(e << 23);
@@ -198,16 +229,14 @@ __global__ __launch_bounds__(256, ATTN_WG_PER_CU) void attn_fwd_kernel(AttnArgs 
           c[t][w] = o;
         }
       }
-      // Lane (r, h) multiplies tile h of this block: it keeps its half of tile h and gets the other half from lane
-      // (r, 1 - h), which in turn needs this lane's half of tile 1 - h.
-      uint32_t keep[2], recv[2];
-#pragma unroll
-      for (int w = 0; w < 2; ++w) {
-        keep[w] = h ? c[1][w] : c[0][w];
-        recv[w] = xor32(h ? c[0][w] : c[1][w]);
-      }
-      const v8i_t pf = v8i_t{(int)__builtin_amdgcn_perm(recv[0], keep[0], sel_lo), (int)__builtin_amdgcn_perm(recv[0], keep[0], sel_hi),
-                             (int)__builtin_amdgcn_perm(recv[1], keep[1], sel_lo), (int)__builtin_amdgcn_perm(recv[1], keep[1], sel_hi),
+      // Lane (r, h) multiplies tile h of this block and needs that tile's 32 codes of row r in key order; it holds the
+      // keys 8 g + 4 h + (0..3) of both tiles.  One half-wave swap per dword hands lane (r, 0) the tile-0 codes of lane
+      // (r, 1) and lane (r, 1) the tile-1 codes of lane (r, 0); in both halves the swapped pair is then {keys 8 g + 0..3,
+      // keys 8 g + 4..7} = {p[0], p[1]}, interleaved 16 bits at a time.
+      const v2u_t p0 = __builtin_amdgcn_permlane32_swap(c[0][0], c[1][0], false, false);
+      const v2u_t p1 = __builtin_amdgcn_permlane32_swap(c[0][1], c[1][1], false, false);
+      const v8i_t pf = v8i_t{(int)__builtin_amdgcn_perm(p0[1], p0[0], 0x05040100u), (int)__builtin_amdgcn_perm(p0[1], p0[0], 0x07060302u),
+                             (int)__builtin_amdgcn_perm(p1[1], p1[0], 0x05040100u), (int)__builtin_amdgcn_perm(p1[1], p1[0], 0x07060302u),
                              0, 0, 0, 0};
       const int pscale = h ? psc[1] : psc[0];
 
@@ -220,12 +249,13 @@ __global__ __launch_bounds__(256, ATTN_WG_PER_CU) void attn_fwd_kernel(AttnArgs 
           for (int v = 0; v < 16; ++v) acc_o[d][v] *= alpha;
       }
       acc_l = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ones, pf, acc_l, 4, 4, 0, 127, 0, pscale);
-#pragma unroll
-      for (int d = 0; d < ND; ++d) {
+      // V scale of (key tile h, column block d) = byte h Dv/32 + d
+      const int vsh = DV == 128 ? (int)(h ? vsw[VS_DW - 1] : vsw[0]) : (int)(vsw[0] >> (16 * h));
+      static_for<ND>([&](auto dc) {
+        constexpr int d = decltype(dc)::value;
         const v8i_t vf = frag16(tile + K_BYTES + (32 * d + r) * 32 + 16 * h);
-        const int vsc = h ? vsblk[d * (a.Sk / 32) + 1] : vsblk[d * (a.Sk / 32)];
-        acc_o[d] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(vf, pf, acc_o[d], 4, 4, 0, vsc, 0, pscale);
-      }
+        acc_o[d] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(vf, pf, acc_o[d], 4, 4, d, vsh, 0, pscale);
+      });
     }
     if (kb + 1 < wg_blk) park((kb + 1) & 1);
     __syncthreads();
@@ -287,6 +317,7 @@ extern "C" int alto_mxfp4_attention_fwd(const void* q_codes, const void* q_scale
   ALTO_REQUIRE(B * Hq * Sq * (D > Dv ? D : Dv) < (1ll << 40), "attention_fwd: tensor too large");
   ALTO_REQUIRE(((uintptr_t)q_codes | (uintptr_t)k_codes | (uintptr_t)vt_codes) % 16 == 0 && (uintptr_t)out % 8 == 0,
                "attention_fwd: code pointers must be 16-byte aligned, out 8-byte aligned");
+  ALTO_REQUIRE(((uintptr_t)k_scales | (uintptr_t)v_scales) % 4 == 0, "attention_fwd: K and V scale pointers must be 4-byte aligned");
   AttnArgs a{(const uint8_t*)q_codes, (const uint8_t*)q_scales, (const uint8_t*)k_codes, (const uint8_t*)k_scales,
              (const uint8_t*)vt_codes, (const uint8_t*)v_scales, out, lse, (int)Hq, (int)Hk, (int)Sq, (int)Sk, sm_scale, causal ? 1 : 0};
   hipStream_t st = (hipStream_t)stream;

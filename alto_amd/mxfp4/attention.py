@@ -23,7 +23,7 @@ def attention_mxfp4_forward(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, q
     """Pre-quantised operands -> (out bf16 [B,Hq,Sq,Dv], lse fp32 [B,Hq,Sq]).
 
     q [B,Hq,Sq,D/2], q_scale [B,Hq,Sq/32,D/32]; k [B,Hk,Sk,D/2], k_scale [B,Hk,Sk/32,D/32]; v packed along the keys:
-    [B,Hk,Dv,Sk/2] with v_scale [B,Hk,Dv/32,Sk/32] (the reference's kernel takes V packed along Dv and unpacks it inside
+    [B,Hk,Dv,Sk/2] with v_scale [B,Hk,Sk/32,Dv/32] (the reference's kernel takes V packed along Dv and unpacks it inside
     ``tl.dot_scaled(..., rhs_k_pack=False)``, :393; same codes, other byte order).
     """
     rt.require_gpu(q, k, v, q_scale, k_scale, v_scale)
@@ -34,7 +34,7 @@ def attention_mxfp4_forward(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, q
     Dv = v.shape[2]
     assert k.shape == (B, Hk, Sk, D // 2) and v.shape == (B, Hk, Dv, Sk // 2)
     assert q_scale.shape == (B, Hq, Sq // 32, D // 32) and k_scale.shape == (B, Hk, Sk // 32, D // 32)
-    assert v_scale.shape == (B, Hk, Dv // 32, Sk // 32)
+    assert v_scale.shape == (B, Hk, Sk // 32, Dv // 32)
     out = torch.empty((B, Hq, Sq, Dv), dtype=torch.bfloat16, device=q.device)
     lse = torch.empty((B, Hq, Sq), dtype=torch.float32, device=q.device)
     check(rt.lib().alto_mxfp4_attention_fwd(q.data_ptr(), q_scale.data_ptr(), k.data_ptr(), k_scale.data_ptr(), v.data_ptr(),
@@ -53,7 +53,9 @@ def quantize_qkv(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor):
     def cols(t):
         t3 = _prep(t.reshape(-1, t.shape[-2], t.shape[-1]))
         _, _, codes, scales = _quantize_call(t3, False, True, True, False, None, None, 0, False)
-        return codes.view(*t.shape[:-2], t.shape[-1], t.shape[-2] // 2), scales.view(*t.shape[:-2], t.shape[-1] // 32, t.shape[-2] // 32)
+        # the block scales go back to the [S/32, D/32] order of the tensor itself (a few KB; 2D-block scales are symmetric)
+        scales = scales.view(*t.shape[:-2], t.shape[-1] // 32, t.shape[-2] // 32).transpose(-1, -2).contiguous()
+        return codes.view(*t.shape[:-2], t.shape[-1], t.shape[-2] // 2), scales
 
     qq, qs = rows(q)
     kq, ks = rows(k)

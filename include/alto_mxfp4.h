@@ -206,9 +206,10 @@ int alto_mxfp4_qdq(const void* x, int dtype, int64_t batch, int64_t M, int64_t C
  * out = O / l as bf16 [B][Hq][Sq][Dv], lse = m + ln(l) as f32 [B][Hq][Sq].
  * q_codes [B][Hq][Sq][D/2], q_scales [B][Hq][Sq/32][D/32]; k_codes [B][Hk][Sk][D/2], k_scales [B][Hk][Sk/32][D/32]:
  * 2D-block quantisations of Q and K along D (mxfp_quantization.py:410-484, is_2d_block=True).  V is the same 2D-block
- * quantisation of [Sk][Dv], handed over packed along the keys: vt_codes [B][Hk][Dv][Sk/2], v_scales [B][Hk][Dv/32][Sk/32]
- * (the column outputs of alto_mxfp4_quantize).  Hq % Hk == 0 (grouped-query heads), D in {64,128,192,256},
- * Dv in {64,128}, Sq % 32 == 0, Sk % 64 == 0, causal needs Sq <= Sk.  All tensors dense.
+ * quantisation of [Sk][Dv], codes handed over packed along the keys (the column codes of alto_mxfp4_quantize):
+ * vt_codes [B][Hk][Dv][Sk/2], v_scales [B][Hk][Sk/32][Dv/32].  K and V scale pointers 4-byte aligned, code pointers
+ * 16-byte aligned.  Hq % Hk == 0 (grouped-query heads), D in {64,128,192,256}, Dv in {64,128}, Sq % 32 == 0,
+ * Sk % 64 == 0, causal needs Sq <= Sk.  All tensors dense.
  */
 int alto_mxfp4_attention_fwd(const void* q_codes, const void* q_scales, const void* k_codes, const void* k_scales,
                              const void* vt_codes, const void* v_scales, void* out, float* lse, int64_t B, int64_t Hq,
