@@ -422,11 +422,15 @@ extern "C" int alto_mxfp4_quantize_pitched(const void* x, int dtype, int64_t bat
   }
   ALTO_REQUIRE(!hadamard || (!is_2d && do_col), "quantize: the Hadamard transform applies to a 1D column output only");
   ALTO_REQUIRE(clip_mode == ALTO_CLIP_NONE || clip_mode == ALTO_CLIP_STATIC || clip_mode == ALTO_CLIP_DYNAMIC, "quantize: bad clip_mode %d", clip_mode);
-  if (clip_mode == ALTO_CLIP_DYNAMIC) {
-    set_error("quantize: clip_mode=dynamic is not implemented");
-    return ALTO_MXFP4_ENOTIMPL;
-  }
   if (batch == 0 || M == 0 || C == 0) return ALTO_MXFP4_OK;
+  if (clip_mode == ALTO_CLIP_DYNAMIC) {   // std-based scale: separate plain kernel, quantisation along the contiguous dim
+    ALTO_REQUIRE(do_row && !do_col && !hadamard && !use_uos,
+                 "quantize: clip_mode=dynamic gives the row output only (no column output, Hadamard or UOS); transpose on the host");
+    ALTO_REQUIRE(ld_row_codes % 16 == 0, "quantize: clip_mode=dynamic needs 16-byte aligned code rows");
+    ALTO_REQUIRE((M + 31) / 32 <= 65535, "quantize: M (%lld) exceeds 65535 row blocks", (long long)M);
+    return quantize_dynamic_launch(x, dtype, batch, M, C, ld_x, bs_x, row_codes, row_scales, ld_row_codes, is_2d, rounding == ALTO_ROUND_SR,
+                                   rand_bits, ld_rand, bs_rand, reinterpret_cast<hipStream_t>(stream));
+  }
 
   QuantParams p;
   p.x = x; p.ld_x = ld_x; p.bs_x = bs_x; p.M = (int)M; p.C = (int)C;

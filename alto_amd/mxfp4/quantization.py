@@ -147,6 +147,8 @@ def convert_to_mxfp4(
         rand_bits = _as_i32(rand_bits)
     if hadamard is not None:
         assert nd == 2 and ax == 0 and not is_2d_block, "hadamard fuses with a 1D axis=-2 quantisation of a 2D tensor"
+    if clip_mode == "dynamic" and data_hp.numel() != 0:
+        return _convert_dynamic(data_hp, ax, is_2d_block, use_sr, rand_bits, hadamard, use_uos)
 
     if data_hp.numel() == 0:
         xt = data_hp.transpose(ax, -1)
@@ -194,6 +196,28 @@ def convert_to_mxfp4(
     return codes.transpose(ax, -1), scales.transpose(ax, -1)
 
 
+def _convert_dynamic(x: torch.Tensor, ax: int, is_2d_block: bool, use_sr: bool, rand_bits: Optional[torch.Tensor],
+                     hadamard: Optional[HadamardTransform], use_uos: bool):
+    """``clip_mode="dynamic"`` (std-based scale, mxfp_quantization.py:54-59,65-70): an optional knob served by a plain
+    kernel that quantises along the contiguous dim; other axes are brought there with a copy, a Hadamard transform runs
+    as its own launch first."""
+    if use_uos:
+        raise NotImplementedError("clip_mode='dynamic' together with use_uos is not implemented")
+    if hadamard is not None:
+        x = hadamard_left(x, hadamard)
+    xt = x.transpose(ax, -1)
+    shp = xt.shape
+    rows = shp[-2] if (is_2d_block and len(shp) >= 2) else 1
+    x3 = xt.contiguous().reshape(-1, rows, shp[-1]) if is_2d_block else xt.contiguous().reshape(1, -1, shp[-1])
+    r3 = None
+    if use_sr:
+        r3 = rand_bits.transpose(ax, -1).contiguous().reshape(x3.shape)
+    codes, scales, _, _ = _quantize_call(x3, True, False, is_2d_block, use_sr, r3, None, rt.CLIP["dynamic"], False)
+    codes = codes.reshape(*shp[:-1], shp[-1] // 2)
+    scales = scales.reshape(*shp[:-2], shp[-2] // 32, shp[-1] // 32) if is_2d_block else scales.reshape(*shp[:-1], shp[-1] // 32)
+    return codes.transpose(ax, -1), scales.transpose(ax, -1)
+
+
 def quantize_rowcol(
     x: torch.Tensor,
     is_2d_block: bool = False,
@@ -217,11 +241,16 @@ def quantize_rowcol(
     M, C = x.shape
     torch._check(M % 32 == 0 and C % 32 == 0)
     clip = _clip_code(clip_mode)
+    if use_sr and rand_bits is None:
+        rand_bits = rt.draw_rand_bits(x.shape, x.device)
+    if clip_mode == "dynamic":   # the row pair is never clipped; the column pair takes the plain path
+        rc, rs = convert_to_mxfp4(x, axis=-1, is_2d_block=is_2d_block, use_sr=use_sr, use_uos=use_uos, rand_bits=rand_bits)
+        cc, cs = convert_to_mxfp4(x, axis=0, is_2d_block=is_2d_block, use_sr=use_sr, clip_mode="dynamic", use_uos=use_uos,
+                                  rand_bits=rand_bits, hadamard=hadamard)
+        return rc, rs, cc, cs
     x3 = _prep(x)
     r3 = None
     if use_sr:
-        if rand_bits is None:
-            rand_bits = rt.draw_rand_bits(x.shape, x.device)
         assert rand_bits.shape == x.shape
         r3 = _as_i32(rand_bits)
         r3 = _batched_view(r3 if r3.stride(-1) == 1 and r3.stride(0) % 4 == 0 and r3.data_ptr() % 16 == 0 else r3.contiguous())

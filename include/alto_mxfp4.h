@@ -40,7 +40,7 @@ extern "C" {
 /* clip modes (mxfp_quantization.py:428-438) */
 #define ALTO_CLIP_NONE 0
 #define ALTO_CLIP_STATIC 1
-#define ALTO_CLIP_DYNAMIC 2
+#define ALTO_CLIP_DYNAMIC 2 /* std-based scale (:54-59,65-70): row output only, no Hadamard, no UOS */
 
 int alto_mxfp4_version(void);
 const char* alto_mxfp4_last_error(void);

@@ -109,13 +109,35 @@ def block_scales(x2d: torch.Tensor, is_2d_block: bool = False, clip_mode: str = 
     """Scales of a quant-axis-last 2D tensor: [R, C/32] (1D) or [R/32, C/32] (2D). mxfp_quantization.py:28-95."""
     blk = _block_view(x2d, is_2d_block)
     if clip_mode == "dynamic":
-        # mxfp_quantization.py:54-59,65-70 (statistics taken in fp32 as Triton promotes bf16*bf16 sums)
-        b = blk.float()
-        n = b.shape[-1]
-        mean_sq = (b * b).sum(-1) / n
-        mean = b.sum(-1) / n
+        # mxfp_quantization.py:54-59,65-70.  The squares are rounded to the input dtype (an elementwise product of bf16
+        # tensors is bf16), the sums run in fp32 (Triton promotes bf16 reductions).  The ORDER of the fp32 sums is left
+        # to Triton's reduction in the reference; it is fixed here: the 32 elements of a block row in index order, then
+        # (2D) the 32 row sums in row order.  Multiply and add of the max_abs formula round separately, as in the
+        # reference's PyTorch twin (tests/unittest/mxfp4/utils.py:320-325).  Parity with the Triton kernel's own order of
+        # additions is unpinned (it could not be run); the HIP kernel follows THIS order bit for bit.
+        R, C = x2d.shape
+        xr = x2d.reshape(R, C // BLOCK, BLOCK)
+        xf = xr.float()
+        sq = (xr * xr).float()
+        s1 = torch.zeros(R, C // BLOCK, dtype=torch.float32)
+        s2 = torch.zeros(R, C // BLOCK, dtype=torch.float32)
+        for i in range(BLOCK):
+            s1 = s1 + xf[..., i]
+            s2 = s2 + sq[..., i]
+        n = float(BLOCK)
+        if is_2d_block:
+            s1 = s1.reshape(R // BLOCK, BLOCK, C // BLOCK)
+            s2 = s2.reshape(R // BLOCK, BLOCK, C // BLOCK)
+            t1 = torch.zeros(R // BLOCK, C // BLOCK, dtype=torch.float32)
+            t2 = torch.zeros(R // BLOCK, C // BLOCK, dtype=torch.float32)
+            for j in range(BLOCK):
+                t1 = t1 + s1[:, j]
+                t2 = t2 + s2[:, j]
+            s1, s2, n = t1, t2, float(BLOCK * BLOCK)
+        mean_sq = s2 / n
+        mean = s1 / n
         std = torch.sqrt(mean_sq - mean * mean)
-        absmax = ((2.92247856 / 6.0) * std + 1e-8).to(x2d.dtype)
+        absmax = (torch.tensor(2.92247856 / 6.0, dtype=torch.float32) * std + torch.tensor(1e-8, dtype=torch.float32)).to(x2d.dtype)
         return e8m0_from_absmax(absmax, use_uos=use_uos, target_max_pow2=0)
     absmax = blk.abs().amax(dim=-1)  # exact in any dtype
     return e8m0_from_absmax(absmax, use_uos=use_uos)

@@ -136,6 +136,38 @@ def test_linear_autograd(m, shape, use_2dblock_x, use_2dblock_w, use_sr, use_h, 
         assert snr_db(gf.T @ xf, wg.grad) > floor
 
 
+@pytest.mark.parametrize("use_sr", [False, True])
+@pytest.mark.parametrize("use_h", [False, True])
+def test_linear_autograd_dynamic_clip(m, use_sr, use_h):
+    """clip_mode="dynamic": the wgrad operands (axis-0 copies of x and dY) take the std-based scale, the rest is unchanged
+    (mxfp_linear.py:383-396,466-494); parity with the oracle's flow."""
+    B, M, N, K = 2, 256, 384, 512
+    x = randn_outliers((B, M, K), torch.bfloat16, seed=41)
+    w = randn_outliers((N, K), torch.bfloat16, seed=42)
+    go = randn_outliers((B, M, N), torch.bfloat16, seed=43) / 1000
+    signs, perm = hadamard_from_seed(1234)
+    had = (signs, perm) if use_h else None
+    r = rand_bits((B * M, N), seed=78)
+    m.set_rand_bits_source(lambda shp, d: r.to(d))
+    try:
+        xg = x.to(DEV).requires_grad_(True)
+        wg = w.to(DEV).requires_grad_(True)
+        h = m.HadamardTransform(signs, perm) if use_h else None
+        y = m.MXFP4LinearFunction.apply(xg, wg, False, True, use_sr, False, "dynamic", False, h, False)
+        y.backward(go.to(DEV))
+    finally:
+        m.set_rand_bits_source(None)
+    y_ref, saved = O.linear_forward_ref(x, w, False, True, hadamard=had, clip_mode="dynamic")
+    dx_ref, dw_ref = O.linear_backward_ref(go.reshape(-1, N), saved, False, True, use_sr_grad=use_sr, rand_bits=r, hadamard=had, clip_mode="dynamic")
+    assert O.rel_frobenius(y.detach().cpu().reshape(-1, N), y_ref) < 4e-3
+    assert O.rel_frobenius(xg.grad.cpu().reshape(-1, K), dx_ref) < 4e-3
+    assert O.rel_frobenius(wg.grad.cpu(), dw_ref) < 4e-3
+    # and it differs from the unclipped flow only in dW
+    _, saved0 = O.linear_forward_ref(x, w, False, True, hadamard=had)
+    _, dw0 = O.linear_backward_ref(go.reshape(-1, N), saved0, False, True, use_sr_grad=use_sr, rand_bits=r, hadamard=had)
+    assert O.rel_frobenius(wg.grad.cpu(), dw0) > 1e-2
+
+
 def test_to_mxfp4_then_scaled_mm_recipe_path(m):
     """The function the weight wrapper dispatches F.linear to (alto/kernels/dispatch/tensor.py:284-295), production flags."""
     x = randn_outliers((2, 128, 256), torch.bfloat16, seed=1).to(DEV).requires_grad_(True)

@@ -216,8 +216,40 @@ def test_edge_cases(m):
     _check_pair(m.convert_to_mxfp4(xt.to(DEV).T.contiguous().T, axis=-1), O.quantize(xt, axis=-1), "transposed input")
     with pytest.raises(RuntimeError):
         m.convert_to_mxfp4(torch.zeros(32, 48, device=DEV))
-    with pytest.raises(NotImplementedError):
-        m.convert_to_mxfp4(torch.zeros(32, 64, device=DEV), clip_mode="dynamic")
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("is_2d", [False, True])
+@pytest.mark.parametrize("use_sr", [False, True])
+@pytest.mark.parametrize("axis", [-1, 0])
+def test_dynamic_clip(m, dtype, is_2d, use_sr, axis):
+    """clip_mode="dynamic" (std-based scale, mxfp_quantization.py:54-59,65-70): bit-equal to the CPU model, whose order of
+    the fp32 sums is the kernel's (the reference leaves it to Triton's reduction: parity with that order is unpinned)."""
+    x = randn_outliers((96, 160), dtype, seed=31)
+    r = rand_bits((96, 160), seed=32) if use_sr else None
+    got = m.convert_to_mxfp4(x.to(DEV), axis=axis, is_2d_block=is_2d, use_sr=use_sr, clip_mode="dynamic",
+                             rand_bits=None if r is None else r.to(DEV))
+    exp = O.quantize(x, axis=axis, is_2d_block=is_2d, use_sr=use_sr, rand_bits=r, clip_mode="dynamic")
+    _check_pair(got, exp, "dynamic clip")
+    # the clip does something: scales differ from the absmax rule somewhere
+    plain = O.quantize(x, axis=axis, is_2d_block=is_2d, use_sr=use_sr, rand_bits=r)
+    assert not torch.equal(exp[1], plain[1])
+
+
+def test_dynamic_clip_edge_blocks_and_hadamard(m):
+    # a constant block has zero variance: max_abs = 1e-8, everything saturates; a zero block likewise gets scale byte 100
+    x = torch.cat([torch.full((32, 64), 3.0), torch.zeros(32, 64), randn_outliers((32, 64), torch.float32, seed=5)]).to(torch.bfloat16)
+    _check_pair(m.convert_to_mxfp4(x.to(DEV), clip_mode="dynamic"), O.quantize(x, clip_mode="dynamic"), "constant / zero blocks")
+    # column copy of the linear layer: Hadamard along the rows, then dynamic clip along axis 0; row copy unclipped
+    g = torch.Generator().manual_seed(3)
+    signs = (torch.randint(0, 2, (32,), generator=g) * 2 - 1).to(torch.int8)
+    perm = torch.randperm(32, generator=g)
+    h = m.HadamardTransform(signs, perm)
+    x = randn_outliers((64, 96), torch.bfloat16, seed=6)
+    r = rand_bits((64, 96), seed=7)
+    rc, rs, cc, cs = m.quantize_rowcol(x.to(DEV), False, use_sr=True, rand_bits=r.to(DEV), hadamard=h, clip_mode="dynamic")
+    _check_pair((rc, rs), O.quantize(x, axis=-1, use_sr=True, rand_bits=r), "row copy")
+    _check_pair((cc, cs), O.quantize(O.rht_left(x, signs, perm), axis=0, use_sr=True, rand_bits=r, clip_mode="dynamic"), "column copy")
 
 
 def test_padded_code_rows_hold_the_same_bytes(m):

@@ -37,8 +37,8 @@ def test_argument_validation_needs_no_gpu():
     p += (-p) % 16
     rc = lib.alto_mxfp4_quantize(p, 0, 1, 32, 40, 40, 1280, p, p, None, None, 0, 0, None, 0, 0, 0, None, None, 0, 0, None)
     assert rc == -1 and b"C (40)" in lib.alto_mxfp4_last_error()
-    rc = lib.alto_mxfp4_quantize(p, 0, 1, 32, 32, 32, 1024, p, p, None, None, 0, 0, None, 0, 0, 0, None, None, 2, 0, None)
-    assert rc == -3  # dynamic clip: declared, not implemented
+    rc = lib.alto_mxfp4_quantize(p, 0, 1, 32, 32, 32, 1024, p, p, p, p, 0, 0, None, 0, 0, 0, None, None, 2, 0, None)
+    assert rc == -1 and b"row output only" in lib.alto_mxfp4_last_error()   # dynamic clip quantises along the contiguous dim
     rc = lib.alto_mxfp4_gemm(p, 16, p, 1, 1, 0, p, 16, p, 1, 1, 0, 32, 32, 48, p, 0, 32, 1.0, None)
     assert rc == -1 and b"K (48)" in lib.alto_mxfp4_last_error()
     bad_perm = (ctypes.c_uint8 * 32)(*([0] * 32))
