@@ -112,22 +112,25 @@ __device__ __forceinline__ int clamp_off(const int32_t* offs, int g, int64_t M_t
   return (int)(v < 0 ? 0 : (v > M_total ? M_total : v));
 }
 
-// Same XCD-aware tile order as the dense kernel: an XCD works on 8 neighbouring N-tiles of one band of rows at a time.
+// Tile order of the grouped kernels.  As in the dense kernel an XCD (wg % 8) works on 8 neighbouring N-tiles of a few row
+// bands at a time, so its L2 shares the A rows and the expert's weight rows; but the row bands are dealt to the XCDs
+// round-robin (band tm belongs to XCD tm % 8) instead of in contiguous ranges: a band that an expert boundary cuts runs
+// once per segment, such bands cluster where the small experts sit, and contiguous ranges left one XCD with most of them.
 __device__ __forceinline__ bool grouped_tile_coords(int wg, int tiles_m, int tiles_n, int& tm, int& tn) {
-  const int T = tiles_m * tiles_n;
-  const int per_xcd = (T + 7) / 8;
-  const int u = (wg & 7) * per_xcd + (wg >> 3);
-  if ((wg >> 3) >= per_xcd || u >= T) return false;
+  const int k = wg & 7, j = wg >> 3;
+  const int nb = (tiles_m - k + 7) / 8;          // bands of this XCD
+  if (nb <= 0 || j >= nb * tiles_n) return false;
   const int GN = 8;
-  const int in_group = GN * tiles_m;
-  const int group = u / in_group;
+  const int group = j / (GN * nb);
   const int first_n = group * GN;
   const int gsize = (tiles_n - first_n) < GN ? (tiles_n - first_n) : GN;
-  const int w = u % in_group;
+  const int w = j - group * GN * nb;
   tn = first_n + w % gsize;
-  tm = w / gsize;
+  tm = k + 8 * (w / gsize);
   return true;
 }
+// workgroups to launch for that order: 8 x the tile count of the XCD with the most bands
+__host__ __device__ inline int64_t grouped_grid_size(int64_t tiles_m, int64_t tiles_n) { return 8 * ((tiles_m + 7) / 8) * tiles_n; }
 
 template <typename OutT>
 __device__ __forceinline__ void zero_rows(OutT* out, int64_t ldo, int64_t r0, int64_t r1, int64_t n0, int64_t n1) {
@@ -312,8 +315,7 @@ int launch_grouped_tiled(const OperandView& A, const uint8_t* w, int64_t w_strid
     attr_set = true;
   }
   const int tiles_m = (int)((M_total + GT_TM - 1) / GT_TM), tiles_n = (int)((N + GT_TN - 1) / GT_TN);
-  const int per_xcd = (tiles_m * tiles_n + 7) / 8;
-  hipLaunchKernelGGL(kern, dim3((unsigned)(per_xcd * 8)), dim3(GT_THREADS), GT_LDS_BYTES, st, A, w, w_stride_e, ldw, w_scales, ws_stride_e, ws_r,
+  hipLaunchKernelGGL(kern, dim3((unsigned)grouped_grid_size(tiles_m, tiles_n)), dim3(GT_THREADS), GT_LDS_BYTES, st, A, w, w_stride_e, ldw, w_scales, ws_stride_e, ws_r,
                      w_is_2d, offs, group_expert, num_groups, num_experts, M_total, N, (int)(K / 32), (OutT*)out, ldo, tiles_m, tiles_n);
   return 0;
 }
@@ -328,8 +330,7 @@ int launch_dw_tiled(const OperandView& P, const OperandView& Q, int64_t NP, int6
     attr_set = true;
   }
   const int tiles_p = (int)((NP + GT_TM - 1) / GT_TM), tiles_q = (int)((NQ + GT_TN - 1) / GT_TN);
-  const int per_xcd = (tiles_p * tiles_q + 7) / 8;
-  hipLaunchKernelGGL(kern, dim3((unsigned)(per_xcd * 8), (unsigned)num_experts), dim3(GT_THREADS), GT_DW_LDS_BYTES, st, P, Q, NP, NQ, offs,
+  hipLaunchKernelGGL(kern, dim3((unsigned)grouped_grid_size(tiles_p, tiles_q), (unsigned)num_experts), dim3(GT_THREADS), GT_DW_LDS_BYTES, st, P, Q, NP, NQ, offs,
                      group_expert, num_groups, M_total, (OutT*)dw, s_e, ld, out_scale, tiles_p, tiles_q);
   return 0;
 }
