@@ -163,3 +163,37 @@ def test_dge_grouped_weight_gradient(m):
     assert torch.equal(grads[True][0], grads[False][0])
     torch.testing.assert_close(grads[True][1], grads[False][1] * 0.2, rtol=4e-7, atol=0)
     assert grads[False][1].abs().max() > 0
+
+
+def test_registered_torch_ops_run_the_hip_kernels(m):
+    """torch.ops.<ns>.* (the reference registers these names as torchtitan::*) give the direct functions' results."""
+    ns = m.register_torch_ops("alto_amd_test")
+    x = randn_outliers((128, 256), torch.bfloat16, seed=51).to(DEV)
+    w = (randn_outliers((192, 256), torch.bfloat16, seed=52) * 0.02).to(DEV)
+    xq, xs = ns.convert_to_mxfp4(x)
+    xq2, xs2 = m.convert_to_mxfp4(x)
+    assert torch.equal(xq, xq2) and torch.equal(xs, xs2)
+    cq, cs = ns.convert_to_mxfp4(x, 32, 0, False)
+    cq2, cs2 = m.convert_to_mxfp4(x, axis=0)
+    assert cq.shape == cq2.shape and cq.stride() == cq2.stride() and torch.equal(cq, cq2) and torch.equal(cs, cs2)
+    wq, ws = ns.convert_to_mxfp4(w, 32, -1, True)
+    assert torch.equal(ns.convert_from_mxfp4(wq, ws, torch.bfloat16, 32, -1, True), m.convert_from_mxfp4(wq, ws, torch.bfloat16, is_2d_block=True))
+    y = ns.blockwise_mxfp4_gemm(xq, xs, wq, ws, False, True, True, True, False, True, 32, torch.bfloat16)
+    assert torch.equal(y, m.blockwise_mxfp4_gemm(xq, xs, wq, ws, use_2dblock_b=True, trans_b=True, output_dtype=torch.bfloat16))
+    # grouped: 2 experts x 128 rows
+    idx = (torch.arange(256, device=DEV, dtype=torch.int32) // 128)
+    a = randn_outliers((256, 256), torch.bfloat16, seed=53).to(DEV)
+    ew = (randn_outliers((2, 192, 256), torch.bfloat16, seed=54) * 0.02).to(DEV)
+    aq, as_ = m.convert_to_mxfp4(a)
+    ewq, ews = m.convert_to_mxfp4(ew, is_2d_block=True)
+    out = ns.mxfp4_grouped_gemm_forward(aq, ewq, idx, as_, ews)
+    assert torch.equal(out, m.mxfp4_grouped_gemm_forward(aq, ewq, idx, as_, ews))
+    go = randn_outliers((256, 192), torch.bfloat16, seed=55).to(DEV) / 1000
+    gq, gs = m.convert_to_mxfp4(go)
+    wnq, wns = m.convert_to_mxfp4(ew, axis=-2, is_2d_block=True)               # packed along N: [E, N/2, K]
+    dx = ns.mxfp4_grouped_gemm_backward_inputs(gq, wnq, idx, gs, wns)
+    assert torch.equal(dx, m.mxfp4_grouped_gemm_backward_inputs(gq, wnq, idx, gs, wns)) and dx.shape == (256, 256)
+    gqm, gsm = m.convert_to_mxfp4(go, axis=0)
+    aqm, asm_ = m.convert_to_mxfp4(a, axis=0)
+    dw = ns.mxfp4_grouped_gemm_backward_weights(gqm, aqm, idx, 2, gsm, asm_, True, False, False)
+    assert torch.equal(dw, m.mxfp4_grouped_gemm_backward_weights(gqm, aqm, idx, 2, gsm, asm_, use_2dblock_x=False)) and dw.shape == (2, 192, 256)

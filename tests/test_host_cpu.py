@@ -138,3 +138,46 @@ def test_dge_factor_is_one_fifth_on_the_e2m1_grid():
     half, mid, x = np.float32(0.25), np.float32(1.25), np.float32(1.3)
     off = half ** np.float32(0.8) * np.abs(x - mid) ** np.float32(-0.8) / np.float32(5)
     assert abs(off - 0.2) > 0.1
+
+
+def test_torch_ops_registration_and_fake_shapes():
+    """The six operators exist under torch.ops with the reference's argument lists (mxfp_quantization.py:410,487,
+    mxfp_linear.py:142, cg_forward.py:200, cg_backward.py:398,500) and trace with fake tensors: shapes, dtypes and the
+    transposed-view strides of the quantiser outputs (mxfp_quantization.py:484)."""
+    import torch
+    from torch._subclasses.fake_tensor import FakeTensorMode
+    import alto_amd.mxfp4 as m
+    ns = m.register_torch_ops("alto_amd_test")
+    assert m.register_torch_ops("alto_amd_test") is ns
+    for name in ("convert_to_mxfp4", "convert_from_mxfp4", "blockwise_mxfp4_gemm", "mxfp4_grouped_gemm_forward",
+                 "mxfp4_grouped_gemm_backward_inputs", "mxfp4_grouped_gemm_backward_weights"):
+        assert hasattr(ns, name)
+    with FakeTensorMode():
+        x = torch.empty(4, 128, 64, dtype=torch.bfloat16)
+        c, s = ns.convert_to_mxfp4(x)
+        assert c.shape == (4, 128, 32) and s.shape == (4, 128, 2) and c.dtype == torch.uint8
+        c0, s0 = ns.convert_to_mxfp4(x, 32, -2, False)
+        assert c0.shape == (4, 64, 64) and s0.shape == (4, 4, 64) and c0.stride(-2) == 1      # memory [.., C][M/2]
+        c2, s2 = ns.convert_to_mxfp4(x, 32, -1, True)
+        assert c2.shape == (4, 128, 32) and s2.shape == (4, 4, 2)
+        y = ns.convert_from_mxfp4(c, s, torch.bfloat16)
+        assert y.shape == x.shape and y.dtype == torch.bfloat16
+        a, a_s = torch.empty(96, 64, dtype=torch.uint8), torch.empty(96, 4, dtype=torch.uint8)
+        b, b_s = torch.empty(160, 64, dtype=torch.uint8), torch.empty(5, 4, dtype=torch.uint8)
+        out = ns.blockwise_mxfp4_gemm(a, a_s, b, b_s, False, True, True, True, False, True, 32, torch.bfloat16)
+        assert out.shape == (96, 160) and out.dtype == torch.bfloat16
+        # wgrad form: token-packed operands [M/2, N] and [M/2, K], trans_a
+        gq, gs = torch.empty(64, 160, dtype=torch.uint8), torch.empty(4, 160, dtype=torch.uint8)
+        xq, xs = torch.empty(64, 96, dtype=torch.uint8), torch.empty(4, 96, dtype=torch.uint8)
+        dw = ns.blockwise_mxfp4_gemm(gq, gs, xq, xs, False, False, True, True, True, False)
+        assert dw.shape == (160, 96) and dw.dtype == torch.float32
+        idx = torch.empty(256, dtype=torch.int32)
+        inp, inp_s = torch.empty(256, 64, dtype=torch.uint8), torch.empty(256, 4, dtype=torch.uint8)
+        w, w_s = torch.empty(4, 160, 64, dtype=torch.uint8), torch.empty(4, 5, 4, dtype=torch.uint8)
+        assert ns.mxfp4_grouped_gemm_forward(inp, w, idx, inp_s, w_s).shape == (256, 160)
+        go, go_s = torch.empty(256, 80, dtype=torch.uint8), torch.empty(256, 5, dtype=torch.uint8)
+        wn, wn_s = torch.empty(4, 80, 128, dtype=torch.uint8), torch.empty(4, 5, 4, dtype=torch.uint8)
+        assert ns.mxfp4_grouped_gemm_backward_inputs(go, wn, idx, go_s, wn_s).shape == (256, 128)
+        gom, gom_s = torch.empty(128, 160, dtype=torch.uint8), torch.empty(8, 160, dtype=torch.uint8)
+        xm, xm_s = torch.empty(128, 128, dtype=torch.uint8), torch.empty(8, 128, dtype=torch.uint8)
+        assert ns.mxfp4_grouped_gemm_backward_weights(gom, xm, idx, 4, gom_s, xm_s, True, False, False).shape == (4, 160, 128)
