@@ -154,6 +154,7 @@ def mxfp4_grouped_gemm_backward_weights(grad_output, inputs, expert_indices, num
                       groups_from_indices(expert_indices), num_experts, output_dtype, trans_weights)
 
 
+@torch.compiler.allow_in_graph
 class MXFP4GroupedGEMM(torch.autograd.Function):
     """Grouped GEMM with full backward (cg_backward.py:599-930), recipe branch 1D activations / 2D weights."""
 

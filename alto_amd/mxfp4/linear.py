@@ -171,6 +171,7 @@ def _wgrad_scale(clip_mode: str, use_dge: bool) -> float:
     return s * DGE_FACTOR if use_dge else s
 
 
+@torch.compiler.allow_in_graph
 class MXFP4LinearFunction(torch.autograd.Function):
     """``y = x @ W^T`` with MXFP4 operands in forward and in both backward GEMMs (mxfp_linear.py:258-570).
 
