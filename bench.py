@@ -277,6 +277,49 @@ class AttentionFwd(Workload):
         return run, self.work * 4 / (self.B * self.HQ), "4 of 256 (batch, head) pairs at full sequence length"
 
 
+class LinearStep(Workload):
+    """Config 3 + 4 end to end: MXFP4LinearFunction forward and backward at the Llama-3-8B FFN shape (production flags:
+    1D activations, 2D weights, Hadamard on the wgrad operands, stochastic rounding of dY with supplied bits): three
+    quantizer passes over activations / gradients (plus the weight's unless cached) and three GEMMs per step."""
+    bound = "mfma"
+    kernel = "gemm"
+    M, K, N = 8192, 4096, 14336
+
+    def __init__(self, cached):
+        self.cached = cached
+        self.name = f"cfg3+4_linear_fwd_bwd[8192x4096->14336,{'cached' if cached else 'requantized'} weight]"
+        self.work = 3 * 2.0 * self.M * self.K * self.N
+
+    def setup(self, dev, gen):
+        import torch
+        import alto_amd.mxfp4 as m
+        self.m = m
+        self.x = torch.randn(self.M, self.K, device=dev, generator=gen).bfloat16().requires_grad_(True)
+        self.w = (torch.randn(self.N, self.K, device=dev, generator=gen) * 0.02).bfloat16().requires_grad_(True)
+        self.go = _laplace((self.M, self.N), 1e-3, dev, gen)
+        self.r = torch.randint(-2 ** 31, 2 ** 31 - 1, (self.M, self.N), device=dev, generator=gen, dtype=torch.int64).to(torch.int32)
+        g = torch.Generator().manual_seed(1234)
+        signs = (torch.randint(0, 2, (32,), generator=g) * 2 - 1).to(torch.int8)
+        self.h = m.HadamardTransform(signs, torch.randperm(32, generator=g))
+
+    def step(self):
+        m = self.m
+        m.enable_weight_cache(self.cached)
+        m.set_rand_bits_source(lambda shp, d: self.r)
+        try:
+            self.x.grad = self.w.grad = None
+            y = m.MXFP4LinearFunction.apply(self.x, self.w, False, True, True, False, "none", False, self.h, False)
+            y.backward(self.go)
+        finally:
+            m.set_rand_bits_source(None)
+            if not self.cached:
+                m.enable_weight_cache(False)
+        return y
+
+    def cpu_sample(self):
+        raise NotImplementedError("the end-to-end step is reported beside the per-kernel workloads, without its own CPU leg")
+
+
 class CopyCalibration(Workload):
     """Plain device copy of 256 MiB (torch's elementwise copy kernel): the known-size launch against which the
     FETCH_SIZE / WRITE_SIZE counters of the other kernels are scaled.  Not part of the product path."""
@@ -345,6 +388,8 @@ def make_workloads():
         "cfg4_wgrad": Gemm("cfg4_wgrad_gemm[4096x14336x8192]", 4096, 14336, 8192, False, False, "grad", "act"),
         "cfg5_grouped": GroupedGemm(),
         "attn_fwd": AttentionFwd(),
+        "linear_step": LinearStep(False),
+        "linear_step_cached": LinearStep(True),
         "copy_calib": CopyCalibration(),
         "mfma_probe_const": MfmaProbe(False),
         "mfma_probe_random": MfmaProbe(True),
@@ -414,7 +459,11 @@ def main():
         sys.exit(2)
     primary = wl[args.workload]
     res = measure(primary, dev, gen, args.steps, args.warmup)
-    cpu = None if args.no_cpu else cpu_baseline(primary)
+    try:
+        cpu = None if args.no_cpu else cpu_baseline(primary)
+    except NotImplementedError as e:   # a composite workload without a CPU leg of its own
+        print(f"bench.py: no cpu_baseline for {args.workload}: {e}", file=sys.stderr)
+        cpu = None
     others = {}
     if not args.only:
         for key, w in wl.items():
