@@ -18,7 +18,7 @@ struct AttnArgs {
   const uint8_t* k;  const uint8_t* ks;    // [B, Hk, Sk, D/2],  [B, Hk, Sk/32, D/32]
   const uint8_t* vt; const uint8_t* vs;    // [B, Hk, Dv, Sk/2] packed along keys, [B, Hk, Sk/32, Dv/32]
   void* out; float* lse;                   // [B, Hq, Sq, Dv] bf16, [B, Hq, Sq] fp32
-  int Hq, Hk, Sq, Sk;
+  int Hq, Hk, Sq, Sk, Sk_used;             // Sk keys are allocated (a multiple of 64), the first Sk_used exist
   float sm_scale;
   int causal;
 };
@@ -70,7 +70,7 @@ __global__ __launch_bounds__(256, ATTN_WG_PER_CU) void attn_fwd_kernel(AttnArgs 
   const int hk = hq / (a.Hq / a.Hk);
   const int64_t bhq = (int64_t)b * a.Hq + hq, bhk = (int64_t)b * a.Hk + hk;
   const int qrow = live ? q0 + r : 0;
-  const int shift = a.Sk - a.Sq;                  // causal mask is aligned to the bottom-right corner
+  const int shift = a.Sk_used - a.Sq;                  // causal mask is aligned to the bottom-right corner
 
   // ---- Q pieces: row qrow, K step ks, half h -> 16 bytes; one scale byte per (32-row block, 32-column block)
   v8i_t qf[NK];
@@ -94,7 +94,7 @@ __global__ __launch_bounds__(256, ATTN_WG_PER_CU) void attn_fwd_kernel(AttnArgs 
   const v8i_t ones = v8i_t{0x22222222, 0x22222222, 0x22222222, 0x22222222, 0, 0, 0, 0};   // E2M1 code 2 = 1.0
 
   // blocks this wave needs, and the most any wave of the workgroup needs (the last wave's rows reach furthest)
-  const int all_blk = a.Sk / 64;
+  const int all_blk = (a.Sk_used + 63) / 64;
   int nblk = all_blk, wg_blk = all_blk;
   if (a.causal) {
     const int lim = (q0 + 32 + shift + 63) / 64;
@@ -183,15 +183,15 @@ __global__ __launch_bounds__(256, ATTN_WG_PER_CU) void attn_fwd_kernel(AttnArgs 
           S[t] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(kf, qf[s], S[t], 4, 4, byte % 4, ksh[byte / 4], 0, qsc[s]);
         });
       });
-      // ---- mask (only blocks the diagonal crosses), running max kept in the base-2 domain: m = max(S) * sm_scale * log2(e)
-      if (a.causal && key0 + 63 > q0 + shift) {
+      // ---- mask (only blocks the diagonal crosses or that reach past the last key), running max kept in the base-2 domain: m = max(S) * sm_scale * log2(e)
+      if ((a.causal && key0 + 63 > q0 + shift) || key0 + 64 > a.Sk_used) {
         asm volatile("" ::: "memory");   // keep this a branch: most blocks skip it
 #pragma unroll
         for (int t = 0; t < 2; ++t)
 #pragma unroll
           for (int v = 0; v < 16; ++v) {
             const int key = key0 + 32 * t + 8 * (v >> 2) + 4 * h + (v & 3);
-            if (key > qrow + shift) S[t][v] = -__builtin_inff();
+            if ((a.causal && key > qrow + shift) || key >= a.Sk_used) S[t][v] = -__builtin_inff();
           }
       }
       float mx = -__builtin_inff();
@@ -303,8 +303,8 @@ static int launch_attn_nd(const AttnArgs& a, int B, int Dv, hipStream_t st) {
 
 extern "C" int alto_mxfp4_attention_fwd(const void* q_codes, const void* q_scales, const void* k_codes, const void* k_scales,
                                         const void* vt_codes, const void* v_scales, void* out, float* lse, int64_t B, int64_t Hq,
-                                        int64_t Hk, int64_t Sq, int64_t Sk, int64_t D, int64_t Dv, float sm_scale, int causal,
-                                        void* stream) {
+                                        int64_t Hk, int64_t Sq, int64_t Sk, int64_t Sk_used, int64_t D, int64_t Dv, float sm_scale,
+                                        int causal, void* stream) {
   using namespace alto;
   ALTO_REQUIRE(q_codes && q_scales && k_codes && k_scales && vt_codes && v_scales && out && lse, "attention_fwd: null pointer");
   ALTO_REQUIRE(B > 0 && Hq > 0 && Hk > 0 && Hq % Hk == 0, "attention_fwd: Hq=%lld must be a positive multiple of Hk=%lld", (long long)Hq, (long long)Hk);
@@ -312,14 +312,16 @@ extern "C" int alto_mxfp4_attention_fwd(const void* q_codes, const void* q_scale
   ALTO_REQUIRE(Sk > 0 && Sk % 64 == 0, "attention_fwd: Sk=%lld must be a positive multiple of 64", (long long)Sk);
   ALTO_REQUIRE(D == 64 || D == 128 || D == 192 || D == 256, "attention_fwd: head dim D=%lld must be 64, 128, 192 or 256", (long long)D);
   ALTO_REQUIRE(Dv == 64 || Dv == 128, "attention_fwd: value dim Dv=%lld must be 64 or 128", (long long)Dv);
-  ALTO_REQUIRE(!causal || Sq <= Sk, "attention_fwd: causal attention needs Sq <= Sk (got %lld > %lld)", (long long)Sq, (long long)Sk);
+  ALTO_REQUIRE(Sk_used > 0 && Sk_used <= Sk && Sk - Sk_used < 64 && Sk_used % 32 == 0,
+               "attention_fwd: Sk_used=%lld must be a multiple of 32 in (Sk - 64, Sk]", (long long)Sk_used);
+  ALTO_REQUIRE(!causal || Sq <= Sk_used, "attention_fwd: causal attention needs Sq <= Sk (got %lld > %lld)", (long long)Sq, (long long)Sk_used);
   ALTO_REQUIRE(B <= 65535 && Hq <= 65535, "attention_fwd: B and Hq must fit a grid dimension");
   ALTO_REQUIRE(B * Hq * Sq * (D > Dv ? D : Dv) < (1ll << 40), "attention_fwd: tensor too large");
   ALTO_REQUIRE(((uintptr_t)q_codes | (uintptr_t)k_codes | (uintptr_t)vt_codes) % 16 == 0 && (uintptr_t)out % 8 == 0,
                "attention_fwd: code pointers must be 16-byte aligned, out 8-byte aligned");
   ALTO_REQUIRE(((uintptr_t)k_scales | (uintptr_t)v_scales) % 4 == 0, "attention_fwd: K and V scale pointers must be 4-byte aligned");
   AttnArgs a{(const uint8_t*)q_codes, (const uint8_t*)q_scales, (const uint8_t*)k_codes, (const uint8_t*)k_scales,
-             (const uint8_t*)vt_codes, (const uint8_t*)v_scales, out, lse, (int)Hq, (int)Hk, (int)Sq, (int)Sk, sm_scale, causal ? 1 : 0};
+             (const uint8_t*)vt_codes, (const uint8_t*)v_scales, out, lse, (int)Hq, (int)Hk, (int)Sq, (int)Sk, (int)Sk_used, sm_scale, causal ? 1 : 0};
   hipStream_t st = (hipStream_t)stream;
   switch (D) {
     case 64: return launch_attn_nd<1>(a, (int)B, (int)Dv, st);

@@ -19,12 +19,13 @@ from .quantization import _prep, _quantize_call
 
 
 def attention_mxfp4_forward(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, q_scale: torch.Tensor, k_scale: torch.Tensor,
-                            v_scale: torch.Tensor, sm_scale: float, causal: bool) -> Tuple[torch.Tensor, torch.Tensor]:
+                            v_scale: torch.Tensor, sm_scale: float, causal: bool, seqlen_k: Optional[int] = None) -> Tuple[torch.Tensor, torch.Tensor]:
     """Pre-quantised operands -> (out bf16 [B,Hq,Sq,Dv], lse fp32 [B,Hq,Sq]).
 
     q [B,Hq,Sq,D/2], q_scale [B,Hq,Sq/32,D/32]; k [B,Hk,Sk,D/2], k_scale [B,Hk,Sk/32,D/32]; v packed along the keys:
     [B,Hk,Dv,Sk/2] with v_scale [B,Hk,Sk/32,Dv/32] (the reference's kernel takes V packed along Dv and unpacks it inside
-    ``tl.dot_scaled(..., rhs_k_pack=False)``, :393; same codes, other byte order).
+    ``tl.dot_scaled(..., rhs_k_pack=False)``, :393; same codes, other byte order).  The key dim of k / v is a multiple of
+    64; ``seqlen_k`` (default: all of it) says how many keys exist when the caller padded a sequence of 32 (mod 64) keys.
     """
     rt.require_gpu(q, k, v, q_scale, k_scale, v_scale)
     for t in (q, k, v, q_scale, k_scale, v_scale):
@@ -38,7 +39,8 @@ def attention_mxfp4_forward(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, q
     out = torch.empty((B, Hq, Sq, Dv), dtype=torch.bfloat16, device=q.device)
     lse = torch.empty((B, Hq, Sq), dtype=torch.float32, device=q.device)
     check(rt.lib().alto_mxfp4_attention_fwd(q.data_ptr(), q_scale.data_ptr(), k.data_ptr(), k_scale.data_ptr(), v.data_ptr(),
-                                            v_scale.data_ptr(), out.data_ptr(), lse.data_ptr(), B, Hq, Hk, Sq, Sk, D, Dv,
+                                            v_scale.data_ptr(), out.data_ptr(), lse.data_ptr(), B, Hq, Hk, Sq, Sk,
+                                            Sk if seqlen_k is None else int(seqlen_k), D, Dv,
                                             float(sm_scale), int(bool(causal)), rt.stream_ptr(q.device)), "alto_mxfp4_attention_fwd")
     return out, lse
 
@@ -84,8 +86,12 @@ def triton_attention_mxfp4(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, al
     assert max_seqlens_q in (None, q.shape[2]) and max_seqlens_k in (None, k.shape[2]), "variable lengths are not implemented"
     if sm_scale is None:
         sm_scale = q.shape[-1] ** -0.5
+    seqlen_k = k.shape[2]
+    if seqlen_k % 64 == 32:   # one 32-row block of zeros: quantises to zero codes, the kernel masks those keys out
+        k = torch.nn.functional.pad(k, (0, 0, 0, 32))
+        v = torch.nn.functional.pad(v, (0, 0, 0, 32))
     qq, qs, kq, ks, vq, vs = quantize_qkv(q, k, v)
-    out, lse = attention_mxfp4_forward(qq, kq, vq, qs, ks, vs, sm_scale=sm_scale, causal=causal)
+    out, lse = attention_mxfp4_forward(qq, kq, vq, qs, ks, vs, sm_scale=sm_scale, causal=causal, seqlen_k=seqlen_k)
     return out, lse, torch.empty([], device=q.device, dtype=torch.float32)
 
 

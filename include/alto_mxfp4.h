@@ -209,12 +209,13 @@ int alto_mxfp4_qdq(const void* x, int dtype, int64_t batch, int64_t M, int64_t C
  * quantisation of [Sk][Dv], codes handed over packed along the keys (the column codes of alto_mxfp4_quantize):
  * vt_codes [B][Hk][Dv][Sk/2], v_scales [B][Hk][Sk/32][Dv/32].  K and V scale pointers 4-byte aligned, code pointers
  * 16-byte aligned.  Hq % Hk == 0 (grouped-query heads), D in {64,128,192,256}, Dv in {64,128}, Sq % 32 == 0,
- * Sk % 64 == 0, causal needs Sq <= Sk.  All tensors dense.
+ * Sk % 64 == 0.  Only the first Sk_used keys exist (Sk_used % 32 == 0, Sk - Sk_used < 64: a sequence of 32 (mod 64) keys is
+ * padded with one block of zero rows before it is quantised); causal needs Sq <= Sk_used.  All tensors dense.
  */
 int alto_mxfp4_attention_fwd(const void* q_codes, const void* q_scales, const void* k_codes, const void* k_scales,
                              const void* vt_codes, const void* v_scales, void* out, float* lse, int64_t B, int64_t Hq,
-                             int64_t Hk, int64_t Sq, int64_t Sk, int64_t D, int64_t Dv, float sm_scale, int causal,
-                             void* stream);
+                             int64_t Hk, int64_t Sq, int64_t Sk, int64_t Sk_used, int64_t D, int64_t Dv, float sm_scale,
+                             int causal, void* stream);
 
 /*
  * Diagnostic, no counterpart in the reference: a register-only loop of FP4 scaled-MFMA instructions

@@ -48,6 +48,9 @@ CASES = [
     (1, 2, 1, 64, 192, 256, 128, False),
     (1, 2, 1, 32, 64, 64, 128, True),
     (1, 3, 3, 160, 320, 192, 64, True),
+    (1, 2, 1, 96, 96, 128, 128, True),        # 96 keys: the second block is half there
+    (2, 2, 2, 64, 224, 64, 64, False),
+    (1, 4, 2, 32, 32, 128, 64, True),
 ]
 
 
@@ -139,8 +142,8 @@ def test_rejected_arguments(m):
         m.triton_attention_mxfp4(q, k, v, bias=torch.zeros(1, device=DEV))
     with pytest.raises(AssertionError, match="Sq <= Sk"):
         m.triton_attention_mxfp4(q.repeat(1, 1, 2, 1), k, v, causal=True)
-    qb, kb, vb = (t.to(DEV) for t in _qkv(1, 2, 2, 64, 96, 64, 64, seed=1))
-    with pytest.raises(AssertionError, match="multiple of 64"):
+    qb, kb, vb = (t.to(DEV) for t in _qkv(1, 2, 2, 64, 80, 64, 64, seed=1))
+    with pytest.raises(Exception):      # 80 keys: not a multiple of the 32-row quantisation blocks
         m.triton_attention_mxfp4(qb, kb, vb, causal=False)
     q3, k3, v3 = (t.to(DEV) for t in _qkv(1, 2, 2, 64, 64, 96, 64, seed=1))
     with pytest.raises(AssertionError, match="head dim"):
