@@ -42,6 +42,13 @@ __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
   return (u + 0x7FFFu + ((u >> 16) & 1u)) >> 16;
 }
 
+// two floats -> packed bf16 (round to nearest even), one v_cvt_pk_bf16_f32
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  typedef float f2_t __attribute__((ext_vector_type(2)));
+  bf16x2_t p = __builtin_convertvector(f2_t{lo, hi}, bf16x2_t);
+  return __builtin_bit_cast(uint32_t, p);
+}
+
 // ----------------------------------------------------------------------------- device: E8M0 scale rule
 // Biased exponent of the block absmax after rounding it to one mantissa bit, minus 2, clamped below at 1.
 __device__ __forceinline__ uint32_t e8m0_from_bf16_bits(uint32_t absbits16) {

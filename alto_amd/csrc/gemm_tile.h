@@ -76,13 +76,6 @@ __device__ __forceinline__ TileArgs uniform_args(const TileArgs& t) {
   return o;
 }
 
-// two floats -> packed bf16 (round to nearest even), one v_cvt_pk_bf16_f32
-__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
-  typedef float f2_t __attribute__((ext_vector_type(2)));
-  bf16x2_t p = __builtin_convertvector(f2_t{lo, hi}, bf16x2_t);
-  return __builtin_bit_cast(uint32_t, p);
-}
-
 typedef v16f_t TileAcc[4][2];   // per wave: 4 (M) x 2 (N) MFMA tiles of 32x32
 
 __device__ __forceinline__ void gemm_tile_zero(TileAcc& acc) {

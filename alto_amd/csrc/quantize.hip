@@ -226,8 +226,26 @@ __global__ __launch_bounds__(256) void quant_kernel(const QuantParams p) {
           }
         }
       }
+      // z * (+-1) / float32(sqrt(32)), correctly rounded: quotient estimate, one FMA correction, both with the sign
+      // folded into the (wave-uniform) constants; the sign bit is taken from the estimate so that -0 stays -0.
 #pragma unroll
-      for (int k = 0; k < 32; ++k) z[k] = round_to_T<T>(div_sqrt32_signed(z[k], ((p.sign_mask >> k) & 1u) << 31));
+      for (int k = 0; k < 32; ++k) {
+        const uint32_t flip = ((p.sign_mask >> k) & 1u) << 31;   // scalar: the constants stay in scalar registers
+        const float ck = u2f(f2u(5.656854152679443f) ^ flip);
+        const float rck = u2f(f2u(0.17677669529663689f) ^ flip);
+        const float q = z[k] * rck;
+        float r = __builtin_fmaf(-q, ck, z[k]);
+        r = __builtin_fmaxf(r, -3.0e38f);   // z = +-inf gives r = NaN: drop it so that the quotient stays +-inf
+        z[k] = u2f((f2u(__builtin_fmaf(r, rck, q)) & 0x7FFFFFFFu) | (f2u(q) & 0x80000000u));
+      }
+      if constexpr (BF) {   // round to bf16 two at a time
+#pragma unroll
+        for (int k = 0; k < 32; k += 2) {
+          const uint32_t w = pack_bf16x2(z[k], z[k + 1]);
+          z[k] = u2f(w << 16);
+          z[k + 1] = u2f(w & 0xFFFF0000u);
+        }
+      }
     }
     uint32_t s;
     if (B2D) {
@@ -237,7 +255,7 @@ __global__ __launch_bounds__(256) void quant_kernel(const QuantParams p) {
     } else {
       float am = 0.0f;
 #pragma unroll
-      for (int k = 0; k < 32; ++k) am = __builtin_fmaxf(am, __builtin_fabsf(z[k]));
+      for (int k = 0; k < 32; k += 2) am = __builtin_fmaxf(__builtin_fmaxf(am, __builtin_fabsf(z[k])), __builtin_fabsf(z[k + 1]));
       if (GEN && p.uos) s = e8m0_uos(am);
       else s = BF ? e8m0_from_bf16_bits(f2u(am) >> 16) : e8m0_from_f32_bits(f2u(am));
       p.col_scales[(b * C + cc) * (M / 32) + blockIdx.y] = (uint8_t)s;
