@@ -54,6 +54,18 @@ def main():
     out["gemm_a_codes"], out["gemm_a_scales"] = aq.numpy(), as_.numpy()
     out["gemm_b_codes"], out["gemm_b_scales"] = bq.numpy(), bs.numpy()
     out["gemm_c_f32"] = O.gemm_ref(aq, as_, bq, bs, use_2dblock_b=True, trans_b=True).float().numpy()
+    # 5. flash-attention forward: 2 query heads on 1 KV head, 64 queries x 96 keys (the second key block is half there),
+    #    head dim 64, causal (bottom-right aligned); and the dynamic-clip scales of vector 1's input
+    from oracle.attention_oracle import attention_fwd_ref
+    gq = torch.Generator().manual_seed(21)
+    aq_ = torch.randn(1, 2, 64, 64, generator=gq).to(torch.bfloat16)
+    ak_ = torch.randn(1, 1, 96, 64, generator=gq).to(torch.bfloat16)
+    av_ = torch.randn(1, 1, 96, 64, generator=gq).to(torch.bfloat16)
+    ao, alse = attention_fwd_ref(aq_, ak_, av_, causal=True)
+    out["attn_q_bf16bits"], out["attn_k_bf16bits"], out["attn_v_bf16bits"] = bf16_bits(aq_), bf16_bits(ak_), bf16_bits(av_)
+    out["attn_out_bf16bits"], out["attn_lse_f32"] = bf16_bits(ao), alse.numpy()
+    qd, sd = O.quantize(x, clip_mode="dynamic")
+    out["dyn_codes"], out["dyn_scales"] = qd.numpy(), sd.numpy()
     path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "mxfp4_vectors.npz")
     np.savez_compressed(path, **out)
     print(path, os.path.getsize(path), "bytes;", ", ".join(f"{k}{list(v.shape)}" for k, v in out.items()))

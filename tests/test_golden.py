@@ -22,6 +22,16 @@ def bf16(name):
 
 
 # ----------------------------------------------------------------------------------------------- oracle (CPU)
+def test_oracle_attention_and_dynamic_clip_vectors():
+    from oracle.attention_oracle import attention_fwd_ref
+    o, lse = attention_fwd_ref(bf16("attn_q_bf16bits"), bf16("attn_k_bf16bits"), bf16("attn_v_bf16bits"), causal=True)
+    assert_bytes_equal(o.view(torch.int16), t("attn_out_bf16bits"), "attention output")
+    assert torch.equal(lse, t("attn_lse_f32"))
+    q, s = O.quantize(bf16("rne_x_bf16bits"), clip_mode="dynamic")
+    assert_bytes_equal(q, t("dyn_codes"), "dynamic-clip codes")
+    assert_bytes_equal(s, t("dyn_scales"), "dynamic-clip scales")
+
+
 def test_oracle_rne_vectors():
     q, s = O.quantize(bf16("rne_x_bf16bits"))
     assert_bytes_equal(q, t("rne_codes"), "codes")
@@ -90,3 +100,15 @@ def test_hip_gemm_vector(m):
     # products of E2M1 values are exact and these sums stay far below 2^24 ulps of their scale: fp32 accumulation in any
     # order differs from the float64 reference by rounding only (tolerance of the GEMM parity bar: 1e-2 relative Frobenius)
     assert O.rel_frobenius(c.cpu(), ref) < 1e-5
+
+
+@pytest.mark.gpu
+def test_hip_attention_and_dynamic_clip_vectors(m):
+    o, lse, _ = m.triton_attention_mxfp4(bf16("attn_q_bf16bits").cuda(), bf16("attn_k_bf16bits").cuda(), bf16("attn_v_bf16bits").cuda(), causal=True)
+    ref = bf16("attn_out_bf16bits").float()
+    # floating point through v_exp_f32: tolerance of the attention parity bar (2e-3 relative L2; equal bytes in practice)
+    assert float((o.cpu().float() - ref).norm() / ref.norm()) <= 2e-3
+    assert float((lse.cpu() - t("attn_lse_f32")).abs().max()) <= 1e-4
+    q, s = m.convert_to_mxfp4(bf16("rne_x_bf16bits").cuda(), clip_mode="dynamic")
+    assert_bytes_equal(q, t("dyn_codes"), "dynamic-clip codes")
+    assert_bytes_equal(s, t("dyn_scales"), "dynamic-clip scales")
