@@ -17,7 +17,7 @@ LIBDIR = os.path.join(HERE, "lib")
 OBJDIR = os.path.join(HERE, "lib", "obj")
 LIBNAME = "libalto_mxfp4.so"
 
-SOURCES = ["capi.hip", "quantize.hip", "dequantize.hip", "gemm.hip", "gemm_tiled.hip", "grouped_gemm.hip", "probe.hip", "qdq.hip", "attention.hip", "quantize_dynamic.hip"]
+SOURCES = ["capi.hip", "quantize.hip", "dequantize.hip", "gemm.hip", "gemm_tiled.hip", "grouped_gemm.hip", "probe.hip", "qdq.hip", "attention.hip", "quantize_dynamic.hip", "random.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",

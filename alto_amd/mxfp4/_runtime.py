@@ -41,8 +41,8 @@ def lib():
 
 
 # ---------------------------------------------------------------------------------------------- random bits
-# Stochastic rounding consumes 32 random bits per element.  By default they are drawn from torch's CUDA
-# generator; tests and reproducible runs install their own source.
+# Stochastic rounding consumes 32 random bits per element.  By default the library's Philox4x32-10 kernel fills them;
+# tests and runs that want their own bits install a source.
 _rand_source: Optional[Callable[[torch.Size, torch.device], torch.Tensor]] = None
 
 
@@ -53,12 +53,22 @@ def set_rand_bits_source(fn: Optional[Callable[[torch.Size, torch.device], torch
 
 
 def draw_rand_bits(shape, device, seed: Optional[int] = None, offset: Optional[int] = None) -> torch.Tensor:
+    """32 random bits per element for stochastic rounding (int32 tensor of ``shape`` on ``device``).
+
+    A source installed with ``set_rand_bits_source`` wins.  Otherwise the library's Philox4x32-10 kernel fills the
+    tensor (``alto_mxfp4_random_bits``: memory-bound, several times faster than ``torch.randint``): key = ``seed``,
+    counter start = ``offset``; without a seed, 63 bits are drawn from torch's CPU generator, so ``torch.manual_seed``
+    makes a run repeatable and no device synchronisation is involved.
+    """
     if _rand_source is not None:
         r = _rand_source(torch.Size(shape), device)
         assert r.shape == torch.Size(shape) and r.dtype in (torch.int32, torch.uint32)
         return r
-    gen = None
-    if seed is not None:
-        gen = torch.Generator(device=device)
-        gen.manual_seed(int(seed) * 0x9E3779B1 + (int(offset) if offset is not None else 0) & 0x7FFFFFFFFFFFFFFF)
-    return torch.randint(-2 ** 31, 2 ** 31, tuple(shape), dtype=torch.int32, device=device, generator=gen)
+    if seed is None:
+        seed = int(torch.randint(0, 2 ** 63 - 1, (1,), dtype=torch.int64).item())
+    out = torch.empty(tuple(shape), dtype=torch.int32, device=device)
+    if out.numel():
+        from .._lib import check
+        check(lib().alto_mxfp4_random_bits(out.data_ptr(), out.numel(), int(seed) & (2 ** 64 - 1), int(offset or 0) & (2 ** 64 - 1),
+                                           stream_ptr(out.device)), "alto_mxfp4_random_bits")
+    return out

@@ -127,8 +127,8 @@ def convert_to_mxfp4(
 
     ``use_asm`` is accepted for signature compatibility and ignored (there is one implementation).
     ``use_sr`` consumes ``rand_bits`` (int32/uint32, same shape as ``data_hp``; element ``[i, j]`` uses
-    ``rand_bits[i, j]``); when omitted the bits are drawn from torch's CUDA generator (seeded by
-    ``philox_seed``/``philox_offset`` if given).  ``hadamard`` fuses ``hadamard(x, left_mul=True)`` in front of
+    ``rand_bits[i, j]``); when omitted they come from the library's Philox4x32-10 fill kernel (key and
+    counter start ``philox_seed``/``philox_offset`` if given, else a draw from torch's CPU generator).  ``hadamard`` fuses ``hadamard(x, left_mul=True)`` in front of
     an ``axis=-2`` quantisation of a 2D tensor.
     """
     assert block_size == BLOCK_SIZE_DEFAULT, "only block_size=32 is implemented"

@@ -279,8 +279,8 @@ class AttentionFwd(Workload):
 
 class LinearStep(Workload):
     """Config 3 + 4 end to end: MXFP4LinearFunction forward and backward at the Llama-3-8B FFN shape (production flags:
-    1D activations, 2D weights, Hadamard on the wgrad operands, stochastic rounding of dY with supplied bits): three
-    quantizer passes over activations / gradients (plus the weight's unless cached) and three GEMMs per step."""
+    1D activations, 2D weights, Hadamard on the wgrad operands, stochastic rounding of dY): per step three quantizer
+    passes over activations / gradients (plus the weight's unless cached), one fill of random words for dY and three GEMMs."""
     bound = "mfma"
     kernel = "gemm"
     M, K, N = 8192, 4096, 14336
@@ -297,7 +297,6 @@ class LinearStep(Workload):
         self.x = torch.randn(self.M, self.K, device=dev, generator=gen).bfloat16().requires_grad_(True)
         self.w = (torch.randn(self.N, self.K, device=dev, generator=gen) * 0.02).bfloat16().requires_grad_(True)
         self.go = _laplace((self.M, self.N), 1e-3, dev, gen)
-        self.r = torch.randint(-2 ** 31, 2 ** 31 - 1, (self.M, self.N), device=dev, generator=gen, dtype=torch.int64).to(torch.int32)
         g = torch.Generator().manual_seed(1234)
         signs = (torch.randint(0, 2, (32,), generator=g) * 2 - 1).to(torch.int8)
         self.h = m.HadamardTransform(signs, torch.randperm(32, generator=g))
@@ -305,13 +304,11 @@ class LinearStep(Workload):
     def step(self):
         m = self.m
         m.enable_weight_cache(self.cached)
-        m.set_rand_bits_source(lambda shp, d: self.r)
-        try:
+        try:   # the random words of the stochastic rounding are drawn inside the step (Philox fill kernel), as in training
             self.x.grad = self.w.grad = None
             y = m.MXFP4LinearFunction.apply(self.x, self.w, False, True, True, False, "none", False, self.h, False)
             y.backward(self.go)
         finally:
-            m.set_rand_bits_source(None)
             if not self.cached:
                 m.enable_weight_cache(False)
         return y

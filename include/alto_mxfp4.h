@@ -218,6 +218,15 @@ int alto_mxfp4_attention_fwd(const void* q_codes, const void* q_scales, const vo
                              int causal, void* stream);
 
 /*
+ * Fills out[0 .. n) with random 32-bit words for stochastic rounding: word 4 c + j is word j of Philox4x32-10 (Salmon et
+ * al., SC'11) with the 128-bit counter c + offset and the 64-bit key `seed`.  The reference draws its bits inside its
+ * kernel from the same generator family (tl.randint4x, alto/kernels/fp4/fp4_common/triton_fp4_ops.py:15-18) with
+ * tile-local offsets; here they are a tensor so that the quantizer's result can be reproduced from its inputs.
+ * out 16-byte aligned.
+ */
+int alto_mxfp4_random_bits(uint32_t* out, int64_t n, uint64_t seed, uint64_t offset, void* stream);
+
+/*
  * Diagnostic, no counterpart in the reference: a register-only loop of FP4 scaled-MFMA instructions
  * (8 per iteration and wave, 8 waves per workgroup, `workgroups` workgroups; 2*32*32*64 FLOP each),
  * with constant (random_operands = 0) or pseudo-random FP4 operands.  bench.py times it to report

@@ -261,3 +261,37 @@ def test_padded_code_rows_hold_the_same_bytes(m):
     assert padded[0].stride(0) == 1536 and padded[2].transpose(0, 1).stride(0) == 128
     for d, p_ in zip(dense, padded):
         assert d.shape == p_.shape and torch.equal(d, p_)
+
+
+@pytest.mark.parametrize("n,seed,offset", [(4096, 1, 0), (1003, 0xDEADBEEFCAFEF00D, 12345), (7, 5, 2 ** 64 - 1), (4 * 3000 + 2, 9, 2 ** 64 - 1000)])
+def test_random_bits_kernel_is_philox4x32_10(m, n, seed, offset):
+    """alto_mxfp4_random_bits against the numpy Philox4x32-10 (pinned by the Random123 known answers), including a count
+    that is not a multiple of 4 and counters that carry into the high 64 bits."""
+    from alto_amd.mxfp4 import _runtime as rt
+    from alto_amd._lib import check
+    from oracle.philox import random_bits as philox_bits
+    out = torch.full((n + 8,), 0x55555555, dtype=torch.int32, device=DEV)   # 8 guard words behind the output
+    check(rt.lib().alto_mxfp4_random_bits(out.data_ptr(), n, seed, offset, rt.stream_ptr(out.device)), "random_bits")
+    got = out.cpu().numpy().view(np.uint32)
+    assert np.array_equal(got[:n], philox_bits(n, seed, offset))
+    assert np.all(got[n:] == 0x55555555)
+
+
+def test_default_random_bits_follow_the_torch_seed(m):
+    """Without supplied bits, stochastic rounding draws from the Philox kernel keyed by torch's CPU generator."""
+    x = laplace((64, 96), 1e-3, torch.bfloat16, seed=3).to(DEV)
+    torch.manual_seed(123)
+    a = m.convert_to_mxfp4(x, use_sr=True)
+    torch.manual_seed(123)
+    b = m.convert_to_mxfp4(x, use_sr=True)
+    c = m.convert_to_mxfp4(x, use_sr=True)
+    assert torch.equal(a[0], b[0]) and not torch.equal(a[0], c[0])
+    d = m.convert_to_mxfp4(x, use_sr=True, philox_seed=7, philox_offset=11)
+    from oracle.philox import random_bits as philox_bits
+    r = torch.from_numpy(philox_bits(64 * 96, 7, 11).view(np.int32).copy()).reshape(64, 96)
+    _check_pair(d, O.quantize(x.cpu(), use_sr=True, rand_bits=r), "philox_seed / philox_offset")
+    # the words look random: every bit position is set about half of the time
+    from alto_amd.mxfp4 import _runtime as rt
+    w = rt.draw_rand_bits((1 << 20,), torch.device(DEV), seed=1).cpu().numpy().view(np.uint32)
+    frac = np.array([((w >> b) & 1).mean() for b in range(32)])
+    assert np.all(np.abs(frac - 0.5) < 0.005)

@@ -392,3 +392,25 @@ def test_grouped_reference_and_offsets():
     wt = w.transpose(-1, -2).contiguous()
     wq2, ws2 = O.quantize(wt, axis=-2, is_2d_block=True)
     assert torch.equal(O.grouped_gemm_ref(aq, as_, wq2, ws2, idx, trans_weights=False), out)
+
+
+def test_philox4x32_10_known_answers():
+    """The three known-answer vectors of the Random123 library (kat_vectors, philox4x32 with 10 rounds): zeros, all ones,
+    digits of pi.  A wrong multiplier, Weyl constant, word order or round count fails all of them."""
+    import numpy as np
+    from oracle.philox import philox4x32_10, random_bits
+
+    def run(c, k):
+        return [int(v) for v in philox4x32_10(np.array(c, dtype=np.uint32), np.array(k, dtype=np.uint32))]
+    assert run([0, 0, 0, 0], [0, 0]) == [0x6627e8d5, 0xe169c58d, 0xbc57ac4c, 0x9b00dbd8]
+    assert run([0xffffffff] * 4, [0xffffffff] * 2) == [0x408f276d, 0x41c83b0e, 0xa20bc7c6, 0x6d5451fd]
+    assert run([0x243f6a88, 0x85a308d3, 0x13198a2e, 0x03707344], [0xa4093822, 0x299f31d0]) == [0xd16cfe09, 0x94fdcceb, 0x5001e420, 0x24126ea1]
+    # stream layout: word 4 c + j = word j of block (c + offset); a count that is not a multiple of 4 is a prefix
+    a = random_bits(10, seed=7, offset=0)
+    b = random_bits(6, seed=7, offset=1)
+    assert np.array_equal(a[4:10], b) and np.array_equal(random_bits(7, 7), a[:7])
+    assert [int(v) for v in random_bits(4, seed=0, offset=0)] == [0x6627e8d5, 0xe169c58d, 0xbc57ac4c, 0x9b00dbd8]
+    # the vectorised path (>= 1024 blocks) agrees with the block-by-block path, also across the 64-bit carry of the counter
+    big = random_bits(4 * 1500, seed=3, offset=2 ** 64 - 700)
+    assert np.array_equal(big[:4 * 600], random_bits(4 * 600, seed=3, offset=2 ** 64 - 700))
+    assert np.array_equal(big[4 * 700:4 * 704], random_bits(16, seed=3, offset=2 ** 64))
