@@ -197,3 +197,29 @@ def test_registered_torch_ops_run_the_hip_kernels(m):
     aqm, asm_ = m.convert_to_mxfp4(a, axis=0)
     dw = ns.mxfp4_grouped_gemm_backward_weights(gqm, aqm, idx, 2, gsm, asm_, True, False, False)
     assert torch.equal(dw, m.mxfp4_grouped_gemm_backward_weights(gqm, aqm, idx, 2, gsm, asm_, use_2dblock_x=False)) and dw.shape == (2, 192, 256)
+
+
+def test_forward_replays_from_a_hip_graph(m):
+    """Quantizer and GEMM launches allocate nothing and sync nothing, so a linear forward can be captured once and
+    replayed; every replay (with eager work and synchronisations between them) equals the eager result."""
+    x = randn_outliers((256, 512), torch.bfloat16, seed=61).to(DEV)
+    w = (randn_outliers((384, 512), torch.bfloat16, seed=62) * 0.02).to(DEV)
+    eager = m._to_mxfp4_then_scaled_mm(x, w, False, True, False, False, "none", False)
+    torch.cuda.synchronize()
+    static_x = x.clone()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):            # warm-up on the capture stream (one-time per-kernel set-up happens here)
+        m._to_mxfp4_then_scaled_mm(static_x, w, False, True, False, False, "none", False)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        static_y = m._to_mxfp4_then_scaled_mm(static_x, w, False, True, False, False, "none", False)
+    for i in range(3):
+        static_x.copy_(x if i != 1 else x * 2)
+        g.replay()
+        torch.cuda.synchronize()
+        ref = eager if i != 1 else m._to_mxfp4_then_scaled_mm(x * 2, w, False, True, False, False, "none", False)
+        assert torch.equal(static_y, ref), f"replay {i}"
+        (x.float() @ w.float().T).sum().item()   # unrelated eager work and a host sync between replays
