@@ -194,12 +194,15 @@ __global__ __launch_bounds__(256, ATTN_WG_PER_CU) void attn_fwd_kernel(AttnArgs 
             if ((a.causal && key > qrow + shift) || key >= a.Sk_used) S[t][v] = -__builtin_inff();
           }
       }
-      float mx = -__builtin_inff();
+      float tmx[2];   // row maximum of each 32-key tile (exp2 is monotonic: its largest probability comes from this score)
 #pragma unroll
-      for (int t = 0; t < 2; ++t)
+      for (int t = 0; t < 2; ++t) {
+        float x = -__builtin_inff();
 #pragma unroll
-        for (int v = 0; v < 16; ++v) mx = fmaxf(mx, S[t][v]);
-      mx = pair_max(mx);
+        for (int v = 0; v < 16; ++v) x = fmaxf(x, S[t][v]);
+        tmx[t] = pair_max(x);
+      }
+      const float mx = fmaxf(tmx[0], tmx[1]);
       const float m_new = fmaxf(m_i, mx * c2);
       const float alpha = __builtin_amdgcn_exp2f(m_i - m_new);
       m_i = m_new;
@@ -209,13 +212,9 @@ __global__ __launch_bounds__(256, ATTN_WG_PER_CU) void attn_fwd_kernel(AttnArgs 
       int psc[2];
 #pragma unroll
       for (int t = 0; t < 2; ++t) {
-        float am = 0.0f;
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-          S[t][v] = __builtin_amdgcn_exp2f(__builtin_fmaf(S[t][v], c2, -m_new));
-          am = fmaxf(am, S[t][v]);
-        }
-        am = pair_max(am);
+        for (int v = 0; v < 16; ++v) S[t][v] = __builtin_amdgcn_exp2f(__builtin_fmaf(S[t][v], c2, -m_new));
+        const float am = __builtin_amdgcn_exp2f(__builtin_fmaf(tmx[t], c2, -m_new));   // = max of the 32 values above
         const uint32_t e = e8m0_from_f32_bits(f2u(am));
         psc[t] = (int)e;
         const float scale_f = u2f(e << 23);
