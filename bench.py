@@ -193,6 +193,18 @@ class Gemm(Workload):
         return run, self.work * rows / self.M, f"{rows} of {self.M} rows of A against all of B, dequantize + fp32 matmul"
 
 
+class VendorGemm(Gemm):
+    """The same config-3 operands through ``torch._scaled_mm`` (PyTorch's MXFP4 path into hipBLASLt): a comparator, not part of
+    the product; reported beside the kernel's own number."""
+    kernel = "hipBLASLt via torch._scaled_mm"
+
+    def step(self):
+        import torch
+        a = self.aq.view(torch.float4_e2m1fn_x2)
+        b = self.bq.view(torch.float4_e2m1fn_x2)
+        return torch._scaled_mm(a, b.t(), self.as_.view(torch.float8_e8m0fnu), self.bs.view(torch.float8_e8m0fnu), out_dtype=torch.bfloat16)
+
+
 class GroupedGemm(Workload):
     """Config 5: 32 experts, hidden 2880 -> 5760, 65536 routed rows with Zipf(1.1) expert skew, ragged int32 offsets [33]."""
     name = "cfg5_grouped_gemm[65536x5760x2880,E=32]"
@@ -378,6 +390,8 @@ def load_traffic(key):
 def make_workloads():
     return {
         "cfg3_fprop": Gemm("cfg3_fprop_gemm[8192x14336x4096]", 8192, 14336, 4096, False, True, "act", "weight"),
+        "cfg3_fprop_vendor": VendorGemm("cfg3_fprop_gemm[8192x14336x4096] via torch._scaled_mm (1D scales on both operands)", 8192, 14336, 4096, False, False,
+                                        "act", "weight"),
         "cfg2_quant": FusedGradQuant(),
         "cfg1_quant": RneQuant(),
         # config 4: dgrad dX[8192,14336] = dY[8192,4096] . W^T-packed[14336,4096]; wgrad dW[4096,14336] over 8192 tokens
@@ -473,7 +487,13 @@ def main():
                 continue
             primary_mem_release = None  # noqa: F841
             try:
-                r = measure(w, dev, gen, max(5, args.steps // 2), max(2, args.warmup // 2))
+                try:
+                    r = measure(w, dev, gen, max(5, args.steps // 2), max(2, args.warmup // 2))
+                except (RuntimeError, AttributeError, NotImplementedError) as e:
+                    if key != "cfg3_fprop_vendor":
+                        raise
+                    others[key] = {"workload": w.name, "error": str(e)[:200]}
+                    continue
                 others[key] = {"workload": r["workload"], "ms": round(r["ms"], 4), "achieved": round(r["achieved"], 2), "unit": r["unit"],
                                "bound": r["bound"], "frac": round(r["frac"], 4)}
             finally:
