@@ -315,20 +315,24 @@ __device__ __forceinline__ void gemm_tile_mainloop(const TileArgs& ta, TileAcc& 
   // clocks per compute unit: a burst of eight loads per wave would hold the MFMAs behind it for a thousand clocks.)
   auto stage = [&](auto msc, int s, int kb) {
     constexpr int MS = decltype(msc)::value;
+    __builtin_amdgcn_s_setprio(2);
     ld.gload(smem, s + 1, MS ^ 1, 4, 8);
     mfma8(msc, std::integral_constant<int, 0>{}, fa0, fb0);
     read_frags(MS, 1, fa1, fb1);
     interleave_loads();
     __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_setprio(1);
     mfma8(msc, std::integral_constant<int, 1>{}, fa1, fb1);
     read_frags(MS, 2, fa0, fb0);
     interleave();
     __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_setprio(0);
     mfma8(msc, std::integral_constant<int, 2>{}, fa0, fb0);
     read_frags(MS, 3, fa1, fb1);
     interleave();
     __builtin_amdgcn_sched_barrier(0);
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    __builtin_amdgcn_s_setprio(3);
     if constexpr (MS == 0) {
       swrite(kb + 1);          // block kb+1 -> the other scale buffer (last read at the end of block kb-1)
       ld.template sload<KTAIL>(kb + 2, sreg);
