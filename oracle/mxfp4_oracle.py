@@ -32,6 +32,12 @@ closed forms, exhaustive enumeration against brute force, counting identities
 for stochastic rounding and a second, scalar pure-Python-int model in
 ``oracle/scalar_model.py``.
 
+Parity unpinned (no check available without running the reference's Triton kernels on gfx950):
+* ``clip_mode="dynamic"`` (``block_scales``): the ORDER of the fp32 sums of the block statistics and whether the final
+  multiply-add is contracted are Triton's choice in the reference; the order used here is this build's (the HIP kernel
+  follows it bit for bit).  Everything after ``max_abs`` is the pinned exponent rule.
+* the accumulation order inside ``tl.dot_scaled`` / ``v_mfma_scale`` (GEMMs are compared with a tolerance).
+
 Two deliberate departures from the reference (both are inputs the reference
 draws from hidden state and this build takes explicitly):
 
