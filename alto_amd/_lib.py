@@ -56,13 +56,21 @@ class AltoMxfp4Error(RuntimeError):
 
 
 def load():
-    """Load the in-tree shared library (building it first only when it does not exist)."""
+    """Load the in-tree shared library.  It is built first when it does not exist, and rebuilt when it was made from
+    other sources than the tree holds now (a digest of the sources is recorded beside it), so that an edited kernel is
+    never tested through a stale binary; ``ALTO_MXFP4_NO_REBUILD=1`` turns a stale library into an error instead."""
     global _lib
     with _lock:
         if _lib is not None:
             return _lib
         path = _build.lib_path()
         if not os.path.exists(path):
+            _build.build(verbose=False)
+        elif _build.is_stale():
+            if os.environ.get("ALTO_MXFP4_NO_REBUILD") == "1":
+                raise AltoMxfp4Error(f"{path} was not built from the sources in this tree: run `python -m alto_amd.build`")
+            import sys
+            print(f"alto_amd: {path} is older than its sources, rebuilding", file=sys.stderr, flush=True)
             _build.build(verbose=False)
         lib = ctypes.CDLL(path)
         for name, (res, args) in SIGNATURES.items():

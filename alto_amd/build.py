@@ -35,6 +35,32 @@ def lib_path() -> str:
     return os.path.join(LIBDIR, LIBNAME)
 
 
+def stamp_path() -> str:
+    return lib_path() + ".srchash"
+
+
+def source_hash() -> str:
+    """Digest of every file the library is built from (kernels, their headers, the C ABI header, the compiler flags)."""
+    import hashlib
+    h = hashlib.sha256(" ".join(HIPCC_FLAGS).encode())
+    files = sorted(os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith((".hip", ".h")))
+    files.append(os.path.join(HERE, "..", "include", "alto_mxfp4.h"))
+    for f in files:
+        h.update(os.path.basename(f).encode())
+        with open(f, "rb") as fh:
+            h.update(fh.read())
+    return h.hexdigest()
+
+
+def is_stale() -> bool:
+    """True when the built library does not come from the sources in the tree (or carries no record of its sources)."""
+    try:
+        with open(stamp_path()) as f:
+            return f.read().strip() != source_hash()
+    except OSError:
+        return True
+
+
 def _hipcc() -> str:
     exe = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
     if not os.path.exists(exe):
@@ -54,6 +80,7 @@ def _compile(src: str) -> str:
 def build(verbose: bool = True) -> str:
     """Compile every HIP source and link the shared library; always rebuilds."""
     os.makedirs(OBJDIR, exist_ok=True)
+    digest = source_hash()   # taken before compiling: an edit made during the build leaves the library marked stale
     with ThreadPoolExecutor(max_workers=min(8, len(SOURCES))) as pool:
         objs = list(pool.map(_compile, SOURCES))
     out = lib_path()
@@ -63,6 +90,8 @@ def build(verbose: bool = True) -> str:
     if res.returncode != 0:
         raise RuntimeError(f"link failed:\n{res.stdout}\n{res.stderr}")
     os.replace(tmp, out)
+    with open(stamp_path(), "w") as f:
+        f.write(digest + "\n")
     if verbose:
         print(f"built {out} ({os.path.getsize(out)} bytes)")
     return out

@@ -1,4 +1,6 @@
 // Tuned LDS-tiled MXFP4 GEMM for gfx950: dense entry (one 256x256 tile per 512-thread workgroup, XCD-aware tile order).
+#include <mutex>
+
 #include "gemm_tiled.h"
 #include "gemm_tile.h"
 
@@ -38,12 +40,13 @@ __global__ __launch_bounds__(GT_THREADS) void gemm_tiled_kernel(OperandView A, O
 
 template <typename OutT, bool KTAIL>
 int launch_tiled(const OperandView& A, const OperandView& B, int64_t M, int64_t N, int64_t K, void* c, int64_t ldc, float out_scale, hipStream_t st) {
-  static bool attr_set = false;  // the opt-in for > 64 KB of dynamic LDS is per function, set once per process
+  // the opt-in for > 64 KB of dynamic LDS is per function, set once per process (two host threads may make their first
+  // call together: forward on the caller's thread, backward on the autograd thread)
   auto kern = gemm_tiled_kernel<OutT, KTAIL>;
-  if (!attr_set) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, GT_LDS_BYTES) != hipSuccess) return -1;
-    attr_set = true;
-  }
+  static std::once_flag once;
+  static hipError_t attr_rc = hipSuccess;
+  std::call_once(once, [&] { attr_rc = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, GT_LDS_BYTES); });
+  if (attr_rc != hipSuccess) return -1;
   const int tiles_m = (int)((M + GT_TM - 1) / GT_TM), tiles_n = (int)((N + GT_TN - 1) / GT_TN);
   const int T = tiles_m * tiles_n;
   const int per_xcd = (T + 7) / 8;

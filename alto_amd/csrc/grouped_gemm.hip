@@ -1,4 +1,6 @@
 // Ragged grouped MXFP4 GEMMs for MoE experts (gfx950): forward / dX (rows grouped by expert) and dW (reduction grouped by expert).
+#include <mutex>
+
 #include "common.h"
 #include "gemm_simple.h"
 #include "gemm_tile.h"
@@ -31,6 +33,11 @@ __device__ __forceinline__ TileRef locate_tile(const int32_t* offs, int num_grou
     lo = hi;
   }
   return ref;
+}
+
+__device__ __forceinline__ int clamp_off(const int32_t* offs, int g, int64_t M_total) {
+  const int64_t v = offs[g];
+  return (int)(v < 0 ? 0 : (v > M_total ? M_total : v));
 }
 
 template <typename OutT>
@@ -73,20 +80,28 @@ __global__ __launch_bounds__(256) void grouped_dw_simple_kernel(OperandView GO, 
   v16f_t acc;
 #pragma unroll
   for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
-  const int gmax = (int)(M_total / 32);
+  int bad = 0;   // a boundary of this expert's token ranges that is not a multiple of 32: the MX blocks along the token dim
+                 // would be shared with another expert, so the gradient is poisoned with NaN instead of being silently wrong
   if (group_expert == nullptr) {
-    int g0 = offs[e] / 32, g1 = offs[e + 1] / 32;
-    g0 = g0 < 0 ? 0 : g0;
-    g1 = g1 > gmax ? gmax : g1;
+    const int lo = clamp_off(offs, e, M_total), hi = clamp_off(offs, e + 1, M_total);
+    if (hi > lo) bad = (lo | hi) & 31;
+    int g0 = lo / 32, g1 = hi / 32;
     mma_tile_32x32_acc(acc, GO, X, n0, k0, 0, N, K, g0, g1);
   } else {
     for (int g = 0; g < num_groups; ++g) {
       if (group_expert[g] != e) continue;
-      int g0 = offs[g] / 32, g1 = offs[g + 1] / 32;
-      g0 = g0 < 0 ? 0 : g0;
-      g1 = g1 > gmax ? gmax : g1;
+      const int lo = clamp_off(offs, g, M_total), hi = clamp_off(offs, g + 1, M_total);
+      if (hi > lo) {   // a boundary shared with a neighbouring group of the same expert splits nothing
+        if (!(g > 0 && group_expert[g - 1] == e)) bad |= lo & 31;
+        if (!(g + 1 < num_groups && group_expert[g + 1] == e)) bad |= hi & 31;
+      }
+      int g0 = lo / 32, g1 = hi / 32;
       mma_tile_32x32_acc(acc, GO, X, n0, k0, 0, N, K, g0, g1);
     }
+  }
+  if (bad) {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[i] = __builtin_nanf("");
   }
   const int lane = threadIdx.x & 63;
   const int64_t j = k0 + (lane & 31);
@@ -107,10 +122,6 @@ __global__ __launch_bounds__(256) void grouped_dw_simple_kernel(OperandView GO, 
 }
 
 // ----------------------------------------------------------------------------- 256x256 tiles (large problems)
-__device__ __forceinline__ int clamp_off(const int32_t* offs, int g, int64_t M_total) {
-  const int64_t v = offs[g];
-  return (int)(v < 0 ? 0 : (v > M_total ? M_total : v));
-}
 
 // Tile order of the grouped kernels.  As in the dense kernel an XCD (wg % 8) works on 8 neighbouring N-tiles of a few row
 // bands at a time, so its L2 shares the A rows and the expert's weight rows; but the row bands are dealt to the XCDs
@@ -234,7 +245,10 @@ __global__ __launch_bounds__(GT_THREADS) void grouped_dw_tiled_kernel(OperandVie
   gemm_tile_zero(acc);
   const int64_t p_bytes = (NP - 1) * P.ld + M_total / 2, q_bytes = (NQ - 1) * Q.ld + M_total / 2;
   const int64_t ps_bytes = (NP - 1) * P.ss_r + M_total / 32, qs_bytes = (NQ - 1) * Q.ss_r + M_total / 32;
-  auto tok = [&](int g) { return (int64_t)(clamp_off(offs, g, M_total) & ~31); };
+  // Boundaries of this expert's token runs; one that is not a multiple of 32 would share an MX block along the token dim
+  // with another expert: the tile is then poisoned with NaN instead of being silently wrong.
+  int bad = 0;
+  auto tok = [&](int g) { return (int64_t)clamp_off(offs, g, M_total); };
   uint64_t* mstart = reinterpret_cast<uint64_t*>(smem + GT_LDS_BYTES);
   uint64_t* mend = mstart + GT_DW_MAX_GROUPS / 64;
   const int words = group_expert ? (num_groups + 63) >> 6 : 0;
@@ -293,12 +307,24 @@ __global__ __launch_bounds__(GT_THREADS) void grouped_dw_tiled_kernel(OperandVie
     }
     if (!have) break;
     if (t1 <= t0) continue;
+    bad |= (int)(t0 | t1) & 31;
+    t0 &= ~(int64_t)31;
+    t1 &= ~(int64_t)31;
+    if (t1 <= t0) continue;
     OperandView Pv = P, Qv = Q;   // codes start at the run; the scale rows keep their base and the run's offset rides in s_k0
     Pv.codes += t0 / 2;
     Qv.codes += t0 / 2;
     TileArgs ta{Pv, Qv, (int64_t)tm * GT_TM, (int64_t)tn * GT_TN, 0, NP, NQ, (int)((t1 - t0) / 32), out_scale,
                 p_bytes - t0 / 2, q_bytes - t0 / 2, ps_bytes, qs_bytes, (int)(t0 / 32), (int)(M_total / 32)};
     gemm_tile_mainloop<true>(ta, acc, smem);
+  }
+  if (bad) {
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int u = 0; u < 2; ++u)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[t][u][v] = __builtin_nanf("");
   }
   TileArgs ta{P, Q, (int64_t)tm * GT_TM, (int64_t)tn * GT_TN, 0, NP, NQ, 0, out_scale, 0, 0, 0, 0, 0, 0};
   gemm_tile_store<OutT>(ta, acc, dw + e * s_e, ld, smem);
@@ -308,12 +334,13 @@ template <typename OutT, bool KTAIL>
 int launch_grouped_tiled(const OperandView& A, const uint8_t* w, int64_t w_stride_e, int64_t ldw, const uint8_t* w_scales, int64_t ws_stride_e,
                          int64_t ws_r, int w_is_2d, const int32_t* offs, const int32_t* group_expert, int num_groups, int num_experts,
                          int64_t M_total, int64_t N, int64_t K, void* out, int64_t ldo, hipStream_t st) {
-  static bool attr_set = false;  // the opt-in for > 64 KB of dynamic LDS is per function, set once per process
+  // the opt-in for > 64 KB of dynamic LDS is per function, set once per process (thread-safe: forward and backward may
+  // make their first calls from two host threads)
   auto kern = grouped_tiled_kernel<OutT, KTAIL>;
-  if (!attr_set) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, GT_LDS_BYTES) != hipSuccess) return -1;
-    attr_set = true;
-  }
+  static std::once_flag once;
+  static hipError_t attr_rc = hipSuccess;
+  std::call_once(once, [&] { attr_rc = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, GT_LDS_BYTES); });
+  if (attr_rc != hipSuccess) return -1;
   const int tiles_m = (int)((M_total + GT_TM - 1) / GT_TM), tiles_n = (int)((N + GT_TN - 1) / GT_TN);
   hipLaunchKernelGGL(kern, dim3((unsigned)grouped_grid_size(tiles_m, tiles_n)), dim3(GT_THREADS), GT_LDS_BYTES, st, A, w, w_stride_e, ldw, w_scales, ws_stride_e, ws_r,
                      w_is_2d, offs, group_expert, num_groups, num_experts, M_total, N, (int)(K / 32), (OutT*)out, ldo, tiles_m, tiles_n);
@@ -323,12 +350,11 @@ int launch_grouped_tiled(const OperandView& A, const uint8_t* w, int64_t w_strid
 template <typename OutT>
 int launch_dw_tiled(const OperandView& P, const OperandView& Q, int64_t NP, int64_t NQ, const int32_t* offs, const int32_t* group_expert,
                     int num_groups, int num_experts, int64_t M_total, void* dw, int64_t s_e, int64_t ld, float out_scale, hipStream_t st) {
-  static bool attr_set = false;
   auto kern = grouped_dw_tiled_kernel<OutT>;
-  if (!attr_set) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, GT_DW_LDS_BYTES) != hipSuccess) return -1;
-    attr_set = true;
-  }
+  static std::once_flag once;
+  static hipError_t attr_rc = hipSuccess;
+  std::call_once(once, [&] { attr_rc = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, GT_DW_LDS_BYTES); });
+  if (attr_rc != hipSuccess) return -1;
   const int tiles_p = (int)((NP + GT_TM - 1) / GT_TM), tiles_q = (int)((NQ + GT_TN - 1) / GT_TN);
   hipLaunchKernelGGL(kern, dim3((unsigned)grouped_grid_size(tiles_p, tiles_q), (unsigned)num_experts), dim3(GT_THREADS), GT_DW_LDS_BYTES, st, P, Q, NP, NQ, offs,
                      group_expert, num_groups, M_total, (OutT*)dw, s_e, ld, out_scale, tiles_p, tiles_q);

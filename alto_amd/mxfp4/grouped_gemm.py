@@ -182,9 +182,9 @@ class MXFP4GroupedGEMM(torch.autograd.Function):
         # weights: one pass gives the K-packed codes (forward) and the N-packed codes (dX)
         w = expert_weights if trans_weights else expert_weights.transpose(1, 2)   # logical [E, N, K]
         if w.stride(2) == 1:
-            wq_nk, ws_nk, wq_kn, ws_kn = _quantize_experts(w, use_uos)            # [E,N,K/2], [E,N/32,K/32], [E,K,N/2], [E,K/32,N/32]
+            wq_nk, ws_nk, wq_kn, ws_kn = _quantize_experts(expert_weights, w, use_uos)   # [E,N,K/2], [E,N/32,K/32], [E,K,N/2], [E,K/32,N/32]
         else:                                                                     # stored [E, K, N]: same pass, roles swapped
-            wq_kn, ws_kn, wq_nk, ws_nk = _quantize_experts(w.transpose(1, 2), use_uos)
+            wq_kn, ws_kn, wq_nk, ws_nk = _quantize_experts(expert_weights, w.transpose(1, 2), use_uos)
         out = grouped_forward(a_q, a_s, wq_nk, ws_nk, groups, False, True, original_dtype)
         ctx.save_for_backward(a_qm, a_sm, wq_kn, ws_kn, groups.offs, groups.expert)
         ctx.num_groups = groups.n
@@ -214,11 +214,12 @@ class MXFP4GroupedGEMM(torch.autograd.Function):
         return (grad_inputs, grad_weights) + (None,) * 11
 
 
-def _quantize_experts(w: torch.Tensor, use_uos: bool):
-    """w [E, R, C] (unit stride along C) -> codes packed along C [E,R,C/2], 2D scales [E,R/32,C/32], codes packed along R
-    [E,C,R/2] and the same scales stored transposed [E,C/32,R/32] (each operand of a GEMM wants unit stride along its K)."""
+def _quantize_experts(owner: torch.Tensor, w: torch.Tensor, use_uos: bool):
+    """w [E, R, C] (unit stride along C; ``owner`` or a transposed view of it) -> codes packed along C [E,R,C/2], 2D scales
+    [E,R/32,C/32], codes packed along R [E,C,R/2] and the same scales stored transposed [E,C/32,R/32] (each operand of a
+    GEMM wants unit stride along its K).  The cache entry belongs to ``owner``, the tensor object the caller keeps."""
     from .quantization import _prep, _quantize_call
-    return cached_weight_quantisation(w, ("experts2d", bool(use_uos)),
+    return cached_weight_quantisation(owner, ("experts2d", bool(use_uos), tuple(w.shape), tuple(w.stride())),
                                       lambda: _quantize_call(_prep(w), True, True, True, False, None, None, 0, use_uos, True))
 
 

@@ -5,6 +5,7 @@ Mirrors ``alto/kernels/fp4/mxfp4/mxfp_linear.py``: ``blockwise_mxfp4_gemm`` (:14
 """
 from __future__ import annotations
 
+import weakref
 from typing import Optional
 
 import torch
@@ -28,8 +29,12 @@ def unwrap_weight_wrapper(weight: torch.Tensor) -> torch.Tensor:
 # ----------------------------------------------------------------------------------------------- quantized-weight cache
 # The reference re-quantizes the weight in every forward (mxfp_linear.py:317-322).  Between two optimizer steps the
 # weight does not change (gradient accumulation, activation recomputation), so the four tensors of its 2D-block
-# quantisation can be kept.  An entry is valid while the weight's storage, shape and autograd version counter are the
-# ones it was made from: any in-place update (optimizer step, copy_) bumps the counter and the entry is rebuilt.
+# quantisation can be kept.  An entry belongs to one tensor OBJECT (held through a weak reference, so a new tensor that
+# the allocator places at a freed weight's address never matches) and is valid while that object's storage address,
+# shape, strides, dtype and autograd version counter are the ones it was made from: any in-place update (optimizer
+# step, copy_) bumps the counter and the entry is rebuilt.  The entry dies with the weight.  Writes that bypass the
+# version counter (``weight.data.copy_(...)``, some sharded-optimizer paths) are invisible to it: call
+# ``clear_weight_cache()`` after them.
 _WEIGHT_CACHE_ENABLED = False
 _WEIGHT_CACHE: dict = {}
 _WEIGHT_CACHE_STATS = {"hits": 0, "misses": 0}
@@ -53,18 +58,20 @@ def weight_cache_stats() -> dict:
 
 
 def cached_weight_quantisation(weight: torch.Tensor, tag, make):
-    """``make()`` or, with the cache enabled and the weight unchanged since, the tensors it returned last time."""
+    """``make()`` or, with the cache enabled and the tensor object ``weight`` unchanged since, what it returned last time."""
     if not _WEIGHT_CACHE_ENABLED:
         return make()
-    key = (weight.data_ptr(), weight.device.index, tag)
-    stamp = (weight._version, tuple(weight.shape), tuple(weight.stride()), weight.dtype)
+    key = (id(weight), tag)
+    stamp = (weight._version, weight.data_ptr(), tuple(weight.shape), tuple(weight.stride()), weight.dtype, weight.device)
     hit = _WEIGHT_CACHE.get(key)
-    if hit is not None and hit[0] == stamp:
+    if hit is not None and hit[0]() is weight and hit[1] == stamp:
         _WEIGHT_CACHE_STATS["hits"] += 1
-        return hit[1]
+        return hit[2]
     _WEIGHT_CACHE_STATS["misses"] += 1
     out = make()
-    _WEIGHT_CACHE[key] = (stamp, out)
+    if hit is None or hit[0]() is not weight:   # first entry of this object: drop it when the object goes away
+        weakref.finalize(weight, _WEIGHT_CACHE.pop, key, None)
+    _WEIGHT_CACHE[key] = (weakref.ref(weight), stamp, out)
     return out
 
 

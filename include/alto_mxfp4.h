@@ -174,8 +174,10 @@ int alto_mxfp4_grouped_gemm(const uint8_t* a, int64_t lda, const uint8_t* a_scal
  * operands packed along the token dim:  go [N][M_total/2], x [K][M_total/2] with
  * scales [N][M_total/32], [K][M_total/32] (1D along tokens; strides given).
  * Replaces _kernel_mxfp4_grouped_gemm_backward_dw (cg_backward.py:213-395); with group_expert == NULL the
- * expert's row range comes from offs directly instead of a scan over all groups.  Every offs[g] must be a
- * multiple of 32 (the reference requires 128, cg_backward.py:443-447).
+ * expert's row range comes from offs directly instead of a scan over all groups.  Every boundary between the
+ * token ranges of two experts must be a multiple of 32 (the reference requires 128, cg_backward.py:443-447): an MX
+ * block along the token dim cannot be split between experts.  The kernel checks this on the device (no host sync):
+ * dW[e] of an expert with a misaligned boundary is written with NaN, never with a silently wrong gradient.
  * dW of experts with no tokens is written with zeros.  Element (e, n, k) lands at
  * dw[e * dw_stride_e + n * dw_stride_n + k * dw_stride_k].
  */

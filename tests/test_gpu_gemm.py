@@ -320,3 +320,35 @@ def test_grouped_many_groups_sorted_runs(m):
     dw_ref = O.grouped_gemm_dw_ref(gqm, gsm, aqm, asm, idx, E, trans_weights=True)
     assert O.rel_frobenius(wg.grad.cpu(), dw_ref) < 4e-3
     assert bool((wg.grad[3] == 0).all())
+
+
+@pytest.mark.parametrize("tiled", [False, True])
+def test_grouped_dw_misaligned_boundaries_are_poisoned(m, tiled):
+    """The weight gradient reduces whole MX blocks of 32 tokens per expert.  Offsets that split a block between two
+    experts cannot give the right gradient: the kernels then write NaN into the gradients of the experts involved (a loud
+    failure, decided on the device without a host sync) and still give the oracle's result for the others; an expert
+    without tokens gets zeros wherever its (empty) range lies."""
+    from alto_amd.mxfp4 import grouped_gemm as G
+    N, K = (256, 256) if tiled else (64, 96)
+    scale = 4 if tiled else 1
+    offs = torch.tensor([0, 37, 37, 160, 224, 256], dtype=torch.int32) * scale      # tiled: 148 is not a multiple of 32 either
+    M_total, E = 256 * scale, 5
+    go = randn_outliers((M_total, N), torch.bfloat16, seed=90) / 100
+    a = randn_outliers((M_total, K), torch.bfloat16, seed=91)
+    gqm, gsm = O.quantize(go, axis=0)
+    aqm, asm = O.quantize(a, axis=0)
+    dw = G.grouped_dw(gqm.to(DEV).transpose(0, 1), gsm.to(DEV).transpose(0, 1), aqm.to(DEV).transpose(0, 1), asm.to(DEV).transpose(0, 1),
+                      G.groups_from_offsets(offs.to(DEV)), E, torch.float32)
+    assert bool(torch.isnan(dw[0]).all()) and bool(torch.isnan(dw[2]).all()), "experts that share a block must be poisoned"
+    assert bool((dw[1] == 0).all()), "an empty expert gets zeros"
+    idx = O.indices_from_offsets(offs[1:])
+    ref = O.grouped_gemm_dw_ref(gqm, gsm, aqm, asm, idx, E)
+    for e in (3, 4):
+        assert O.rel_frobenius(dw[e].cpu(), ref[e]) < 1e-5
+    # per-group expert ids: the boundary between two adjacent groups of ONE expert may lie anywhere
+    offs2 = torch.tensor([0, 37, 128, 256], dtype=torch.int32) * scale
+    groups = G.Groups(offs2.to(DEV), torch.tensor([1, 1, 0], dtype=torch.int32, device=DEV), 3)
+    dw2 = G.grouped_dw(gqm.to(DEV).transpose(0, 1), gsm.to(DEV).transpose(0, 1), aqm.to(DEV).transpose(0, 1), asm.to(DEV).transpose(0, 1),
+                       groups, 2, torch.float32)
+    idx2 = torch.cat([torch.ones(128 * scale, dtype=torch.int32), torch.zeros(128 * scale, dtype=torch.int32)])
+    assert O.rel_frobenius(dw2.cpu(), O.grouped_gemm_dw_ref(gqm, gsm, aqm, asm, idx2, 2)) < 1e-5

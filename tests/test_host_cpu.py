@@ -181,3 +181,34 @@ def test_torch_ops_registration_and_fake_shapes():
         gom, gom_s = torch.empty(128, 160, dtype=torch.uint8), torch.empty(8, 160, dtype=torch.uint8)
         xm, xm_s = torch.empty(128, 128, dtype=torch.uint8), torch.empty(8, 128, dtype=torch.uint8)
         assert ns.mxfp4_grouped_gemm_backward_weights(gom, xm, idx, 4, gom_s, xm_s, True, False, False).shape == (4, 160, 128)
+
+
+def test_weight_cache_is_keyed_by_object_identity():
+    """A cache entry belongs to one tensor object: a new tensor of the same shape at the same address (what the caching
+    allocator hands out after a weight is freed) must miss, an in-place update must miss, and entries die with the weight."""
+    import gc
+    from alto_amd.mxfp4 import linear as L
+    calls = []
+
+    def make():
+        calls.append(1)
+        return ("q", len(calls))
+
+    L.enable_weight_cache(True)
+    try:
+        storage = torch.zeros(64, 32)
+        w1 = storage.view(64, 32)
+        a = L.cached_weight_quantisation(w1, "t", make)
+        assert L.cached_weight_quantisation(w1, "t", make) is a and len(calls) == 1
+        w2 = storage.view(64, 32)                      # another object, same address, shape, strides, version
+        assert w2.data_ptr() == w1.data_ptr() and w2._version == w1._version
+        b = L.cached_weight_quantisation(w2, "t", make)
+        assert b is not a and len(calls) == 2
+        w1.add_(1.0)                                   # in-place update bumps the version counter
+        assert L.cached_weight_quantisation(w1, "t", make) is not a and len(calls) == 3
+        assert L.weight_cache_stats()["entries"] == 2
+        del w1, w2
+        gc.collect()
+        assert L.weight_cache_stats()["entries"] == 0, "entries must die with their weight"
+    finally:
+        L.enable_weight_cache(False)
