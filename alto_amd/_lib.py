@@ -30,6 +30,11 @@ SIGNATURES = {
                                             c_vp, c_vp, c_vp, c_vp, c_i64, c_i64,
                                             c_int, c_int, c_vp, c_i64, c_i64,
                                             c_int, c_vp, c_vp, c_int, c_int, c_vp]),
+    "alto_mxfp4_quantize_sr_philox": (c_int, [c_vp, c_int, c_i64, c_i64, c_i64, c_i64, c_i64,
+                                              c_vp, c_vp, c_vp, c_vp, c_i64, c_i64, c_int,
+                                              ctypes.c_uint64, ctypes.c_uint64, c_vp,
+                                              c_int, c_vp, c_vp, c_int, c_int, c_vp]),
+    "alto_mxfp4_philox_advance": (c_int, [c_vp, ctypes.c_uint64, c_vp]),
     "alto_mxfp4_hadamard": (c_int, [c_vp, c_int, c_i64, c_i64, c_i64, c_vp, c_i64, c_vp, c_vp, c_vp]),
     "alto_mxfp4_dequantize": (c_int, [c_vp, c_vp, c_i64, c_i64, c_int, c_vp, c_int, c_i64, c_i64, c_int, c_vp]),
     "alto_mxfp4_transpose_codes": (c_int, [c_vp, c_i64, c_i64, c_vp, c_vp]),
@@ -63,6 +68,15 @@ def load():
     with _lock:
         if _lib is not None:
             return _lib
+        path = os.environ.get("ALTO_MXFP4_LIB")   # an explicit library (a build with other options) is loaded as it is
+        if path:
+            lib = ctypes.CDLL(path)
+            for name, (res, args) in SIGNATURES.items():
+                fn = getattr(lib, name)
+                fn.restype = res
+                fn.argtypes = args
+            _lib = lib
+            return lib
         path = _build.lib_path()
         if not os.path.exists(path):
             _build.build(verbose=False)

@@ -69,19 +69,40 @@ __device__ __forceinline__ uint32_t e8m0_uos(float absmax) {
 }
 
 // ----------------------------------------------------------------------------- device: E2M1 encode
-// Stochastic rounding of a non-negative magnitude m (already divided by the scale) with 32 random bits.
-// Returns the 3-bit code (0..7).
-__device__ __forceinline__ uint32_t e2m1_sr_mag(float m, uint32_t r) {
-  uint32_t mb = f2u(m);
-  // normal lane: add the low 22 random bits under the kept mantissa bit, truncate, saturate at 7
-  uint32_t n = mb - 0x3F000000u + (r & 0x3FFFFFu);
-  n = (n < 0x01FFFFFFu ? n : 0x01FFFFFFu) >> 22;
-  // subnormal lane: threshold compare with 32-bit resolution; g = 2m in [0, 2)
-  float g = m + m;
-  float fr = __builtin_amdgcn_fractf(g);
-  uint32_t thr = (uint32_t)__builtin_ldexpf(fr, 32);
-  uint32_t den = (g >= 1.0f ? 1u : 0u) + (r <= thr ? 1u : 0u);
-  return m < 1.0f ? den : n;
+// Stochastic rounding of q (already divided by the scale, any sign) with 32 random bits; returns the 3-bit magnitude
+// code (0..7).  The rule of the reference (triton_fp4_ops.py:49-61,79-80):
+//   |q| >= 1: add the low 22 random bits under the kept mantissa bit and truncate, saturating at code 7 (the clamp of |q|
+//             to 6 does the saturation: 6.0 has no bits under the kept one);
+//   |q| <  1: g = 2|q| in [0, 2): code = floor(g) + (r <= trunc(frac(g) * 2^32)), an unsigned 32-bit compare.
+__device__ __forceinline__ uint32_t e2m1_sr_mag(float q, uint32_t r) {
+  const float m6 = __builtin_fminf(__builtin_fabsf(q), 6.0f);
+  const uint32_t n = (f2u(m6) - 0x3F000000u + (r & 0x3FFFFFu)) >> 22;
+  const float g = m6 + m6;
+  const uint32_t thr = (uint32_t)__builtin_ldexpf(__builtin_amdgcn_fractf(g), 32);
+  const uint32_t den = (uint32_t)g + (r <= thr ? 1u : 0u);
+  return m6 < 1.0f ? den : n;
+}
+
+// ----------------------------------------------------------------------------- device: Philox4x32-10
+// Salmon, Moraes, Dror, Shaw: "Parallel random numbers: as easy as 1, 2, 3" (SC'11): counter-based, so any word of the
+// stream can be regenerated from (key, counter).
+__device__ __forceinline__ void philox_round(uint32_t (&c)[4], uint32_t k0, uint32_t k1) {
+  const uint64_t p0 = (uint64_t)0xD2511F53u * c[0], p1 = (uint64_t)0xCD9E8D57u * c[2];   // 32 x 32 -> 64 bits each
+  const uint32_t lo0 = (uint32_t)p0, hi0 = (uint32_t)(p0 >> 32), lo1 = (uint32_t)p1, hi1 = (uint32_t)(p1 >> 32);
+  const uint32_t n0 = hi1 ^ c[1] ^ k0, n2 = hi0 ^ c[3] ^ k1;
+  c[0] = n0; c[1] = lo1; c[2] = n2; c[3] = lo0;
+}
+
+__device__ __forceinline__ uint4 philox4x32_10(uint64_t ctr_lo, uint64_t ctr_hi, uint64_t key) {
+  uint32_t c[4] = {(uint32_t)ctr_lo, (uint32_t)(ctr_lo >> 32), (uint32_t)ctr_hi, (uint32_t)(ctr_hi >> 32)};
+  uint32_t k0 = (uint32_t)key, k1 = (uint32_t)(key >> 32);
+#pragma unroll
+  for (int r = 0; r < 10; ++r) {
+    philox_round(c, k0, k1);
+    k0 += 0x9E3779B9u;
+    k1 += 0xBB67AE85u;
+  }
+  return make_uint4(c[0], c[1], c[2], c[3]);
 }
 
 // Round-to-nearest-even of a non-negative magnitude; software form (used where the packed HW convert does not fit).

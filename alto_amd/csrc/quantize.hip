@@ -25,20 +25,26 @@ struct QuantParams {
   int M, C;
   const uint32_t* rand;
   int64_t ld_r, bs_r;
+  uint64_t seed, ctr0;            // in-kernel Philox: key and first counter (used when philox_state is NULL)
+  const uint64_t* philox_state;   // device memory {key, first counter}, or NULL
   uint8_t* row_codes;
   uint8_t* row_scales;
   uint8_t* col_codes;
   uint8_t* col_scales;
   int64_t ld_rc, ld_cc;  // row pitch in bytes of the row / column code outputs (>= C/2, M/2)
   uint32_t sign_mask;    // bit k set: Q[k] == -1 (k = position after the permutation)
-  uint8_t perm[32];      // row j of a block -> position perm[j]
-  uint8_t perm_inv[32];  // position k -> row
+  uint32_t perm4[8];     // row j of a block -> position perm[j], four bytes per word
+  uint32_t pinv4[8];     // position k -> row
   int clip_row;          // 1: multiply by 3/4 (in the input dtype) before encoding the row output
   int clip_col;
   int uos;
 };
 
+// byte k of a packed table that lives in scalar registers (k is a compile-time constant where this is used)
+__device__ __forceinline__ int packed_byte(const uint32_t (&t)[8], int k) { return (int)((t[k >> 2] >> (8 * (k & 3))) & 0xFFu); }
+
 typedef unsigned short us2_t __attribute__((ext_vector_type(2)));
+typedef unsigned int v4u_t __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ uint32_t pk_max_u16(uint32_t a, uint32_t b) {
   us2_t r = __builtin_elementwise_max(__builtin_bit_cast(us2_t, a), __builtin_bit_cast(us2_t, b));
@@ -72,13 +78,22 @@ __device__ __forceinline__ float round_to_T(float v) {
   return v;
 }
 
-template <typename T, bool DO_ROW, bool DO_COL, bool SR, bool RHT, bool B2D, bool GEN>
+// SR: 0 = round to nearest even, 1 = stochastic with supplied random words, 2 = stochastic with Philox words made here.
+// Memory is addressed through buffer descriptors that start at the tile (32-bit per-lane offsets, row steps as scalar
+// offsets; an offset with bit 31 set is out of range: such a load returns zeros and such a store is dropped, which is
+// how rows past M and columns past C are masked).
+template <typename T, bool DO_ROW, bool DO_COL, int SR, bool RHT, bool B2D, bool GEN>
 __global__ __launch_bounds__(256) void quant_kernel(const QuantParams p) {
   constexpr bool BF = sizeof(T) == 2;
+  // The random words of the tile stay in LDS between the phases whenever the row phase holds them anyway: the column
+  // phase then reads nothing from memory.  (Column output alone with supplied words: one read either way, no staging.)
+  constexpr bool STASH = DO_COL && (SR == 2 || (SR == 1 && DO_ROW));
+  constexpr int OOB = (int)0x80000000;
   __shared__ __align__(16) T tile[DO_COL ? 32 * TILE_C : 8];
+  __shared__ __align__(16) uint32_t stash[STASH ? 32 * TILE_C : 4];
   __shared__ uint32_t blkmax[8];
-  __shared__ uint32_t stage[(DO_COL && RHT) ? 256 * STAGE_PITCH : 1];
   __shared__ uint8_t sperm[32];
+  static_assert(!(DO_COL && RHT) || sizeof(T) * 32 * TILE_C >= 256 * STAGE_PITCH * 4, "the byte scratch of the column phase reuses the tile");
 
   const int tid = threadIdx.x;
   const int col0 = blockIdx.x * TILE_C;
@@ -87,50 +102,77 @@ __global__ __launch_bounds__(256) void quant_kernel(const QuantParams p) {
   const int M = p.M, C = p.C;
 
   if (RHT || B2D) {
-    if (tid == 0) {
-#pragma unroll
-      for (int k = 0; k < 32; ++k) sperm[k] = p.perm[k];
-    }
+    if (tid < 32) sperm[tid] = (uint8_t)((p.perm4[tid >> 2] >> (8 * (tid & 3))) & 0xFFu);
     if (tid < 8) blkmax[tid] = 0;
     __syncthreads();
   }
 
-  // Tile-relative addressing: the descriptors start at the tile's first row, per-lane offsets are 32-bit, and the row
-  // step of each load is a scalar offset, so no load needs 64-bit address arithmetic.  (The host bounds ld_x / ld_rand.)
   const int rows_here = M - row0 < 32 ? M - row0 : 32;
   const T* xt = reinterpret_cast<const T*>(p.x) + b * p.bs_x + (int64_t)row0 * p.ld_x;
   const __amdgpu_buffer_rsrc_t rsrc_x = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<T*>(xt), 0, (int)(((int64_t)(rows_here - 1) * p.ld_x + C) * (int64_t)sizeof(T)), 0x00020000);
-  const uint32_t* rt_ = SR ? p.rand + b * p.bs_r + (int64_t)row0 * p.ld_r : nullptr;
+  const uint32_t* rt_ = SR == 1 ? p.rand + b * p.bs_r + (int64_t)row0 * p.ld_r : nullptr;
   const __amdgpu_buffer_rsrc_t rsrc_r = __builtin_amdgcn_make_buffer_rsrc(
-      const_cast<uint32_t*>(rt_), 0, SR ? (int)(((int64_t)(rows_here - 1) * p.ld_r + C) * 4) : 0, 0x00020000);
+      const_cast<uint32_t*>(rt_), 0, SR == 1 ? (int)(((int64_t)(rows_here - 1) * p.ld_r + C) * 4) : 0, 0x00020000);
   const int ldx_b = (int)p.ld_x * (int)sizeof(T), ldr_b = (int)p.ld_r * 4;   // row pitches in bytes
 
+  // Philox: element (b, i, j) consumes word ((b M + i) C + j) of the stream, i.e. word j % 4 of the block with the
+  // counter ctr0 + ((b M + i) C + j) / 4.  A lane owns 8 consecutive elements of a row = two blocks.
+  uint64_t key = 0, ctr0 = 0, qbase = 0;
+  if constexpr (SR == 2) {
+    key = p.philox_state ? p.philox_state[0] : p.seed;
+    ctr0 = p.philox_state ? p.philox_state[1] : p.ctr0;
+    qbase = ctr0 + (((uint64_t)b * (uint64_t)M + (uint64_t)row0) * (uint64_t)C >> 2);
+  }
+
   // ------------------------------------------------------------------ row phase
-  const int chunk = tid & 31;
+  const int chunk = tid & 31, rsub = tid >> 5;
   const int c = col0 + chunk * 8;
+  const bool cok = c < C;
   uint32_t w[4][BF ? 4 : 8];
+  uint32_t rr[4][(SR != 0 && (DO_ROW || STASH)) ? 8 : 1];
   uint32_t amax_i[4];
   bool valid[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    const int r = (tid >> 5) + 8 * i;
-    valid[i] = (row0 + r < M) && (c < C);
-    {
-      // rows past M are out of the descriptor's range and read as zeros; columns past C get an out-of-range offset
-      const int voff = valid[i] ? (tid >> 5) * ldx_b + c * (int)sizeof(T) : (int)0x80000000;
-      const v4i_t v0 = __builtin_amdgcn_raw_buffer_load_b128(rsrc_x, voff, 8 * i * ldx_b, 0);
-      w[i][0] = v0[0]; w[i][1] = v0[1]; w[i][2] = v0[2]; w[i][3] = v0[3];
-      if constexpr (!BF) {
-        const v4i_t v1 = __builtin_amdgcn_raw_buffer_load_b128(rsrc_x, voff, 8 * i * ldx_b + 16, 0);
-        w[i][4] = v1[0]; w[i][5] = v1[1]; w[i][6] = v1[2]; w[i][7] = v1[3];
-      }
+    const int r = rsub + 8 * i;
+    valid[i] = (row0 + r < M) && cok;
+    // rows past M are out of the descriptor's range and read as zeros; columns past C get an out-of-range offset
+    const int voff = valid[i] ? rsub * ldx_b + c * (int)sizeof(T) : OOB;
+    const v4i_t v0 = __builtin_amdgcn_raw_buffer_load_b128(rsrc_x, voff, 8 * i * ldx_b, 0);
+    w[i][0] = v0[0]; w[i][1] = v0[1]; w[i][2] = v0[2]; w[i][3] = v0[3];
+    if constexpr (!BF) {
+      const v4i_t v1 = __builtin_amdgcn_raw_buffer_load_b128(rsrc_x, voff, 8 * i * ldx_b + 16, 0);
+      w[i][4] = v1[0]; w[i][5] = v1[1]; w[i][6] = v1[2]; w[i][7] = v1[3];
+    }
+    if constexpr (SR == 1 && (DO_ROW || STASH)) {
+      const int roff = valid[i] ? rsub * ldr_b + c * 4 : OOB;
+      const v4i_t r0 = __builtin_amdgcn_raw_buffer_load_b128(rsrc_r, roff, 8 * i * ldr_b, 0);
+      const v4i_t r1 = __builtin_amdgcn_raw_buffer_load_b128(rsrc_r, roff, 8 * i * ldr_b + 16, 0);
+      rr[i][0] = r0[0]; rr[i][1] = r0[1]; rr[i][2] = r0[2]; rr[i][3] = r0[3];
+      rr[i][4] = r1[0]; rr[i][5] = r1[1]; rr[i][6] = r1[2]; rr[i][7] = r1[3];
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = rsub + 8 * i;
+    if constexpr (SR == 2) {
+      const uint64_t q0 = qbase + (uint64_t)(uint32_t)((r * C + c) >> 2), q1 = q0 + 1;   // 128-bit counters: the carry goes up
+      const uint4 a = philox4x32_10(q0, q0 < ctr0 ? 1ull : 0ull, key);
+      const uint4 d = philox4x32_10(q1, q1 < ctr0 ? 1ull : 0ull, key);
+      rr[i][0] = a.x; rr[i][1] = a.y; rr[i][2] = a.z; rr[i][3] = a.w;
+      rr[i][4] = d.x; rr[i][5] = d.y; rr[i][6] = d.z; rr[i][7] = d.w;
     }
     if (DO_COL) {
       const int pos = RHT ? sperm[r] : r;
       uint4* dst = reinterpret_cast<uint4*>(&tile[pos * TILE_C + chunk * 8]);
       dst[0] = make_uint4(w[i][0], w[i][1], w[i][2], w[i][3]);
       if constexpr (!BF) dst[1] = make_uint4(w[i][4], w[i][5], w[i][6], w[i][7]);
+      if constexpr (STASH) {   // the word of row r waits at the position its element takes in the transform
+        uint4* sd = reinterpret_cast<uint4*>(&stash[pos * TILE_C + chunk * 8]);
+        sd[0] = make_uint4(rr[i][0], rr[i][1], rr[i][2], rr[i][3]);
+        sd[1] = make_uint4(rr[i][4], rr[i][5], rr[i][6], rr[i][7]);
+      }
     }
     if (DO_ROW || B2D) {
       uint32_t a;
@@ -152,26 +194,27 @@ __global__ __launch_bounds__(256) void quant_kernel(const QuantParams p) {
   if (B2D || DO_COL) __syncthreads();
 
   if (DO_ROW || B2D) {
+    // descriptors of the row outputs start at the tile's first row
+    const __amdgpu_buffer_rsrc_t rsrc_rc = __builtin_amdgcn_make_buffer_rsrc(
+        DO_ROW ? p.row_codes + (b * M + row0) * p.ld_rc : nullptr, 0, DO_ROW ? 0x7FFFFFFF : 0, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc_rs = __builtin_amdgcn_make_buffer_rsrc(
+        (DO_ROW && !B2D) ? p.row_scales + (b * M + row0) * (int64_t)(C / 32) : nullptr, 0, (DO_ROW && !B2D) ? 0x7FFFFFFF : 0, 0x00020000);
+    const int ldrc = (int)p.ld_rc, ldrs = C / 32;
     uint32_t blk = B2D ? blkmax[chunk >> 2] : 0;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const int r = (tid >> 5) + 8 * i;
       const uint32_t a = B2D ? blk : amax_i[i];
       uint32_t s;
       if (GEN && p.uos) s = e8m0_uos(BF ? u2f(a << 16) : u2f(a));
       else s = BF ? e8m0_from_bf16_bits(a) : e8m0_from_f32_bits(a);
-      if (!valid[i]) continue;
-      const int64_t row = row0 + r;
       // scales
-      if ((tid & 3) == 0) {
-        if (!B2D) {
-          if (DO_ROW) p.row_scales[(b * M + row) * (C / 32) + (c >> 5)] = (uint8_t)s;
-        } else if (r == 0) {
-          if (DO_ROW) p.row_scales[(b * (M / 32) + blockIdx.y) * (C / 32) + (c >> 5)] = (uint8_t)s;
-          if (DO_COL) p.col_scales[(b * (C / 32) + (c >> 5)) * (M / 32) + blockIdx.y] = (uint8_t)s;
-        }
+      if (!B2D) {
+        if (DO_ROW) __builtin_amdgcn_raw_buffer_store_b8((uint8_t)s, rsrc_rs, (valid[i] && (tid & 3) == 0) ? rsub * ldrs + (c >> 5) : OOB, 8 * i * ldrs, 0);
+      } else if (i == 0 && rsub == 0 && (tid & 3) == 0 && valid[0]) {
+        if (DO_ROW) p.row_scales[(b * (M / 32) + blockIdx.y) * (C / 32) + (c >> 5)] = (uint8_t)s;
+        if (DO_COL) p.col_scales[(b * (C / 32) + (c >> 5)) * (M / 32) + blockIdx.y] = (uint8_t)s;
       }
-      if (!DO_ROW) continue;
+      if constexpr (DO_ROW) {
       const float scale_f = u2f(s << 23);
       float v[8];
 #pragma unroll
@@ -181,33 +224,29 @@ __global__ __launch_bounds__(256) void quant_kernel(const QuantParams p) {
         if (GEN && p.clip_row) v[e] = round_to_T<T>(v[e] * 0.75f);
       }
       uint32_t out = 0;
-      if (!SR) {
+      if constexpr (SR == 0) {
         out = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(out, v[0], v[1], scale_f, 0);
         out = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(out, v[2], v[3], scale_f, 1);
         out = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(out, v[4], v[5], scale_f, 2);
         out = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(out, v[6], v[7], scale_f, 3);
       } else {
         const float inv = u2f((254u - s) << 23);
-        const int roff = (tid >> 5) * ldr_b + c * 4;
-        const v4i_t r0 = __builtin_amdgcn_raw_buffer_load_b128(rsrc_r, roff, 8 * i * ldr_b, 0);
-        const v4i_t r1 = __builtin_amdgcn_raw_buffer_load_b128(rsrc_r, roff, 8 * i * ldr_b + 16, 0);
-        uint32_t rr[8] = {(uint32_t)r0[0], (uint32_t)r0[1], (uint32_t)r0[2], (uint32_t)r0[3],
-                          (uint32_t)r1[0], (uint32_t)r1[1], (uint32_t)r1[2], (uint32_t)r1[3]};
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
-          float q = v[e] * inv;
-          uint32_t code = e2m1_sr_mag(__builtin_fabsf(q), rr[e]) | ((f2u(q) >> 28) & 8u);
+          const float q = v[e] * inv;
+          const uint32_t code = e2m1_sr_mag(q, rr[i][e]) | ((f2u(q) >> 28) & 8u);
           out |= code << (4 * e);
         }
       }
-      *reinterpret_cast<uint32_t*>(p.row_codes + (b * M + row) * p.ld_rc + (c >> 1)) = out;
+      __builtin_amdgcn_raw_buffer_store_b32(out, rsrc_rc, valid[i] ? rsub * ldrc + (c >> 1) : OOB, 8 * i * ldrc, 0);
+      }
     }
   }
 
   // ------------------------------------------------------------------ column phase
   if (DO_COL) {
     const int cc = col0 + tid;
-    if (cc >= C) return;
+    const bool cvalid = cc < C;
     float z[32];
 #pragma unroll
     for (int k = 0; k < 32; ++k) {
@@ -215,6 +254,7 @@ __global__ __launch_bounds__(256) void quant_kernel(const QuantParams p) {
       else z[k] = reinterpret_cast<const float*>(tile)[k * TILE_C + tid];
     }
     if (RHT) {
+      __syncthreads();   // every thread holds its column: the tile's memory becomes the byte scratch used further down
 #pragma unroll
       for (int h = 1; h < 32; h <<= 1) {
 #pragma unroll
@@ -241,9 +281,9 @@ __global__ __launch_bounds__(256) void quant_kernel(const QuantParams p) {
       if constexpr (BF) {   // round to bf16 two at a time
 #pragma unroll
         for (int k = 0; k < 32; k += 2) {
-          const uint32_t w = pack_bf16x2(z[k], z[k + 1]);
-          z[k] = u2f(w << 16);
-          z[k + 1] = u2f(w & 0xFFFF0000u);
+          const uint32_t w2 = pack_bf16x2(z[k], z[k + 1]);
+          z[k] = u2f(w2 << 16);
+          z[k + 1] = u2f(w2 & 0xFFFF0000u);
         }
       }
     }
@@ -258,7 +298,9 @@ __global__ __launch_bounds__(256) void quant_kernel(const QuantParams p) {
       for (int k = 0; k < 32; k += 2) am = __builtin_fmaxf(__builtin_fmaxf(am, __builtin_fabsf(z[k])), __builtin_fabsf(z[k + 1]));
       if (GEN && p.uos) s = e8m0_uos(am);
       else s = BF ? e8m0_from_bf16_bits(f2u(am) >> 16) : e8m0_from_f32_bits(f2u(am));
-      p.col_scales[(b * C + cc) * (M / 32) + blockIdx.y] = (uint8_t)s;
+      const __amdgpu_buffer_rsrc_t rsrc_cs = __builtin_amdgcn_make_buffer_rsrc(
+          p.col_scales + (b * C + col0) * (int64_t)(M / 32) + blockIdx.y, 0, 0x7FFFFFFF, 0x00020000);
+      __builtin_amdgcn_raw_buffer_store_b8((uint8_t)s, rsrc_cs, cvalid ? tid * (M / 32) : OOB, 0, 0);
     }
     const float scale_f = u2f(s << 23);
     const float inv = u2f((254u - s) << 23);
@@ -267,21 +309,27 @@ __global__ __launch_bounds__(256) void quant_kernel(const QuantParams p) {
     for (int k = 0; k < 32; ++k) {
       float v = z[k];
       if (GEN && p.clip_col) v = round_to_T<T>(v * 0.75f);
-      if (!SR) {
+      if constexpr (SR == 0) {
         codes[k] = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(0u, v, 0.0f, scale_f, 0) & 0xFu;
       } else {
-        const int row = RHT ? p.perm_inv[k] : k;
-        const uint32_t r = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rsrc_r, tid * 4 + col0 * 4, __builtin_amdgcn_readfirstlane(row * ldr_b), 0);
-        float q = v * inv;
-        codes[k] = e2m1_sr_mag(__builtin_fabsf(q), r) | ((f2u(q) >> 28) & 8u);
+        uint32_t r;
+        if constexpr (STASH) {
+          r = stash[k * TILE_C + tid];
+        } else {
+          const int row = RHT ? packed_byte(p.pinv4, k) : k;
+          r = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rsrc_r, cvalid ? tid * 4 + col0 * 4 : OOB, __builtin_amdgcn_readfirstlane(row * ldr_b), 0);
+        }
+        const float q = v * inv;
+        codes[k] = e2m1_sr_mag(q, r) | ((f2u(q) >> 28) & 8u);
       }
     }
     uint32_t out[4];
     if (RHT) {
       // undo the permutation: position k belongs to row perm_inv[k]; a private byte scratch in LDS does the indexing
+      uint32_t* stage = reinterpret_cast<uint32_t*>(tile);
       uint8_t* sb = reinterpret_cast<uint8_t*>(stage + tid * STAGE_PITCH);
 #pragma unroll
-      for (int k = 0; k < 32; ++k) sb[p.perm_inv[k]] = (uint8_t)codes[k];
+      for (int k = 0; k < 32; ++k) sb[packed_byte(p.pinv4, k)] = (uint8_t)codes[k];
       // same thread reads what it wrote: LDS ops of one wave complete in order, no barrier needed
       uint32_t d[8];
 #pragma unroll
@@ -301,7 +349,9 @@ __global__ __launch_bounds__(256) void quant_kernel(const QuantParams p) {
         out[j] = o;
       }
     }
-    *reinterpret_cast<uint4*>(p.col_codes + (b * C + cc) * p.ld_cc + blockIdx.y * 16) = make_uint4(out[0], out[1], out[2], out[3]);
+    const __amdgpu_buffer_rsrc_t rsrc_cc = __builtin_amdgcn_make_buffer_rsrc(
+        p.col_codes + (b * C + col0) * p.ld_cc + blockIdx.y * 16, 0, 0x7FFFFFFF, 0x00020000);
+    __builtin_amdgcn_raw_buffer_store_b128(v4u_t{out[0], out[1], out[2], out[3]}, rsrc_cc, cvalid ? tid * (int)p.ld_cc : OOB, 0, 0);
   }
 }
 
@@ -316,7 +366,7 @@ __global__ __launch_bounds__(256) void hadamard_kernel(const T* __restrict__ x, 
   float z[32];
 #pragma unroll
   for (int k = 0; k < 32; ++k) {
-    const T v = x[(row0 + p.perm_inv[k]) * ld_x + cc];
+    const T v = x[(row0 + packed_byte(p.pinv4, k)) * ld_x + cc];
     if constexpr (sizeof(T) == 2) z[k] = u2f((uint32_t)__builtin_bit_cast(unsigned short, v) << 16);
     else z[k] = v;
   }
@@ -337,7 +387,7 @@ __global__ __launch_bounds__(256) void hadamard_kernel(const T* __restrict__ x, 
     T o;
     if constexpr (sizeof(T) == 2) o = __builtin_bit_cast(T, (unsigned short)f32_to_bf16_bits(q));
     else o = q;
-    y[(row0 + p.perm_inv[k]) * ld_y + cc] = o;
+    y[(row0 + packed_byte(p.pinv4, k)) * ld_y + cc] = o;
   }
 }
 
@@ -346,12 +396,13 @@ int fill_hadamard(QuantParams& p, const int8_t* signs, const uint8_t* perm, cons
   p.sign_mask = 0;
   uint32_t seen = 0;
   ALTO_REQUIRE(signs != nullptr, "%s: hadamard set but signs is NULL", who);
+  for (int w = 0; w < 8; ++w) p.perm4[w] = p.pinv4[w] = 0;
   for (int j = 0; j < 32; ++j) {
     int k = perm ? perm[j] : j;
     ALTO_REQUIRE(k >= 0 && k < 32 && !((seen >> k) & 1u), "%s: perm is not a permutation of 0..31", who);
     seen |= 1u << k;
-    p.perm[j] = (uint8_t)k;
-    p.perm_inv[k] = (uint8_t)j;
+    p.perm4[j >> 2] |= (uint32_t)k << (8 * (j & 3));
+    p.pinv4[k >> 2] |= (uint32_t)j << (8 * (k & 3));
   }
   for (int k = 0; k < 32; ++k) {
     ALTO_REQUIRE(signs[k] == 1 || signs[k] == -1, "%s: signs[%d] = %d is not +1/-1", who, k, (int)signs[k]);
@@ -360,12 +411,12 @@ int fill_hadamard(QuantParams& p, const int8_t* signs, const uint8_t* perm, cons
   return ALTO_MXFP4_OK;
 }
 
-template <typename T, bool DO_ROW, bool DO_COL, bool SR, bool RHT, bool B2D, bool GEN>
+template <typename T, bool DO_ROW, bool DO_COL, int SR, bool RHT, bool B2D, bool GEN>
 void launch(const QuantParams& p, dim3 grid, hipStream_t st) {
   hipLaunchKernelGGL((quant_kernel<T, DO_ROW, DO_COL, SR, RHT, B2D, GEN>), grid, dim3(256), 0, st, p);
 }
 
-template <typename T, bool SR, bool GEN>
+template <typename T, int SR, bool GEN>
 void dispatch_mode(const QuantParams& p, dim3 grid, hipStream_t st, bool do_row, bool do_col, bool rht, bool b2d) {
   if (b2d) {
     if (do_row && do_col) launch<T, true, true, SR, false, true, GEN>(p, grid, st);
@@ -383,14 +434,101 @@ void dispatch_mode(const QuantParams& p, dim3 grid, hipStream_t st, bool do_row,
 }
 
 template <typename T>
-void dispatch(const QuantParams& p, dim3 grid, hipStream_t st, bool do_row, bool do_col, bool rht, bool b2d, bool sr, bool gen) {
+void dispatch(const QuantParams& p, dim3 grid, hipStream_t st, bool do_row, bool do_col, bool rht, bool b2d, int sr, bool gen) {
   if (gen) {
-    if (sr) dispatch_mode<T, true, true>(p, grid, st, do_row, do_col, rht, b2d);
-    else dispatch_mode<T, false, true>(p, grid, st, do_row, do_col, rht, b2d);
+    if (sr == 2) dispatch_mode<T, 2, true>(p, grid, st, do_row, do_col, rht, b2d);
+    else if (sr == 1) dispatch_mode<T, 1, true>(p, grid, st, do_row, do_col, rht, b2d);
+    else dispatch_mode<T, 0, true>(p, grid, st, do_row, do_col, rht, b2d);
   } else {
-    if (sr) dispatch_mode<T, true, false>(p, grid, st, do_row, do_col, rht, b2d);
-    else dispatch_mode<T, false, false>(p, grid, st, do_row, do_col, rht, b2d);
+    if (sr == 2) dispatch_mode<T, 2, false>(p, grid, st, do_row, do_col, rht, b2d);
+    else if (sr == 1) dispatch_mode<T, 1, false>(p, grid, st, do_row, do_col, rht, b2d);
+    else dispatch_mode<T, 0, false>(p, grid, st, do_row, do_col, rht, b2d);
   }
+}
+
+}  // namespace
+}  // namespace alto
+
+namespace alto {
+namespace {
+
+// one-thread kernel: moves the counter of a device-resident Philox state past the blocks a quantizer call consumed
+__global__ void philox_advance_kernel(uint64_t* state, uint64_t blocks) { state[1] += blocks; }
+
+// sr_mode: 0 round to nearest even, 1 stochastic with the words in rand_bits, 2 stochastic with Philox words made in the kernel
+int quantize_impl(const void* x, int dtype, int64_t batch, int64_t M, int64_t C, int64_t ld_x, int64_t bs_x,
+                  uint8_t* row_codes, uint8_t* row_scales, uint8_t* col_codes, uint8_t* col_scales,
+                  int64_t ld_row_codes, int64_t ld_col_codes, int is_2d, int sr_mode,
+                  const uint32_t* rand_bits, int64_t ld_rand, int64_t bs_rand, uint64_t seed, uint64_t offset, const uint64_t* philox_state,
+                  int hadamard, const int8_t* signs, const uint8_t* perm, int clip_mode, int use_uos, void* stream) {
+  if (ld_row_codes == 0) ld_row_codes = C / 2;
+  if (ld_col_codes == 0) ld_col_codes = M / 2;
+  ALTO_REQUIRE(row_codes == nullptr || (ld_row_codes >= C / 2 && ld_row_codes % 4 == 0), "quantize: ld_row_codes must be >= C/2 and a multiple of 4 bytes");
+  ALTO_REQUIRE(col_codes == nullptr || (ld_col_codes >= M / 2 && ld_col_codes % 16 == 0), "quantize: ld_col_codes must be >= M/2 and a multiple of 16 bytes");
+  ALTO_REQUIRE(ld_row_codes < (1ll << 26) && ld_col_codes < (1ll << 23), "quantize: code row pitch out of range");
+  const bool do_row = row_codes != nullptr, do_col = col_codes != nullptr;
+  ALTO_REQUIRE(x != nullptr, "quantize: x is NULL");
+  ALTO_REQUIRE(dtype == ALTO_DT_BF16 || dtype == ALTO_DT_F32, "quantize: dtype %d is neither bf16 (0) nor f32 (1)", dtype);
+  ALTO_REQUIRE(do_row || do_col, "quantize: neither a row nor a column output was requested");
+  ALTO_REQUIRE(!do_row || row_scales != nullptr, "quantize: row_codes given without row_scales");
+  ALTO_REQUIRE(!do_col || col_scales != nullptr, "quantize: col_codes given without col_scales");
+  ALTO_REQUIRE(batch >= 0 && M >= 0 && C >= 0, "quantize: negative size");
+  ALTO_REQUIRE(M < (1ll << 31) && C < (1ll << 31) && batch < 65536, "quantize: size out of range");
+  ALTO_REQUIRE(C % 8 == 0, "quantize: C (%lld) must be a multiple of 8", (long long)C);
+  ALTO_REQUIRE(!do_row || C % 32 == 0, "quantize: row output needs C (%lld) %% 32 == 0", (long long)C);
+  ALTO_REQUIRE(!(do_col || is_2d) || M % 32 == 0, "quantize: column output / 2D blocks need M (%lld) %% 32 == 0", (long long)M);
+  ALTO_REQUIRE(!is_2d || C % 32 == 0, "quantize: 2D blocks need C (%lld) %% 32 == 0", (long long)C);
+  const int64_t vec = dtype == ALTO_DT_BF16 ? 8 : 4;
+  ALTO_REQUIRE(ld_x >= C && ld_x % vec == 0 && bs_x % vec == 0, "quantize: ld_x/bs_x must be >= C and multiples of %lld elements", (long long)vec);
+  ALTO_REQUIRE((reinterpret_cast<uintptr_t>(x) & 15) == 0, "quantize: x must be 16-byte aligned");
+  ALTO_REQUIRE(ld_x < (1ll << 24) && ld_rand < (1ll << 24), "quantize: row strides of 2^24 elements or more are not supported");
+  if (sr_mode == 1) {
+    ALTO_REQUIRE(rand_bits != nullptr, "quantize: stochastic rounding needs rand_bits");
+    ALTO_REQUIRE(ld_rand >= C && ld_rand % 4 == 0 && bs_rand % 4 == 0, "quantize: ld_rand/bs_rand must be >= C and multiples of 4");
+    ALTO_REQUIRE((reinterpret_cast<uintptr_t>(rand_bits) & 15) == 0, "quantize: rand_bits must be 16-byte aligned");
+  }
+  ALTO_REQUIRE(!hadamard || (!is_2d && do_col), "quantize: the Hadamard transform applies to a 1D column output only");
+  ALTO_REQUIRE(clip_mode == ALTO_CLIP_NONE || clip_mode == ALTO_CLIP_STATIC || clip_mode == ALTO_CLIP_DYNAMIC, "quantize: bad clip_mode %d", clip_mode);
+  if (batch == 0 || M == 0 || C == 0) return ALTO_MXFP4_OK;
+  if (clip_mode == ALTO_CLIP_DYNAMIC) {   // std-based scale: separate plain kernel, quantisation along the contiguous dim
+    ALTO_REQUIRE(do_row && !do_col && !hadamard && !use_uos,
+                 "quantize: clip_mode=dynamic gives the row output only (no column output, Hadamard or UOS); transpose on the host");
+    if (sr_mode == 2) {
+      set_error("quantize: clip_mode=dynamic takes its random words from a tensor (fill one with alto_mxfp4_random_bits)");
+      return ALTO_MXFP4_ENOTIMPL;
+    }
+    ALTO_REQUIRE(ld_row_codes % 16 == 0, "quantize: clip_mode=dynamic needs 16-byte aligned code rows");
+    ALTO_REQUIRE((M + 31) / 32 <= 65535, "quantize: M (%lld) exceeds 65535 row blocks", (long long)M);
+    return quantize_dynamic_launch(x, dtype, batch, M, C, ld_x, bs_x, row_codes, row_scales, ld_row_codes, is_2d, sr_mode == 1,
+                                   rand_bits, ld_rand, bs_rand, reinterpret_cast<hipStream_t>(stream));
+  }
+
+  QuantParams p;
+  p.x = x; p.ld_x = ld_x; p.bs_x = bs_x; p.M = (int)M; p.C = (int)C;
+  p.rand = rand_bits; p.ld_r = ld_rand; p.bs_r = bs_rand;
+  p.seed = seed; p.ctr0 = offset; p.philox_state = philox_state;
+  p.row_codes = row_codes; p.row_scales = row_scales; p.col_codes = col_codes; p.col_scales = col_scales;
+  p.ld_rc = ld_row_codes; p.ld_cc = ld_col_codes;
+  p.sign_mask = 0;
+  for (int w = 0; w < 8; ++w) p.perm4[w] = p.pinv4[w] = 0x03020100u + 0x04040404u * (uint32_t)w;   // identity
+  if (hadamard) {
+    int rc = fill_hadamard(p, signs, perm, "quantize");
+    if (rc != ALTO_MXFP4_OK) return rc;
+  }
+  const bool both = do_row && do_col;
+  p.clip_row = (clip_mode == ALTO_CLIP_STATIC && !both) ? 1 : 0;
+  p.clip_col = (clip_mode == ALTO_CLIP_STATIC) ? 1 : 0;
+  if (!do_col) p.clip_col = 0;
+  if (!do_row) p.clip_row = 0;
+  p.uos = use_uos ? 1 : 0;
+  const bool gen = p.clip_row || p.clip_col || p.uos;
+
+  dim3 grid((unsigned)((C + TILE_C - 1) / TILE_C), (unsigned)((M + 31) / 32), (unsigned)batch);
+  ALTO_REQUIRE(grid.y <= 65535u, "quantize: M (%lld) exceeds 65535 row blocks", (long long)M);
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  if (dtype == ALTO_DT_BF16) dispatch<__bf16>(p, grid, st, do_row, do_col, hadamard != 0, is_2d != 0, sr_mode, gen);
+  else dispatch<float>(p, grid, st, do_row, do_col, hadamard != 0, is_2d != 0, sr_mode, gen);
+  return check_launch("quantize");
 }
 
 }  // namespace
@@ -412,69 +550,29 @@ extern "C" int alto_mxfp4_quantize_pitched(const void* x, int dtype, int64_t bat
                                            int hadamard, const int8_t* signs, const uint8_t* perm,
                                            int clip_mode, int use_uos, void* stream) {
   using namespace alto;
-  if (ld_row_codes == 0) ld_row_codes = C / 2;
-  if (ld_col_codes == 0) ld_col_codes = M / 2;
-  ALTO_REQUIRE(row_codes == nullptr || (ld_row_codes >= C / 2 && ld_row_codes % 4 == 0), "quantize: ld_row_codes must be >= C/2 and a multiple of 4 bytes");
-  ALTO_REQUIRE(col_codes == nullptr || (ld_col_codes >= M / 2 && ld_col_codes % 16 == 0), "quantize: ld_col_codes must be >= M/2 and a multiple of 16 bytes");
-  const bool do_row = row_codes != nullptr, do_col = col_codes != nullptr;
-  ALTO_REQUIRE(x != nullptr, "quantize: x is NULL");
-  ALTO_REQUIRE(dtype == ALTO_DT_BF16 || dtype == ALTO_DT_F32, "quantize: dtype %d is neither bf16 (0) nor f32 (1)", dtype);
-  ALTO_REQUIRE(do_row || do_col, "quantize: neither a row nor a column output was requested");
-  ALTO_REQUIRE(!do_row || row_scales != nullptr, "quantize: row_codes given without row_scales");
-  ALTO_REQUIRE(!do_col || col_scales != nullptr, "quantize: col_codes given without col_scales");
-  ALTO_REQUIRE(batch >= 0 && M >= 0 && C >= 0, "quantize: negative size");
-  ALTO_REQUIRE(M < (1ll << 31) && C < (1ll << 31) && batch < 65536, "quantize: size out of range");
-  ALTO_REQUIRE(C % 8 == 0, "quantize: C (%lld) must be a multiple of 8", (long long)C);
-  ALTO_REQUIRE(!do_row || C % 32 == 0, "quantize: row output needs C (%lld) %% 32 == 0", (long long)C);
-  ALTO_REQUIRE(!(do_col || is_2d) || M % 32 == 0, "quantize: column output / 2D blocks need M (%lld) %% 32 == 0", (long long)M);
-  ALTO_REQUIRE(!is_2d || C % 32 == 0, "quantize: 2D blocks need C (%lld) %% 32 == 0", (long long)C);
-  const int64_t vec = dtype == ALTO_DT_BF16 ? 8 : 4;
-  ALTO_REQUIRE(ld_x >= C && ld_x % vec == 0 && bs_x % vec == 0, "quantize: ld_x/bs_x must be >= C and multiples of %lld elements", (long long)vec);
-  ALTO_REQUIRE((reinterpret_cast<uintptr_t>(x) & 15) == 0, "quantize: x must be 16-byte aligned");
-  ALTO_REQUIRE(ld_x < (1ll << 24) && ld_rand < (1ll << 24), "quantize: row strides of 2^24 elements or more are not supported");
   ALTO_REQUIRE(rounding == ALTO_ROUND_RNE || rounding == ALTO_ROUND_SR, "quantize: bad rounding mode %d", rounding);
-  if (rounding == ALTO_ROUND_SR) {
-    ALTO_REQUIRE(rand_bits != nullptr, "quantize: stochastic rounding needs rand_bits");
-    ALTO_REQUIRE(ld_rand >= C && ld_rand % 4 == 0 && bs_rand % 4 == 0, "quantize: ld_rand/bs_rand must be >= C and multiples of 4");
-    ALTO_REQUIRE((reinterpret_cast<uintptr_t>(rand_bits) & 15) == 0, "quantize: rand_bits must be 16-byte aligned");
-  }
-  ALTO_REQUIRE(!hadamard || (!is_2d && do_col), "quantize: the Hadamard transform applies to a 1D column output only");
-  ALTO_REQUIRE(clip_mode == ALTO_CLIP_NONE || clip_mode == ALTO_CLIP_STATIC || clip_mode == ALTO_CLIP_DYNAMIC, "quantize: bad clip_mode %d", clip_mode);
-  if (batch == 0 || M == 0 || C == 0) return ALTO_MXFP4_OK;
-  if (clip_mode == ALTO_CLIP_DYNAMIC) {   // std-based scale: separate plain kernel, quantisation along the contiguous dim
-    ALTO_REQUIRE(do_row && !do_col && !hadamard && !use_uos,
-                 "quantize: clip_mode=dynamic gives the row output only (no column output, Hadamard or UOS); transpose on the host");
-    ALTO_REQUIRE(ld_row_codes % 16 == 0, "quantize: clip_mode=dynamic needs 16-byte aligned code rows");
-    ALTO_REQUIRE((M + 31) / 32 <= 65535, "quantize: M (%lld) exceeds 65535 row blocks", (long long)M);
-    return quantize_dynamic_launch(x, dtype, batch, M, C, ld_x, bs_x, row_codes, row_scales, ld_row_codes, is_2d, rounding == ALTO_ROUND_SR,
-                                   rand_bits, ld_rand, bs_rand, reinterpret_cast<hipStream_t>(stream));
-  }
+  return quantize_impl(x, dtype, batch, M, C, ld_x, bs_x, row_codes, row_scales, col_codes, col_scales, ld_row_codes, ld_col_codes, is_2d,
+                       rounding == ALTO_ROUND_SR ? 1 : 0, rand_bits, ld_rand, bs_rand, 0, 0, nullptr, hadamard, signs, perm, clip_mode, use_uos, stream);
+}
 
-  QuantParams p;
-  p.x = x; p.ld_x = ld_x; p.bs_x = bs_x; p.M = (int)M; p.C = (int)C;
-  p.rand = rand_bits; p.ld_r = ld_rand; p.bs_r = bs_rand;
-  p.row_codes = row_codes; p.row_scales = row_scales; p.col_codes = col_codes; p.col_scales = col_scales;
-  p.ld_rc = ld_row_codes; p.ld_cc = ld_col_codes;
-  p.sign_mask = 0;
-  for (int k = 0; k < 32; ++k) { p.perm[k] = (uint8_t)k; p.perm_inv[k] = (uint8_t)k; }
-  if (hadamard) {
-    int rc = fill_hadamard(p, signs, perm, "quantize");
-    if (rc != ALTO_MXFP4_OK) return rc;
-  }
-  const bool both = do_row && do_col;
-  p.clip_row = (clip_mode == ALTO_CLIP_STATIC && !both) ? 1 : 0;
-  p.clip_col = (clip_mode == ALTO_CLIP_STATIC) ? 1 : 0;
-  if (!do_col) p.clip_col = 0;
-  if (!do_row) p.clip_row = 0;
-  p.uos = use_uos ? 1 : 0;
-  const bool gen = p.clip_row || p.clip_col || p.uos;
+extern "C" int alto_mxfp4_quantize_sr_philox(const void* x, int dtype, int64_t batch, int64_t M, int64_t C, int64_t ld_x, int64_t bs_x,
+                                             uint8_t* row_codes, uint8_t* row_scales, uint8_t* col_codes, uint8_t* col_scales,
+                                             int64_t ld_row_codes, int64_t ld_col_codes, int is_2d,
+                                             uint64_t seed, uint64_t offset, const uint64_t* philox_state,
+                                             int hadamard, const int8_t* signs, const uint8_t* perm,
+                                             int clip_mode, int use_uos, void* stream) {
+  using namespace alto;
+  ALTO_REQUIRE(C < (1ll << 26), "quantize_sr_philox: C (%lld) out of range", (long long)C);
+  ALTO_REQUIRE((reinterpret_cast<uintptr_t>(philox_state) & 7) == 0, "quantize_sr_philox: philox_state must be 8-byte aligned");
+  return quantize_impl(x, dtype, batch, M, C, ld_x, bs_x, row_codes, row_scales, col_codes, col_scales, ld_row_codes, ld_col_codes, is_2d,
+                       2, nullptr, 0, 0, seed, offset, philox_state, hadamard, signs, perm, clip_mode, use_uos, stream);
+}
 
-  dim3 grid((unsigned)((C + TILE_C - 1) / TILE_C), (unsigned)((M + 31) / 32), (unsigned)batch);
-  ALTO_REQUIRE(grid.y <= 65535u, "quantize: M (%lld) exceeds 65535 row blocks", (long long)M);
-  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-  if (dtype == ALTO_DT_BF16) dispatch<__bf16>(p, grid, st, do_row, do_col, hadamard != 0, is_2d != 0, rounding == ALTO_ROUND_SR, gen);
-  else dispatch<float>(p, grid, st, do_row, do_col, hadamard != 0, is_2d != 0, rounding == ALTO_ROUND_SR, gen);
-  return check_launch("quantize");
+extern "C" int alto_mxfp4_philox_advance(uint64_t* philox_state, uint64_t words, void* stream) {
+  using namespace alto;
+  ALTO_REQUIRE(philox_state != nullptr && (reinterpret_cast<uintptr_t>(philox_state) & 7) == 0, "philox_advance: philox_state must be a non-NULL 8-byte aligned device pointer");
+  hipLaunchKernelGGL(philox_advance_kernel, dim3(1), dim3(1), 0, reinterpret_cast<hipStream_t>(stream), philox_state, (words + 3) / 4);
+  return check_launch("philox_advance");
 }
 
 extern "C" int alto_mxfp4_hadamard(const void* x, int dtype, int64_t M, int64_t C, int64_t ld_x, void* y, int64_t ld_y,

@@ -52,6 +52,19 @@ def set_rand_bits_source(fn: Optional[Callable[[torch.Size, torch.device], torch
     _rand_source = fn
 
 
+def philox_in_kernel() -> bool:
+    """True when the quantizer may draw its random words itself (no source installed with ``set_rand_bits_source``)."""
+    return _rand_source is None
+
+
+def philox_seed_offset(seed: Optional[int], offset: Optional[int]):
+    """(key, counter start) of a Philox stream: the given ones, else 63 bits from torch's CPU generator (so that
+    ``torch.manual_seed`` makes a run repeatable and no device synchronisation is involved) and counter 0."""
+    if seed is None:
+        seed = int(torch.randint(0, 2 ** 63 - 1, (1,), dtype=torch.int64).item())
+    return int(seed) & (2 ** 64 - 1), int(offset or 0) & (2 ** 64 - 1)
+
+
 def draw_rand_bits(shape, device, seed: Optional[int] = None, offset: Optional[int] = None) -> torch.Tensor:
     """32 random bits per element for stochastic rounding (int32 tensor of ``shape`` on ``device``).
 
@@ -64,8 +77,7 @@ def draw_rand_bits(shape, device, seed: Optional[int] = None, offset: Optional[i
         r = _rand_source(torch.Size(shape), device)
         assert r.shape == torch.Size(shape) and r.dtype in (torch.int32, torch.uint32)
         return r
-    if seed is None:
-        seed = int(torch.randint(0, 2 ** 63 - 1, (1,), dtype=torch.int64).item())
+    seed, offset = philox_seed_offset(seed, offset)
     out = torch.empty(tuple(shape), dtype=torch.int32, device=device)
     if out.numel():
         from .._lib import check

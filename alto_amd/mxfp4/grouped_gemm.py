@@ -204,7 +204,8 @@ class MXFP4GroupedGEMM(torch.autograd.Function):
         groups = Groups(g_offs, g_expert, ctx.num_groups)
         go = grad_output if grad_output.is_contiguous() else grad_output.contiguous()
         sr = bool(ctx.use_sr_grad)
-        rand = rt.draw_rand_bits(go.shape, go.device) if sr else None
+        # random words: made inside the quantizer (Philox) unless a source of explicit words is installed
+        rand = rt.draw_rand_bits(go.shape, go.device) if (sr and not rt.philox_in_kernel()) else None
         go_q, go_s, go_qm, go_sm = quantize_rowcol(go, False, use_sr=sr, rand_bits=rand, hadamard=ctx.hadamard_transform,
                                                    clip_mode=ctx.clip_mode, use_uos=ctx.use_uos, pad_codes=True)
         grad_inputs = grouped_forward(go_q, go_s, wq_kn, ws_kn, groups, False, True, ctx.original_dtype)

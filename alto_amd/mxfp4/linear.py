@@ -237,7 +237,8 @@ class MXFP4LinearFunction(torch.autograd.Function):
         go = grad_output.reshape(-1, original_shape[-1])
         x_qm, x_sm, w_bwd, w_bwd_s = ctx.saved_tensors
         sr = bool(ctx.use_sr_grad)
-        rand = rt.draw_rand_bits(go.shape, go.device) if sr else None
+        # random words: made inside the quantizer (Philox) unless a source of explicit words is installed
+        rand = rt.draw_rand_bits(go.shape, go.device) if (sr and not rt.philox_in_kernel()) else None
         if ctx.use_2dblock_x:
             go_q, go_s = convert_to_mxfp4(go, axis=-1, is_2d_block=True, use_sr=sr, rand_bits=rand, use_uos=ctx.use_uos)
             go_qm, go_sm = go_q, go_s

@@ -49,9 +49,11 @@ def _code_buffer(B: int, R: int, nbytes: int, dev, pad: bool) -> torch.Tensor:
 
 def _quantize_call(x3: torch.Tensor, want_row: bool, want_col: bool, is_2d: bool, use_sr: bool,
                    rand3: Optional[torch.Tensor], hadamard: Optional[HadamardTransform], clip: int, use_uos: bool,
-                   pad_codes: bool = False):
+                   pad_codes: bool = False, philox: Optional[Tuple[int, int]] = None):
     """x3: [B, M, C] with unit stride along C and uniform row / batch strides. Returns the outputs (or None): dense, or
-    with ``pad_codes`` code tensors whose rows are padded to whole 128-byte cache lines (for GEMM operands)."""
+    with ``pad_codes`` code tensors whose rows are padded to whole 128-byte cache lines (for GEMM operands).
+    ``philox = (seed, offset)`` with ``use_sr`` and no ``rand3``: the kernel makes the random words itself, element
+    (b, i, j) taking word (b M + i) C + j of the stream ``alto_mxfp4_random_bits(.., seed, offset)`` writes."""
     B, M, C = x3.shape
     dev = x3.device
     row_codes = row_scales = col_codes = col_scales = None
@@ -65,9 +67,19 @@ def _quantize_call(x3: torch.Tensor, want_row: bool, want_col: bool, is_2d: bool
     ld_x = x3.stride(1) if M > 1 else C
     bs_x = x3.stride(0) if B > 1 else M * ld_x
     ld_r = bs_r = 0
-    if use_sr:
+    if use_sr and rand3 is not None:
         ld_r = rand3.stride(1) if M > 1 else C
         bs_r = rand3.stride(0) if B > 1 else M * ld_r
+    if use_sr and rand3 is None:
+        assert philox is not None, "stochastic rounding needs rand_bits or a Philox (seed, offset)"
+        rc = rt.lib().alto_mxfp4_quantize_sr_philox(
+            x3.data_ptr(), rt.dtype_code(x3.dtype), B, M, C, ld_x, bs_x,
+            rt.ptr(row_codes), rt.ptr(row_scales), rt.ptr(col_codes), rt.ptr(col_scales),
+            row_codes.stride(1) if want_row else 0, col_codes.stride(1) if want_col else 0,
+            int(is_2d), philox[0] & (2 ** 64 - 1), philox[1] & (2 ** 64 - 1), None,
+            had, sp, pp, clip, int(use_uos), rt.stream_ptr(dev))
+        check(rc, "alto_mxfp4_quantize_sr_philox")
+        return row_codes, row_scales, col_codes, col_scales
     rc = rt.lib().alto_mxfp4_quantize_pitched(
         x3.data_ptr(), rt.dtype_code(x3.dtype), B, M, C, ld_x, bs_x,
         rt.ptr(row_codes), rt.ptr(row_scales), rt.ptr(col_codes), rt.ptr(col_scales),
@@ -139,12 +151,17 @@ def convert_to_mxfp4(
     rt.require_gpu(data_hp)
     nd = data_hp.dim()
     ax = axis % nd
+    philox = None
     if use_sr:
-        if rand_bits is None:
-            rand_bits = rt.draw_rand_bits(data_hp.shape, data_hp.device, philox_seed, philox_offset)
-        assert rand_bits.shape == data_hp.shape, "rand_bits must have the shape of data_hp"
-        rt.require_gpu(rand_bits)
-        rand_bits = _as_i32(rand_bits)
+        if rand_bits is None and ax >= nd - 2 and clip_mode != "dynamic" and data_hp.shape[-1] < 2 ** 26 and rt.philox_in_kernel():
+            # the kernel makes the words itself: same bytes as rand_bits = draw_rand_bits(shape, seed, offset), no tensor
+            philox = rt.philox_seed_offset(philox_seed, philox_offset)
+        else:
+            if rand_bits is None:
+                rand_bits = rt.draw_rand_bits(data_hp.shape, data_hp.device, philox_seed, philox_offset)
+            assert rand_bits.shape == data_hp.shape, "rand_bits must have the shape of data_hp"
+            rt.require_gpu(rand_bits)
+            rand_bits = _as_i32(rand_bits)
     if hadamard is not None:
         assert nd == 2 and ax == 0 and not is_2d_block, "hadamard fuses with a 1D axis=-2 quantisation of a 2D tensor"
     if clip_mode == "dynamic" and data_hp.numel() != 0:
@@ -161,10 +178,10 @@ def convert_to_mxfp4(
         # quantise along the second-to-last dim: column output of the [.., M, C] matrices
         x3 = _prep(data_hp)
         r3 = None
-        if use_sr:
+        if use_sr and philox is None:
             r3 = rand_bits.expand_as(data_hp)
             r3 = _batched_view(r3 if r3.is_contiguous() else r3.contiguous())
-        _, _, cc, cs = _quantize_call(x3, False, True, is_2d_block, use_sr, r3, hadamard, clip, use_uos)
+        _, _, cc, cs = _quantize_call(x3, False, True, is_2d_block, use_sr, r3, hadamard, clip, use_uos, philox=philox)
         lead = data_hp.shape[:-2]
         M, C = data_hp.shape[-2], data_hp.shape[-1]
         codes = cc.reshape(*lead, C, M // 2).transpose(-1, -2)
@@ -174,13 +191,16 @@ def convert_to_mxfp4(
     # general case: move the axis last (view), then quantise along the contiguous dim
     xt = data_hp.transpose(ax, -1)
     shp = xt.shape
-    rtens = rand_bits.transpose(ax, -1) if use_sr else None
+    if philox is not None and ax != nd - 1:   # (only the last-axis case reaches here with Philox; other axes take a tensor)
+        rand_bits = _as_i32(rt.draw_rand_bits(data_hp.shape, data_hp.device, philox[0], philox[1]))
+        philox = None
+    rtens = rand_bits.transpose(ax, -1) if (use_sr and philox is None) else None
     if is_2d_block:
         x3 = _prep(xt)
         r3 = None
-        if use_sr:
+        if use_sr and philox is None:
             r3 = _batched_view(rtens.contiguous())
-        rcodes, rscales, _, _ = _quantize_call(x3, True, False, True, use_sr, r3, None, clip, use_uos)
+        rcodes, rscales, _, _ = _quantize_call(x3, True, False, True, use_sr, r3, None, clip, use_uos, philox=philox)
         codes = rcodes.reshape(*shp[:-1], shp[-1] // 2)
         scales = rscales.reshape(*shp[:-2], shp[-2] // 32, shp[-1] // 32)
     else:
@@ -188,9 +208,9 @@ def convert_to_mxfp4(
         if x2.stride(-1) != 1 or not _aligned(x2):
             x2 = x2.contiguous()
         r3 = None
-        if use_sr:
+        if use_sr and philox is None:
             r3 = rtens.reshape(-1, shp[-1]).contiguous().unsqueeze(0)
-        rcodes, rscales, _, _ = _quantize_call(x2.unsqueeze(0), True, False, False, use_sr, r3, None, clip, use_uos)
+        rcodes, rscales, _, _ = _quantize_call(x2.unsqueeze(0), True, False, False, use_sr, r3, None, clip, use_uos, philox=philox)
         codes = rcodes.reshape(*shp[:-1], shp[-1] // 2)
         scales = rscales.reshape(*shp[:-1], shp[-1] // 32)
     return codes.transpose(ax, -1), scales.transpose(ax, -1)
@@ -241,8 +261,12 @@ def quantize_rowcol(
     M, C = x.shape
     torch._check(M % 32 == 0 and C % 32 == 0)
     clip = _clip_code(clip_mode)
+    philox = None
     if use_sr and rand_bits is None:
-        rand_bits = rt.draw_rand_bits(x.shape, x.device)
+        if clip_mode != "dynamic" and C < 2 ** 26 and rt.philox_in_kernel():
+            philox = rt.philox_seed_offset(None, None)   # the kernel makes the words: no tensor, no fill launch
+        else:
+            rand_bits = rt.draw_rand_bits(x.shape, x.device)
     if clip_mode == "dynamic":   # the row pair is never clipped; the column pair takes the plain path
         rc, rs = convert_to_mxfp4(x, axis=-1, is_2d_block=is_2d_block, use_sr=use_sr, use_uos=use_uos, rand_bits=rand_bits)
         cc, cs = convert_to_mxfp4(x, axis=0, is_2d_block=is_2d_block, use_sr=use_sr, clip_mode="dynamic", use_uos=use_uos,
@@ -250,11 +274,11 @@ def quantize_rowcol(
         return rc, rs, cc, cs
     x3 = _prep(x)
     r3 = None
-    if use_sr:
+    if use_sr and philox is None:
         assert rand_bits.shape == x.shape
         r3 = _as_i32(rand_bits)
         r3 = _batched_view(r3 if r3.stride(-1) == 1 and r3.stride(0) % 4 == 0 and r3.data_ptr() % 16 == 0 else r3.contiguous())
-    rc, rs, cc, cs = _quantize_call(x3, True, True, is_2d_block, use_sr, r3, hadamard, clip, use_uos, pad_codes)
+    rc, rs, cc, cs = _quantize_call(x3, True, True, is_2d_block, use_sr, r3, hadamard, clip, use_uos, pad_codes, philox=philox)
     return rc[0], rs[0], cc[0].transpose(0, 1), cs[0].transpose(0, 1)
 
 

@@ -116,6 +116,29 @@ class FusedGradQuant(Workload):
         return run, self.work * rows / self.M, f"first {rows} of {self.M} rows, both copies"
 
 
+class FusedGradQuantPhilox(FusedGradQuant):
+    """The same pass as config 2 with the random words made inside the kernel (Philox4x32-10), as the autograd functions
+    run it: no random tensor is read (and none has to be filled first), so the algorithmic bytes are dY in and the four
+    outputs out."""
+    name = "cfg2_fused_rht_sr_quantizer[8192x4096], random words made in the kernel"
+    kernel = "quant_kernel<bf16, row+col, SR Philox, RHT>"
+
+    def setup(self, dev, gen):
+        super().setup(dev, gen)
+        self.r = None
+        self.work = self.M * self.C * 2 + 2 * (self.M * self.C // 2 + self.M * self.C // 32)
+
+    def step(self):
+        rt, (rc, rs, cc, cs) = self.rt, self.out
+        code = rt.lib().alto_mxfp4_quantize_sr_philox(self.x.data_ptr(), rt.dtype_code(self.x.dtype), 1, self.M, self.C, self.C, self.M * self.C,
+                                                      rc.data_ptr(), rs.data_ptr(), cc.data_ptr(), cs.data_ptr(), 0, 0, 0, 1234, 0, None,
+                                                      1, self.h.signs.data_ptr(), self.h.perm.data_ptr(), 0, 0, self.stream)
+        assert code == 0, code
+
+    def cpu_sample(self):
+        raise NotImplementedError("the CPU leg is the supplied-words workload's")
+
+
 class RneQuant(Workload):
     """Config 1: bf16 [4096, 4096] ~ N(0,1) with 1% x50 outliers, 1D-32 blocks, RNE, no Hadamard."""
     name = "cfg1_rne_quantizer[4096x4096]"
@@ -393,6 +416,7 @@ def make_workloads():
         "cfg3_fprop_vendor": VendorGemm("cfg3_fprop_gemm[8192x14336x4096] via torch._scaled_mm (1D scales on both operands)", 8192, 14336, 4096, False, False,
                                         "act", "weight"),
         "cfg2_quant": FusedGradQuant(),
+        "cfg2_quant_philox": FusedGradQuantPhilox(),
         "cfg1_quant": RneQuant(),
         # config 4: dgrad dX[8192,14336] = dY[8192,4096] . W^T-packed[14336,4096]; wgrad dW[4096,14336] over 8192 tokens
         "cfg4_dgrad": Gemm("cfg4_dgrad_gemm[8192x14336x4096]", 8192, 14336, 4096, False, True, "grad", "weight"),

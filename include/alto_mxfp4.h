@@ -101,6 +101,32 @@ int alto_mxfp4_quantize_pitched(const void* x, int dtype, int64_t batch, int64_t
                                 int clip_mode, int use_uos, void* stream);
 
 /*
+ * The same quantizer with stochastic rounding whose random words are made INSIDE the kernel: element x[b][i][j] consumes
+ * word ((b * M + i) * C + j) of the stream that alto_mxfp4_random_bits(out, n, seed, offset) writes (Philox4x32-10,
+ * key = seed, counter = offset + word / 4), for the row AND the column output.  Filling a dense [batch][M][C] tensor with
+ * alto_mxfp4_random_bits and passing it to alto_mxfp4_quantize_pitched gives the same bytes; this entry point reads no
+ * random tensor and needs no fill launch.  It stands for the in-kernel draw of the reference
+ * (tl.randint4x in alto/kernels/fp4/fp4_common/triton_fp4_ops.py:11-21, used at mxfp_quantization.py:129,184-185).
+ * philox_state: NULL, or DEVICE memory holding {uint64 key, uint64 counter}: the kernel then takes key and counter from
+ * there and ignores seed / offset, so that a captured launch (HIP graph) draws fresh words on every replay once the
+ * state is advanced between replays (alto_mxfp4_philox_advance).  clip_mode = dynamic is not offered here
+ * (ALTO_MXFP4_ENOTIMPL).  C < 2^26.
+ */
+int alto_mxfp4_quantize_sr_philox(const void* x, int dtype, int64_t batch, int64_t M, int64_t C, int64_t ld_x, int64_t bs_x,
+                                  uint8_t* row_codes, uint8_t* row_scales, uint8_t* col_codes, uint8_t* col_scales,
+                                  int64_t ld_row_codes, int64_t ld_col_codes, int is_2d,
+                                  uint64_t seed, uint64_t offset, const uint64_t* philox_state,
+                                  int hadamard, const int8_t* signs, const uint8_t* perm,
+                                  int clip_mode, int use_uos, void* stream);
+
+/*
+ * Moves the counter of a device-resident Philox state {key, counter} past `words` random words (counter += ceil(words / 4)),
+ * enqueued on `stream` after the quantizer call that consumed them.  A one-thread kernel; it can be captured together
+ * with that call.  No counterpart in the reference (its Philox offsets are host integers).
+ */
+int alto_mxfp4_philox_advance(uint64_t* philox_state, uint64_t words, void* stream);
+
+/*
  * Standalone randomized Hadamard transform along M in blocks of 32 rows:
  *   y[32b + i][c] = cast((sum_j W[i][j] * fp32(x[32b + j][c])) / float32(sqrt(32)))
  * with W built from signs/perm as in alto_mxfp4_quantize (same summation order, so

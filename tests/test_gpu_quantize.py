@@ -295,3 +295,41 @@ def test_default_random_bits_follow_the_torch_seed(m):
     w = rt.draw_rand_bits((1 << 20,), torch.device(DEV), seed=1).cpu().numpy().view(np.uint32)
     frac = np.array([((w >> b) & 1).mean() for b in range(32)])
     assert np.all(np.abs(frac - 0.5) < 0.005)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("shape", [(256, 512), (3, 64, 96), (8192, 4096)])
+def test_in_kernel_philox_equals_supplied_words(m, dtype, shape):
+    """Stochastic rounding with the random words made inside the kernel (Philox4x32-10, counter = element index / 4) gives
+    the bytes of the supplied-words path when the tensor is filled by alto_mxfp4_random_bits with the same key and
+    counter start -- which the oracle checks in turn: row copy, Hadamard column copy, 2D blocks, column copy alone."""
+    from alto_amd.mxfp4 import _runtime as rt
+    if dtype == torch.float32 and shape[0] == 8192:
+        pytest.skip("the large case runs in bf16")
+    seed, offset = 0x1234_5678_9ABC_DEF0, 2 ** 64 - 7          # the 128-bit counter wraps its low word inside the tensor
+    x = (laplace(shape, 1e-3, dtype, seed=5) if len(shape) == 2 else randn_outliers(shape, dtype, seed=6)).to(DEV)
+    words = rt.draw_rand_bits(x.shape, x.device, seed, offset)
+    n = x.numel()
+    import oracle.philox as P
+    head = torch.from_numpy(P.random_bits(min(n, 4096), seed, offset).view("int32"))
+    assert torch.equal(words.reshape(-1)[:head.numel()].cpu(), head), "fill kernel differs from the Philox oracle"
+    for kw in (dict(axis=-1), dict(axis=-2), dict(axis=-1, is_2d_block=True), dict(axis=-2, is_2d_block=True)):
+        q1, s1 = m.convert_to_mxfp4(x, use_sr=True, philox_seed=seed, philox_offset=offset, **kw)
+        q2, s2 = m.convert_to_mxfp4(x, use_sr=True, rand_bits=words, **kw)
+        assert torch.equal(q1, q2) and torch.equal(s1, s2), kw
+    if len(shape) == 2:
+        signs, perm = hadamard_from_seed(1234)
+        h = m.HadamardTransform(signs, perm)
+        torch.manual_seed(99)
+        a = m.quantize_rowcol(x, False, use_sr=True, hadamard=h)       # key drawn from torch's CPU generator
+        torch.manual_seed(99)
+        key, ctr = rt.philox_seed_offset(None, None)
+        b = m.quantize_rowcol(x, False, use_sr=True, rand_bits=rt.draw_rand_bits(x.shape, x.device, key, ctr), hadamard=h)
+        for t1, t2 in zip(a, b):
+            assert torch.equal(t1, t2)
+        # and the supplied-words result is the oracle's
+        if shape[0] <= 256:
+            eq, es = O.quantize(O.rht_left(x.cpu(), signs, perm), axis=0, use_sr=True, rand_bits=words.cpu())
+            cq, cs = m.convert_to_mxfp4(x, axis=0, use_sr=True, philox_seed=seed, philox_offset=offset, hadamard=h)
+            assert_bytes_equal(cq, eq, "Hadamard column codes (in-kernel Philox)")
+            assert_bytes_equal(cs, es, "Hadamard column scales (in-kernel Philox)")
