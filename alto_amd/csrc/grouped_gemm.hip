@@ -155,74 +155,108 @@ __device__ __forceinline__ void zero_rows(OutT* out, int64_t ldo, int64_t r0, in
   }
 }
 
-// The tile as a real function: inlined into the segment loop below, its address set-up competes with the loop's own
-// state for registers and spills.
-template <typename OutT, bool KTAIL>
-__device__ __noinline__ void grouped_tile_call(const TileArgs& ta_mem, OutT* out_v, int64_t ldo_v) {
-  extern __shared__ __align__(16) uint8_t smem[];
-  const TileArgs ta = uniform_args(ta_mem);
-  OutT* out = reinterpret_cast<OutT*>(uniform_i64(reinterpret_cast<int64_t>(out_v)));
-  const int64_t ldo = uniform_i64(ldo_v);
-  gemm_tile_256x256<OutT, KTAIL>(ta, out, ldo, smem);
+// ---- pass list.  The output rows are cut into passes: a pass is the part of one 256-row band that one expert serves
+// (adjacent groups of the same expert merge; rows that no group owns, or whose expert id is out of range, form passes of
+// expert -1 that are zero-filled).  A small plan kernel walks the offsets once and writes the list to a workspace in
+// device memory; the GEMM kernel then runs one workgroup per (pass, 256-column tile), exactly like the dense kernel:
+// no loop around the tile routine (which needs nearly every vector register), and passes of one band run in parallel.
+//   workspace: int32 n_pass, 3 x pad, then n_pass x {band row, first row, end row, expert}
+struct PassWalk {
+  const int32_t* offs;
+  const int32_t* group_expert;
+  int num_groups, num_experts;
+  int64_t M_total;
+  __device__ __forceinline__ int off_at(int g) const { return clamp_off(offs, g, M_total); }
+  __device__ __forceinline__ int expert_of(int g) const { return group_expert ? group_expert[g] : g; }
+  // calls emit(first row, end row, expert) for every pass of band tm, in row order
+  template <typename F>
+  __device__ __forceinline__ void band(int tm, F&& emit) const {
+    const int Mt = (int)M_total;
+    const int row0 = tm * GT_TM;
+    const int row1 = row0 + GT_TM < Mt ? row0 + GT_TM : Mt;
+    int lo = 0, hi = num_groups;   // first group that ends after row0
+    while (lo < hi) {
+      const int mid = (lo + hi) >> 1;
+      if (off_at(mid + 1) > row0) hi = mid; else lo = mid + 1;
+    }
+    int g = lo, cur = row0;
+    while (cur < row1) {
+      int e = -1, seg_end = row1;
+      while (g < num_groups && off_at(g + 1) <= cur) ++g;
+      if (g < num_groups) {
+        const int start = off_at(g);
+        if (start > cur) {   // rows before the next group
+          seg_end = start < row1 ? start : row1;
+        } else {
+          e = expert_of(g);
+          int end = off_at(g + 1);
+          while (end < row1 && g + 1 < num_groups && expert_of(g + 1) == e) {
+            ++g;
+            const int e2 = off_at(g + 1);
+            end = e2 > end ? e2 : end;
+          }
+          seg_end = end < row1 ? end : row1;
+          ++g;
+          if (e < 0 || e >= num_experts) e = -1;
+        }
+      }
+      emit(cur, seg_end, e);
+      cur = seg_end;
+    }
+  }
+};
+
+constexpr int PLAN_THREADS = 256;
+
+// one workgroup: thread t owns the bands [t nb, (t + 1) nb); counts their passes, then writes them at the offset an
+// exclusive scan of the counts gives, so the list is in band order
+__global__ __launch_bounds__(PLAN_THREADS) void grouped_plan_kernel(PassWalk wk, int tiles_m, int32_t* ws, int max_pass) {
+  __shared__ int scan[PLAN_THREADS];
+  const int t = threadIdx.x;
+  const int nb = (tiles_m + PLAN_THREADS - 1) / PLAN_THREADS;
+  const int b0 = t * nb, b1 = (b0 + nb) < tiles_m ? (b0 + nb) : tiles_m;
+  int cnt = 0;
+  for (int tm = b0; tm < b1; ++tm) wk.band(tm, [&](int, int, int) { ++cnt; });
+  scan[t] = cnt;
+  __syncthreads();
+  for (int d = 1; d < PLAN_THREADS; d <<= 1) {   // inclusive scan
+    const int v = t >= d ? scan[t - d] : 0;
+    __syncthreads();
+    scan[t] += v;
+    __syncthreads();
+  }
+  int at = scan[t] - cnt;
+  int4* list = reinterpret_cast<int4*>(ws + 4);
+  for (int tm = b0; tm < b1; ++tm)
+    wk.band(tm, [&](int lo, int hi, int e) {
+      if (at < max_pass) list[at] = make_int4(tm * GT_TM, lo, hi, e);
+      ++at;
+    });
+  if (t == PLAN_THREADS - 1) ws[0] = scan[t] < max_pass ? scan[t] : max_pass;
 }
 
-// One workgroup owns rows [256 tm, 256 tm + 256) x columns [256 tn, 256 tn + 256) of the output.  The rows are cut
-// into segments of one expert each (adjacent groups of the same expert merge); every segment is one pass of the tile
-// with its rows masked, rows that belong to no group or to an invalid expert are zero-filled.
 template <typename OutT, bool KTAIL>
 __global__ __launch_bounds__(GT_THREADS) void grouped_tiled_kernel(OperandView A, const uint8_t* w, int64_t w_stride_e, int64_t ldw,
                                                                    const uint8_t* w_scales, int64_t ws_stride_e, int64_t ws_r, int w_is_2d,
-                                                                   const int32_t* offs, const int32_t* group_expert, int num_groups, int num_experts,
-                                                                   int64_t M_total, int64_t N, int G, OutT* out, int64_t ldo, int tiles_m, int tiles_n) {
+                                                                   const int32_t* plan, int64_t M_total, int64_t N, int G, OutT* out, int64_t ldo, int tiles_n) {
   extern __shared__ __align__(16) uint8_t smem[];
-  int tm, tn;
-  if (!grouped_tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn)) return;
+  const int n_pass = __builtin_amdgcn_readfirstlane(plan[0]);
+  int pi, tn;
+  if (!grouped_tile_coords(blockIdx.x, n_pass, tiles_n, pi, tn)) return;
+  const int4 d = reinterpret_cast<const int4*>(plan + 4)[pi];
+  const int row0 = __builtin_amdgcn_readfirstlane(d.x), m_lo = __builtin_amdgcn_readfirstlane(d.y), m_hi = __builtin_amdgcn_readfirstlane(d.z);
+  const int e = __builtin_amdgcn_readfirstlane(d.w);
   const int n0 = tn * GT_TN;
-  const int n1 = n0 + GT_TN < (int)N ? n0 + GT_TN : (int)N;
-  const int Mt = (int)M_total;   // the host checks M_total < 2^31
-  const int row0 = tm * GT_TM;
-  const int row1 = row0 + GT_TM < Mt ? row0 + GT_TM : Mt;
-  // first group that ends after row0 (binary search over the group ends)
-  int lo = 0, hi = num_groups;
-  while (lo < hi) {
-    const int mid = (lo + hi) >> 1;
-    if (clamp_off(offs, mid + 1, M_total) > row0) hi = mid; else lo = mid + 1;
+  if (e < 0) {
+    const int n1 = n0 + GT_TN < (int)N ? n0 + GT_TN : (int)N;
+    zero_rows<OutT>(out, ldo, m_lo, m_hi, n0, n1);
+    return;
   }
-  int g = lo;
-  int cur = row0;
-  while (cur < row1) {
-    // next segment [cur, seg_end): expert e, or -1 for rows to zero-fill
-    int e = -1, seg_end = row1;
-    while (g < num_groups && clamp_off(offs, g + 1, M_total) <= cur) ++g;
-    if (g < num_groups) {
-      const int start = clamp_off(offs, g, M_total);
-      if (start > cur) {   // rows before the next group
-        seg_end = start < row1 ? start : row1;
-      } else {
-        e = group_expert ? group_expert[g] : g;
-        int end = clamp_off(offs, g + 1, M_total);
-        while (end < row1 && g + 1 < num_groups && (group_expert ? group_expert[g + 1] : g + 1) == e) {
-          ++g;
-          const int e2 = clamp_off(offs, g + 1, M_total);
-          end = e2 > end ? e2 : end;
-        }
-        seg_end = end < row1 ? end : row1;
-        ++g;
-        if (e >= num_experts) e = -1;
-      }
-    }
-    if (e < 0) {
-      zero_rows<OutT>(out, ldo, cur, seg_end, n0, n1);
-    } else {
-      OperandView B{w + e * w_stride_e, ldw, w_scales + e * ws_stride_e, ws_r, 1, w_is_2d};
-      TileArgs ta{A, B, row0, n0, cur, seg_end, N, G, 1.0f,
-                  (M_total - 1) * A.ld + G * 16, (N - 1) * ldw + G * 16,
-                  ((A.is_2d ? M_total / 32 : M_total) - 1) * A.ss_r + G, ((w_is_2d ? N / 32 : N) - 1) * ws_r + G, 0, G};
-      grouped_tile_call<OutT, KTAIL>(ta, out, ldo);
-      __syncthreads();   // the next segment reuses the LDS the store staged through
-    }
-    cur = seg_end;
-  }
+  OperandView B{w + e * w_stride_e, ldw, w_scales + e * ws_stride_e, ws_r, 1, w_is_2d};
+  TileArgs ta{A, B, row0, n0, m_lo, m_hi, N, G, 1.0f,
+              (M_total - 1) * A.ld + G * 16, (N - 1) * ldw + G * 16,
+              ((A.is_2d ? M_total / 32 : M_total) - 1) * A.ss_r + G, ((w_is_2d ? N / 32 : N) - 1) * ws_r + G, 0, G};
+  gemm_tile_256x256<OutT, KTAIL>(ta, out, ldo, smem);
 }
 
 // dW[e] tile: rows [256 tm, +256) of the first operand (P) x rows [256 tn, +256) of the second (Q), reduced over the
@@ -330,10 +364,14 @@ __global__ __launch_bounds__(GT_THREADS) void grouped_dw_tiled_kernel(OperandVie
   gemm_tile_store<OutT>(ta, acc, dw + e * s_e, ld, smem);
 }
 
+// upper bound on the number of passes: every band is one, every group start inside a band adds one, plus the unrouted head and tail
+inline int64_t grouped_max_passes(int64_t M_total, int64_t num_groups) { return (M_total + GT_TM - 1) / GT_TM + num_groups + 2; }
+inline int64_t grouped_workspace_bytes(int64_t M_total, int64_t num_groups) { return 16 + 16 * grouped_max_passes(M_total, num_groups); }
+
 template <typename OutT, bool KTAIL>
 int launch_grouped_tiled(const OperandView& A, const uint8_t* w, int64_t w_stride_e, int64_t ldw, const uint8_t* w_scales, int64_t ws_stride_e,
                          int64_t ws_r, int w_is_2d, const int32_t* offs, const int32_t* group_expert, int num_groups, int num_experts,
-                         int64_t M_total, int64_t N, int64_t K, void* out, int64_t ldo, hipStream_t st) {
+                         int64_t M_total, int64_t N, int64_t K, void* out, int64_t ldo, int32_t* plan, hipStream_t st) {
   // the opt-in for > 64 KB of dynamic LDS is per function, set once per process (thread-safe: forward and backward may
   // make their first calls from two host threads)
   auto kern = grouped_tiled_kernel<OutT, KTAIL>;
@@ -342,8 +380,11 @@ int launch_grouped_tiled(const OperandView& A, const uint8_t* w, int64_t w_strid
   std::call_once(once, [&] { attr_rc = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, GT_LDS_BYTES); });
   if (attr_rc != hipSuccess) return -1;
   const int tiles_m = (int)((M_total + GT_TM - 1) / GT_TM), tiles_n = (int)((N + GT_TN - 1) / GT_TN);
-  hipLaunchKernelGGL(kern, dim3((unsigned)grouped_grid_size(tiles_m, tiles_n)), dim3(GT_THREADS), GT_LDS_BYTES, st, A, w, w_stride_e, ldw, w_scales, ws_stride_e, ws_r,
-                     w_is_2d, offs, group_expert, num_groups, num_experts, M_total, N, (int)(K / 32), (OutT*)out, ldo, tiles_m, tiles_n);
+  const int max_pass = (int)grouped_max_passes(M_total, num_groups);
+  PassWalk wk{offs, group_expert, num_groups, num_experts, M_total};
+  hipLaunchKernelGGL(grouped_plan_kernel, dim3(1), dim3(PLAN_THREADS), 0, st, wk, tiles_m, plan, max_pass);
+  hipLaunchKernelGGL(kern, dim3((unsigned)grouped_grid_size(max_pass, tiles_n)), dim3(GT_THREADS), GT_LDS_BYTES, st, A, w, w_stride_e, ldw, w_scales, ws_stride_e, ws_r,
+                     w_is_2d, plan, M_total, N, (int)(K / 32), (OutT*)out, ldo, tiles_n);
   return 0;
 }
 
@@ -364,12 +405,16 @@ int launch_dw_tiled(const OperandView& P, const OperandView& Q, int64_t NP, int6
 }  // namespace
 }  // namespace alto
 
-extern "C" int alto_mxfp4_grouped_gemm(const uint8_t* a, int64_t lda, const uint8_t* a_scales, int64_t a_ss_r, int64_t a_ss_k, int a_is_2d,
-                                       const uint8_t* w, int64_t w_stride_e, int64_t ldw,
-                                       const uint8_t* w_scales, int64_t ws_stride_e, int64_t ws_r, int64_t ws_k, int w_is_2d,
-                                       const int32_t* offs, const int32_t* group_expert, int num_groups, int num_experts,
-                                       int64_t M_total, int64_t N, int64_t K, void* out, int out_dtype, int64_t ldo, void* stream) {
-  using namespace alto;
+namespace alto {
+namespace {
+
+// `plan` = device memory for the pass list (plan_bytes of it), needed by the tiled path only
+int grouped_gemm_impl(const uint8_t* a, int64_t lda, const uint8_t* a_scales, int64_t a_ss_r, int64_t a_ss_k, int a_is_2d,
+                      const uint8_t* w, int64_t w_stride_e, int64_t ldw,
+                      const uint8_t* w_scales, int64_t ws_stride_e, int64_t ws_r, int64_t ws_k, int w_is_2d,
+                      const int32_t* offs, const int32_t* group_expert, int num_groups, int num_experts,
+                      int64_t M_total, int64_t N, int64_t K, void* out, int out_dtype, int64_t ldo,
+                      void* plan, int64_t plan_bytes, const char* plan_name, void* stream) {
   ALTO_REQUIRE(a && a_scales && w && w_scales && offs && out, "grouped_gemm: NULL pointer");
   ALTO_REQUIRE(num_groups > 0 && num_groups <= 65536, "grouped_gemm: num_groups (%d) out of range", num_groups);
   ALTO_REQUIRE(group_expert != nullptr || num_groups == num_experts, "grouped_gemm: without group_expert, num_groups must equal num_experts");
@@ -390,16 +435,21 @@ extern "C" int alto_mxfp4_grouped_gemm(const uint8_t* a, int64_t lda, const uint
   const bool tiled = M_total >= 128 && N >= 128 && K >= 512 && a_ss_k == 1 && ws_k == 1 && N % 8 == 0 && ldo % 8 == 0 &&
                      (reinterpret_cast<uintptr_t>(out) & 15) == 0 && M_total * lda < (1ll << 31) && N * ldw < (1ll << 31) &&
                      M_total * a_ss_r < (1ll << 31) && N * ws_r < (1ll << 31) &&
-                     ((M_total + GT_TM - 1) / GT_TM) * ((N + GT_TN - 1) / GT_TN) < (1ll << 28);
+                     grouped_max_passes(M_total, num_groups) * ((N + GT_TN - 1) / GT_TN) < (1ll << 28);
   if (tiled) {
+    const int64_t need = grouped_workspace_bytes(M_total, num_groups);
+    ALTO_REQUIRE(plan != nullptr && plan_bytes >= need && (reinterpret_cast<uintptr_t>(plan) & 15) == 0,
+                 "grouped_gemm: %s of %lld bytes is too small: M_total = %lld with %d groups needs %lld bytes (16-byte aligned)", plan_name,
+                 (long long)plan_bytes, (long long)M_total, num_groups, (long long)need);
     const bool tail = (K / 32) % 16 != 0;
+    int32_t* pl = reinterpret_cast<int32_t*>(plan);
     int rc;
     if (out_dtype == ALTO_DT_BF16)
-      rc = tail ? launch_grouped_tiled<__bf16, true>(A, w, w_stride_e, ldw, w_scales, ws_stride_e, ws_r, w_is_2d, offs, group_expert, num_groups, num_experts, M_total, N, K, out, ldo, st)
-                : launch_grouped_tiled<__bf16, false>(A, w, w_stride_e, ldw, w_scales, ws_stride_e, ws_r, w_is_2d, offs, group_expert, num_groups, num_experts, M_total, N, K, out, ldo, st);
+      rc = tail ? launch_grouped_tiled<__bf16, true>(A, w, w_stride_e, ldw, w_scales, ws_stride_e, ws_r, w_is_2d, offs, group_expert, num_groups, num_experts, M_total, N, K, out, ldo, pl, st)
+                : launch_grouped_tiled<__bf16, false>(A, w, w_stride_e, ldw, w_scales, ws_stride_e, ws_r, w_is_2d, offs, group_expert, num_groups, num_experts, M_total, N, K, out, ldo, pl, st);
     else
-      rc = tail ? launch_grouped_tiled<float, true>(A, w, w_stride_e, ldw, w_scales, ws_stride_e, ws_r, w_is_2d, offs, group_expert, num_groups, num_experts, M_total, N, K, out, ldo, st)
-                : launch_grouped_tiled<float, false>(A, w, w_stride_e, ldw, w_scales, ws_stride_e, ws_r, w_is_2d, offs, group_expert, num_groups, num_experts, M_total, N, K, out, ldo, st);
+      rc = tail ? launch_grouped_tiled<float, true>(A, w, w_stride_e, ldw, w_scales, ws_stride_e, ws_r, w_is_2d, offs, group_expert, num_groups, num_experts, M_total, N, K, out, ldo, pl, st)
+                : launch_grouped_tiled<float, false>(A, w, w_stride_e, ldw, w_scales, ws_stride_e, ws_r, w_is_2d, offs, group_expert, num_groups, num_experts, M_total, N, K, out, ldo, pl, st);
     if (rc != 0) {
       set_error("grouped_gemm: could not reserve %d bytes of LDS", GT_LDS_BYTES);
       return ALTO_MXFP4_ELAUNCH;
@@ -417,6 +467,24 @@ extern "C" int alto_mxfp4_grouped_gemm(const uint8_t* a, int64_t lda, const uint
     hipLaunchKernelGGL(grouped_simple_kernel<float>, grid, dim3(256), 0, st, A, w, w_stride_e, ldw, w_scales, ws_stride_e, ws_r, ws_k, w_is_2d,
                        offs, group_expert, num_groups, num_experts, M_total, N, (int)(K / 32), (float*)out, ldo);
   return check_launch("grouped_gemm");
+}
+
+}  // namespace
+}  // namespace alto
+
+extern "C" int64_t alto_mxfp4_grouped_gemm_workspace_bytes(int64_t M_total, int num_groups) {
+  if (M_total < 0 || num_groups < 0) return 0;
+  return alto::grouped_workspace_bytes(M_total, num_groups);
+}
+
+extern "C" int alto_mxfp4_grouped_gemm(const uint8_t* a, int64_t lda, const uint8_t* a_scales, int64_t a_ss_r, int64_t a_ss_k, int a_is_2d,
+                                       const uint8_t* w, int64_t w_stride_e, int64_t ldw,
+                                       const uint8_t* w_scales, int64_t ws_stride_e, int64_t ws_r, int64_t ws_k, int w_is_2d,
+                                       const int32_t* offs, const int32_t* group_expert, int num_groups, int num_experts,
+                                       int64_t M_total, int64_t N, int64_t K, void* out, int out_dtype, int64_t ldo,
+                                       void* workspace, int64_t workspace_bytes, void* stream) {
+  return alto::grouped_gemm_impl(a, lda, a_scales, a_ss_r, a_ss_k, a_is_2d, w, w_stride_e, ldw, w_scales, ws_stride_e, ws_r, ws_k, w_is_2d, offs, group_expert,
+                                 num_groups, num_experts, M_total, N, K, out, out_dtype, ldo, workspace, workspace_bytes, "the workspace", stream);
 }
 
 extern "C" int alto_mxfp4_grouped_gemm_dw(const uint8_t* go, int64_t ld_go, const uint8_t* go_scales, int64_t gs_r, int64_t gs_k,

@@ -74,11 +74,14 @@ def grouped_forward(a_q, a_s, w_q, w_s, groups: Groups, use_2dblock_x, use_2dblo
     out = torch.empty((a_q.shape[0], N), dtype=output_dtype, device=a_q.device)
     if out.numel() == 0:
         return out
+    # the pass list the kernels exchange (a few KB; torch's caching allocator hands it out without a device call)
+    ws_bytes = rt.lib().alto_mxfp4_grouped_gemm_workspace_bytes(a_q.shape[0], groups.n)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=a_q.device)
     rc = rt.lib().alto_mxfp4_grouped_gemm(
         a_q.data_ptr(), a_q.stride(0), a_s.data_ptr(), a_s.stride(0), a_s.stride(1), int(use_2dblock_x),
         w_q.data_ptr(), w_q.stride(0), w_q.stride(1), w_s.data_ptr(), w_s.stride(0), w_s.stride(1), w_s.stride(2), int(use_2dblock_w),
         groups.offs.data_ptr(), rt.ptr(groups.expert), groups.n, E, a_q.shape[0], N, K, out.data_ptr(), rt.dtype_code(output_dtype), out.stride(0),
-        rt.stream_ptr(a_q.device))
+        ws.data_ptr(), ws_bytes, rt.stream_ptr(a_q.device))
     check(rc, "alto_mxfp4_grouped_gemm")
     return out
 

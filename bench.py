@@ -279,6 +279,56 @@ class GroupedGemm(Workload):
         return run, 2.0 * rows * self.N * self.K, f"{rows} rows of the largest expert, dequantize + fp32 matmul"
 
 
+class GroupedGemmDx(GroupedGemm):
+    """Config 5 backward, input gradient: dX [65536, 2880] = dY [65536, 5760] . W[e] (reduction over N = 5760; the weights
+    are the N-packed copy of their 2D-block quantisation), same ragged offsets."""
+    name = "cfg5_grouped_dx[65536x2880x5760,E=32]"
+
+    def setup(self, dev, gen):
+        import torch
+        super().setup(dev, gen)
+        from alto_amd.mxfp4.quantization import _prep, _quantize_call
+        go = _laplace((self.rows, self.N), 1e-3, dev, gen)
+        gq, gs, _, _ = _quantize_call(_prep(go), True, False, False, False, None, None, 0, False, True)
+        del go
+        self.aq, self.as_ = gq[0], gs[0]
+        w = (torch.randn(self.E, self.N, self.K, device=dev, generator=gen) * 0.02).bfloat16()
+        _, _, self.wq, self.ws = _quantize_call(_prep(w), True, True, True, False, None, None, 0, False, True)   # [E, K, N/2], [E, K/32, N/32]
+        del w
+
+    def cpu_sample(self):
+        raise NotImplementedError("reported beside the forward workload, which carries the CPU leg")
+
+
+class GroupedGemmDw(GroupedGemm):
+    """Config 5 backward, weight gradient: dW[e] [5760, 2880] = sum over the tokens of expert e of dY^T X, token-packed
+    operands, offsets rounded down to 32 rows (one MX block along the tokens belongs to one expert)."""
+    name = "cfg5_grouped_dw[32x5760x2880 over 65536 tokens]"
+
+    def setup(self, dev, gen):
+        import torch
+        super().setup(dev, gen)
+        from alto_amd.mxfp4.quantization import _prep, _quantize_call
+        offs = (self.groups.offs // 32 * 32).to(torch.int32)
+        offs[-1] = self.rows
+        self.groups = self.G.groups_from_offsets(offs)
+        go = _laplace((self.rows, self.N), 1e-3, dev, gen)
+        _, _, gq, gs = _quantize_call(_prep(go), False, True, False, False, None, None, 0, False, True)
+        del go
+        a = torch.randn(self.rows, self.K, device=dev, generator=gen).bfloat16()
+        _, _, xq, xs = _quantize_call(_prep(a), False, True, False, False, None, None, 0, False, True)
+        del a
+        self.gq, self.gs, self.xq, self.xs = gq[0], gs[0], xq[0], xs[0]     # [N, M/2], [N, M/32], [K, M/2], [K, M/32]
+        self.aq = self.as_ = self.wq = self.ws = None
+
+    def step(self):
+        import torch
+        return self.G.grouped_dw(self.gq, self.gs, self.xq, self.xs, self.groups, self.E, torch.bfloat16)
+
+    def cpu_sample(self):
+        raise NotImplementedError("reported beside the forward workload, which carries the CPU leg")
+
+
 class AttentionFwd(Workload):
     """MXFP4 flash-attention forward on pre-quantised Q, K, V: the largest case of the reference's own test list
     (tests/unittest/mxfp4/test_mxfp_attention.py:64: batch 4, 2048 tokens, 64 query / 8 KV heads, head dim 128, causal)."""
@@ -422,6 +472,8 @@ def make_workloads():
         "cfg4_dgrad": Gemm("cfg4_dgrad_gemm[8192x14336x4096]", 8192, 14336, 4096, False, True, "grad", "weight"),
         "cfg4_wgrad": Gemm("cfg4_wgrad_gemm[4096x14336x8192]", 4096, 14336, 8192, False, False, "grad", "act"),
         "cfg5_grouped": GroupedGemm(),
+        "cfg5_grouped_dx": GroupedGemmDx(),
+        "cfg5_grouped_dw": GroupedGemmDw(),
         "attn_fwd": AttentionFwd(),
         "linear_step": LinearStep(False),
         "linear_step_cached": LinearStep(True),

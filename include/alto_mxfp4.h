@@ -188,12 +188,20 @@ int alto_mxfp4_gemm(const uint8_t* a, int64_t lda, const uint8_t* a_scales, int6
  * reference's per-row expert index with 128-row groups maps to offs = 128 * g, group_expert = index[128 * g].
  * Groups need no alignment for 1D activation scales; rows outside every group (and groups whose expert id is
  * out of range) are written with zeros (the reference allocates zeros, cg_forward.py:260).
+ * `workspace`: DEVICE memory of at least alto_mxfp4_grouped_gemm_workspace_bytes(M_total, num_groups) bytes, 16-byte
+ * aligned, owned by the caller.  A one-workgroup kernel first writes the list of (256-row band, expert) passes there
+ * (the reference scans the groups inside every program instead, cg_forward.py:120-140), the GEMM kernel reads it.  Its
+ * contents need not be initialised and mean nothing after the call; two calls that overlap in time need two workspaces.
  */
 int alto_mxfp4_grouped_gemm(const uint8_t* a, int64_t lda, const uint8_t* a_scales, int64_t a_ss_r, int64_t a_ss_k, int a_is_2d,
                             const uint8_t* w, int64_t w_stride_e, int64_t ldw,
                             const uint8_t* w_scales, int64_t ws_stride_e, int64_t ws_r, int64_t ws_k, int w_is_2d,
                             const int32_t* offs, const int32_t* group_expert, int num_groups, int num_experts,
-                            int64_t M_total, int64_t N, int64_t K, void* out, int out_dtype, int64_t ldo, void* stream);
+                            int64_t M_total, int64_t N, int64_t K, void* out, int out_dtype, int64_t ldo,
+                            void* workspace, int64_t workspace_bytes, void* stream);
+
+/* Bytes of workspace alto_mxfp4_grouped_gemm needs for M_total rows in num_groups groups (a bound, not a measurement). */
+int64_t alto_mxfp4_grouped_gemm_workspace_bytes(int64_t M_total, int num_groups);
 
 /*
  * Grouped weight gradient: dW[e][N][K] = sum over the rows r of every group of expert e of dY[r][:]^T . X[r][:],

@@ -258,9 +258,11 @@ def test_cfg5_grouped_forward_full_size(m):
     _check_grouped_bands(out, aq, as_, wq, ws, offs_cpu, "cfg5 grouped forward")
     # NaN sentinel through the C ABI
     out2 = _nan_like((rows, N5), torch.bfloat16)
+    wsp = torch.empty(rt.lib().alto_mxfp4_grouped_gemm_workspace_bytes(rows, E5), dtype=torch.uint8, device=DEV)
     rc = rt.lib().alto_mxfp4_grouped_gemm(aq.data_ptr(), aq.stride(0), as_.data_ptr(), as_.stride(0), as_.stride(1), 0,
                                           wq.data_ptr(), wq.stride(0), wq.stride(1), ws.data_ptr(), ws.stride(0), ws.stride(1), ws.stride(2), 1,
-                                          offs.data_ptr(), None, E5, E5, rows, N5, K5, out2.data_ptr(), rt.DT_BF16, out2.stride(0), rt.stream_ptr(out2.device))
+                                          offs.data_ptr(), None, E5, E5, rows, N5, K5, out2.data_ptr(), rt.DT_BF16, out2.stride(0),
+                                          wsp.data_ptr(), wsp.numel(), rt.stream_ptr(out2.device))
     assert rc == 0
     assert not bool(torch.isnan(out2).any()), "cfg5 grouped forward: an output tile was not written"
     assert torch.equal(out2.view(torch.int16), out.view(torch.int16))
