@@ -44,6 +44,9 @@ SIGNATURES = {
     "alto_mxfp4_grouped_gemm": (c_int, [c_vp, c_i64, c_vp, c_i64, c_i64, c_int,
                                         c_vp, c_i64, c_i64, c_vp, c_i64, c_i64, c_i64, c_int,
                                         c_vp, c_vp, c_int, c_int, c_i64, c_i64, c_i64, c_vp, c_int, c_i64, c_vp, c_i64, c_vp]),
+    "alto_mxfp4_grouped_gemm_noalloc": (c_int, [c_vp, c_i64, c_vp, c_i64, c_i64, c_int,
+                                                c_vp, c_i64, c_i64, c_vp, c_i64, c_i64, c_i64, c_int,
+                                                c_vp, c_vp, c_int, c_int, c_i64, c_i64, c_i64, c_vp, c_int, c_i64, c_vp]),
     "alto_mxfp4_grouped_gemm_workspace_bytes": (c_i64, [c_i64, c_int]),
     "alto_mxfp4_grouped_gemm_dw": (c_int, [c_vp, c_i64, c_vp, c_i64, c_i64,
                                            c_vp, c_i64, c_vp, c_i64, c_i64,

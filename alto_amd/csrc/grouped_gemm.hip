@@ -5,6 +5,12 @@
 #include "gemm_simple.h"
 #include "gemm_tile.h"
 
+// Pass-list memory of alto_mxfp4_grouped_gemm_noalloc: one array per GPU, part of the loaded code object (each GPU the
+// library runs on holds its own copy at its own address until the process ends).  In host code the name is only a
+// handle for hipGetSymbolAddress; kernels get the address that call returns.
+constexpr int64_t ALTO_NOALLOC_SCRATCH_BYTES = 1 << 20;
+static __device__ __align__(256) unsigned char scratch[ALTO_NOALLOC_SCRATCH_BYTES];
+
 namespace alto {
 namespace {
 
@@ -485,6 +491,53 @@ extern "C" int alto_mxfp4_grouped_gemm(const uint8_t* a, int64_t lda, const uint
                                        void* workspace, int64_t workspace_bytes, void* stream) {
   return alto::grouped_gemm_impl(a, lda, a_scales, a_ss_r, a_ss_k, a_is_2d, w, w_stride_e, ldw, w_scales, ws_stride_e, ws_r, ws_k, w_is_2d, offs, group_expert,
                                  num_groups, num_experts, M_total, N, K, out, out_dtype, ldo, workspace, workspace_bytes, "the workspace", stream);
+}
+
+namespace alto {
+namespace {
+constexpr int MAX_DEVICES = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[MAX_DEVICES] = {};
+
+// device address of `scratch` on the current GPU, looked up once per device
+int scratch_of_current_device(void** out) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) {
+    set_error("grouped_gemm_noalloc: no current HIP device (or device index beyond %d)", MAX_DEVICES - 1);
+    return ALTO_MXFP4_ELAUNCH;
+  }
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* p = nullptr;
+    const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || p == nullptr) {
+      set_error("grouped_gemm_noalloc: hipGetSymbolAddress failed on device %d: %s", dev, hipGetErrorString(e));
+      return ALTO_MXFP4_ELAUNCH;
+    }
+    g_scratch_ptr[dev] = p;
+  }
+  *out = g_scratch_ptr[dev];
+  return ALTO_MXFP4_OK;
+}
+}  // namespace
+}  // namespace alto
+
+extern "C" int alto_mxfp4_grouped_gemm_noalloc(const uint8_t* a, int64_t lda, const uint8_t* a_scales, int64_t a_ss_r, int64_t a_ss_k, int a_is_2d,
+                                               const uint8_t* w, int64_t w_stride_e, int64_t ldw,
+                                               const uint8_t* w_scales, int64_t ws_stride_e, int64_t ws_r, int64_t ws_k, int w_is_2d,
+                                               const int32_t* offs, const int32_t* group_expert, int num_groups, int num_experts,
+                                               int64_t M_total, int64_t N, int64_t K, void* out, int out_dtype, int64_t ldo, void* stream) {
+  using namespace alto;
+  ALTO_REQUIRE(M_total >= 0 && num_groups > 0, "grouped_gemm_noalloc: bad sizes");
+  ALTO_REQUIRE(grouped_workspace_bytes(M_total, num_groups) <= ALTO_NOALLOC_SCRATCH_BYTES,
+               "grouped_gemm_noalloc: M_total = %lld rows in %d groups need a pass list of %lld bytes, more than the built-in %lld: use "
+               "alto_mxfp4_grouped_gemm with a workspace", (long long)M_total, num_groups, (long long)grouped_workspace_bytes(M_total, num_groups),
+               (long long)ALTO_NOALLOC_SCRATCH_BYTES);
+  void* plan = nullptr;
+  const int rc = scratch_of_current_device(&plan);
+  if (rc != ALTO_MXFP4_OK) return rc;
+  return grouped_gemm_impl(a, lda, a_scales, a_ss_r, a_ss_k, a_is_2d, w, w_stride_e, ldw, w_scales, ws_stride_e, ws_r, ws_k, w_is_2d, offs, group_expert,
+                           num_groups, num_experts, M_total, N, K, out, out_dtype, ldo, plan, ALTO_NOALLOC_SCRATCH_BYTES, "the built-in scratch array", stream);
 }
 
 extern "C" int alto_mxfp4_grouped_gemm_dw(const uint8_t* go, int64_t ld_go, const uint8_t* go_scales, int64_t gs_r, int64_t gs_k,

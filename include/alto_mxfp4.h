@@ -200,6 +200,21 @@ int alto_mxfp4_grouped_gemm(const uint8_t* a, int64_t lda, const uint8_t* a_scal
                             int64_t M_total, int64_t N, int64_t K, void* out, int out_dtype, int64_t ldo,
                             void* workspace, int64_t workspace_bytes, void* stream);
 
+/*
+ * alto_mxfp4_grouped_gemm without the workspace argument, for callers that cannot allocate device memory (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  The pass list
+ * lives in a 1 MiB array that is part of the library's device code (one copy per GPU, held until the process ends), so
+ * the call allocates nothing; it serves M_total / 256 + num_groups + 2 <= 65535 and rejects larger problems with
+ * ALTO_MXFP4_EINVAL.  Every call on a GPU shares that GPU's array: calls that overlap in time on one GPU (two streams,
+ * two host threads) race on it and must use alto_mxfp4_grouped_gemm with separate workspaces instead.  Same results as
+ * alto_mxfp4_grouped_gemm, bit for bit.
+ */
+int alto_mxfp4_grouped_gemm_noalloc(const uint8_t* a, int64_t lda, const uint8_t* a_scales, int64_t a_ss_r, int64_t a_ss_k, int a_is_2d,
+                                    const uint8_t* w, int64_t w_stride_e, int64_t ldw,
+                                    const uint8_t* w_scales, int64_t ws_stride_e, int64_t ws_r, int64_t ws_k, int w_is_2d,
+                                    const int32_t* offs, const int32_t* group_expert, int num_groups, int num_experts,
+                                    int64_t M_total, int64_t N, int64_t K, void* out, int out_dtype, int64_t ldo, void* stream);
+
 /* Bytes of workspace alto_mxfp4_grouped_gemm needs for M_total rows in num_groups groups (a bound, not a measurement). */
 int64_t alto_mxfp4_grouped_gemm_workspace_bytes(int64_t M_total, int num_groups);
 
