@@ -284,7 +284,7 @@ __global__ __launch_bounds__(GT_THREADS) void grouped_dw_tiled_kernel(OperandVie
   TileAcc acc;
   gemm_tile_zero(acc);
   const int64_t p_bytes = (NP - 1) * P.ld + M_total / 2, q_bytes = (NQ - 1) * Q.ld + M_total / 2;
-  const int64_t ps_bytes = (NP - 1) * P.ss_r + M_total / 32, qs_bytes = (NQ - 1) * Q.ss_r + M_total / 32;
+  const int64_t ps_bytes = ((P.is_2d ? NP / 32 : NP) - 1) * P.ss_r + M_total / 32, qs_bytes = ((Q.is_2d ? NQ / 32 : NQ) - 1) * Q.ss_r + M_total / 32;
   // Boundaries of this expert's token runs; one that is not a multiple of 32 would share an MX block along the token dim
   // with another expert: the tile is then poisoned with NaN instead of being silently wrong.
   int bad = 0;
@@ -540,8 +540,8 @@ extern "C" int alto_mxfp4_grouped_gemm_noalloc(const uint8_t* a, int64_t lda, co
                            num_groups, num_experts, M_total, N, K, out, out_dtype, ldo, plan, ALTO_NOALLOC_SCRATCH_BYTES, "the built-in scratch array", stream);
 }
 
-extern "C" int alto_mxfp4_grouped_gemm_dw(const uint8_t* go, int64_t ld_go, const uint8_t* go_scales, int64_t gs_r, int64_t gs_k,
-                                          const uint8_t* x, int64_t ld_xq, const uint8_t* x_scales, int64_t xs_r, int64_t xs_k,
+extern "C" int alto_mxfp4_grouped_gemm_dw(const uint8_t* go, int64_t ld_go, const uint8_t* go_scales, int64_t gs_r, int64_t gs_k, int go_is_2d,
+                                          const uint8_t* x, int64_t ld_xq, const uint8_t* x_scales, int64_t xs_r, int64_t xs_k, int x_is_2d,
                                           const int32_t* offs, const int32_t* group_expert, int num_groups, int num_experts,
                                           int64_t M_total, int64_t N, int64_t K, void* dw, int dw_dtype, int64_t dw_stride_e, int64_t dw_stride_n, int64_t dw_stride_k,
                                           float out_scale, void* stream) {
@@ -557,8 +557,9 @@ extern "C" int alto_mxfp4_grouped_gemm_dw(const uint8_t* go, int64_t ld_go, cons
   ALTO_REQUIRE(dw_dtype == ALTO_DT_BF16 || dw_dtype == ALTO_DT_F32, "grouped_gemm_dw: bad dw_dtype %d", dw_dtype);
   if (N == 0 || K == 0) return ALTO_MXFP4_OK;
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-  OperandView GO{go, ld_go, go_scales, gs_r, gs_k, 0};
-  OperandView X{x, ld_xq, x_scales, xs_r, xs_k, 0};
+  ALTO_REQUIRE((!go_is_2d || N % 32 == 0) && (!x_is_2d || K % 32 == 0), "grouped_gemm_dw: 2D scales need N (%lld) / K (%lld) %% 32 == 0", (long long)N, (long long)K);
+  OperandView GO{go, ld_go, go_scales, gs_r, gs_k, go_is_2d ? 1 : 0};
+  OperandView X{x, ld_xq, x_scales, xs_r, xs_k, x_is_2d ? 1 : 0};
   {
     // 256x256 tiles: the output's unit-stride dim becomes the GEMM's column dim, so the operands swap roles for dW stored [E, K, N]
     const bool n_major = dw_stride_k == 1;   // dW[e] is [N][K]

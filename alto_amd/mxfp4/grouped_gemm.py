@@ -6,8 +6,9 @@ Mirrors ``alto/kernels/fp4/mxfp4/mxfp_grouped_gemm``: ``mxfp4_grouped_gemm_forwa
 
 The kernels consume expert row ranges (``offs``: E+1 int32 offsets on the device) instead of a per-row expert
 index; the index form of the reference API is converted on the device without a host sync.  Groups may be ragged
-for 1D activation scales; the reference's 128-row alignment is still required by the weight-gradient kernel at a
-granularity of 32 rows (one MX block along the token dim may not straddle two experts).
+for 1D activation scales; the weight gradient (and 2D activation blocks) need every boundary between two experts at a
+multiple of 32 rows, since one MX block along the token dim cannot be split between experts: the kernel checks this on
+the device and writes NaN into the weight gradient of an expert with a misaligned boundary (the reference asks for 128).
 """
 from __future__ import annotations
 
@@ -121,8 +122,9 @@ def mxfp4_grouped_gemm_backward_inputs(grad_output, expert_weights, expert_indic
     return grouped_forward(grad_output, go_scales, w_can, s_can, groups_from_indices(expert_indices), use_2dblock_x, use_2dblock_w, output_dtype)
 
 
-def grouped_dw(go_qm, go_sm, x_qm, x_sm, groups: Groups, num_experts, output_dtype, trans_weights=True, out_scale=1.0):
-    """dW[e] = sum_{rows of e} dY^T X with token-packed operands: go_qm [N, M/2], x_qm [K, M/2] (unit stride along tokens)."""
+def grouped_dw(go_qm, go_sm, x_qm, x_sm, groups: Groups, num_experts, output_dtype, trans_weights=True, out_scale=1.0, is_2d=False):
+    """dW[e] = sum_{rows of e} dY^T X with token-packed operands: go_qm [N, M/2], x_qm [K, M/2] (unit stride along tokens),
+    scales [N, M/32] / [K, M/32], or with ``is_2d`` one scale per 32 x 32 block: [N/32, M/32] / [K/32, M/32]."""
     N, K = go_qm.shape[0], x_qm.shape[0]
     M_total = go_qm.shape[1] * 2
     assert x_qm.shape[1] * 2 == M_total
@@ -130,44 +132,56 @@ def grouped_dw(go_qm, go_sm, x_qm, x_sm, groups: Groups, num_experts, output_dty
         go_qm = go_qm.contiguous()
     if x_qm.stride(1) != 1 or x_qm.stride(0) % 16:
         x_qm = x_qm.contiguous()
+    if go_sm.stride(1) != 1:   # the tiled kernel reads scale rows with unit stride along the tokens
+        go_sm = go_sm.contiguous()
+    if x_sm.stride(1) != 1:
+        x_sm = x_sm.contiguous()
     shape = (num_experts, N, K) if trans_weights else (num_experts, K, N)
     dw = torch.empty(shape, dtype=output_dtype, device=go_qm.device)
     s_e, s_n, s_k = (dw.stride(0), dw.stride(1), dw.stride(2)) if trans_weights else (dw.stride(0), dw.stride(2), dw.stride(1))
     rc = rt.lib().alto_mxfp4_grouped_gemm_dw(
-        go_qm.data_ptr(), go_qm.stride(0), go_sm.data_ptr(), go_sm.stride(0), go_sm.stride(1),
-        x_qm.data_ptr(), x_qm.stride(0), x_sm.data_ptr(), x_sm.stride(0), x_sm.stride(1),
+        go_qm.data_ptr(), go_qm.stride(0), go_sm.data_ptr(), go_sm.stride(0), go_sm.stride(1), int(is_2d),
+        x_qm.data_ptr(), x_qm.stride(0), x_sm.data_ptr(), x_sm.stride(0), x_sm.stride(1), int(is_2d),
         groups.offs.data_ptr(), rt.ptr(groups.expert), groups.n, num_experts, M_total, N, K, dw.data_ptr(), rt.dtype_code(output_dtype), s_e, s_n, s_k,
         float(out_scale), rt.stream_ptr(go_qm.device))
     check(rc, "alto_mxfp4_grouped_gemm_dw")
     return dw
 
 
+def _token_packed(codes: torch.Tensor, k_pack: bool) -> torch.Tensor:
+    """An operand of the weight gradient as [features, M/2] codes with unit stride along the tokens: a transposed view
+    when it arrives packed along the tokens ([M/2, features], ``k_pack``), a nibble transpose when it arrives packed along
+    the features ([M, features/2])."""
+    return codes.transpose(0, 1) if k_pack else transpose_codes(codes)
+
+
 def mxfp4_grouped_gemm_backward_weights(grad_output, inputs, expert_indices, num_experts, go_scales, input_scales,
                                         trans_weights=True, use_2dblock_go=False, use_2dblock_x=True, k_pack_go=True,
                                         k_pack_x=True, output_dtype=torch.bfloat16):
-    """cg_backward.py:398-497.  With ``k_pack_*`` the operands are [M/2, N] / [M/2, K] views packed along tokens."""
+    """cg_backward.py:398-497.  With ``k_pack_*`` the operands are [M/2, N] / [M/2, K] packed along the tokens, otherwise
+    [M, N/2] / [M, K/2]; the scales are [M/32, N] / [M/32, K] (1D along the tokens) or [M/32, N/32] / [M/32, K/32] (2D)."""
     assert expert_indices.is_contiguous(), "Expert indices tensor must be contiguous"
     M_total = expert_indices.shape[0]
     torch._check(M_total > 0)
     torch._check(M_total % ALIGN_SIZE_M == 0)
-    if use_2dblock_go or use_2dblock_x or not (k_pack_go and k_pack_x):
-        raise NotImplementedError("grouped weight gradient: only token-packed 1D-scaled operands are implemented")
+    assert bool(use_2dblock_go) == bool(use_2dblock_x), "the two operands of the weight gradient share their block layout (cg_backward.py:880-893)"
     rt.require_gpu(grad_output, inputs, expert_indices, go_scales, input_scales)
-    return grouped_dw(grad_output.transpose(0, 1), go_scales.transpose(0, 1), inputs.transpose(0, 1), input_scales.transpose(0, 1),
-                      groups_from_indices(expert_indices), num_experts, output_dtype, trans_weights)
+    return grouped_dw(_token_packed(grad_output, k_pack_go), go_scales.transpose(0, 1), _token_packed(inputs, k_pack_x), input_scales.transpose(0, 1),
+                      groups_from_indices(expert_indices), num_experts, output_dtype, trans_weights, is_2d=bool(use_2dblock_x))
 
 
 @torch.compiler.allow_in_graph
 class MXFP4GroupedGEMM(torch.autograd.Function):
-    """Grouped GEMM with full backward (cg_backward.py:599-930), recipe branch 1D activations / 2D weights."""
+    """Grouped GEMM with full backward (cg_backward.py:599-930), every block-layout combination of the reference:
+    activations and gradients with 1D blocks (then the weight-gradient operands are separate token-axis quantisations, with
+    the Hadamard transform and the clip mode) or 2D blocks (one quantisation serves all three GEMMs); weights with 2D
+    blocks (one quantisation, both packings) or 1D blocks (one quantisation along K for the forward, one along N for dX)."""
 
     @staticmethod
     def forward(ctx, inputs, expert_weights, expert_indices, trans_weights=True, use_2dblock_x=False, use_2dblock_w=True,
                 use_sr_grad=False, use_dge=False, clip_mode="none", use_macro_block_scaling=False,
                 hadamard_transform: Optional[HadamardTransform] = None, use_uos: bool = False, offsets: Optional[torch.Tensor] = None):
         assert not use_macro_block_scaling, "Macro block scaling is not supported in real MXFP4 kernels"
-        if use_2dblock_x or not use_2dblock_w:
-            raise NotImplementedError("grouped MXFP4 GEMM: only use_2dblock_x=False, use_2dblock_w=True is implemented")
         original_dtype = inputs.dtype
         expert_weights = unwrap_weight_wrapper(expert_weights)
         E = expert_weights.shape[0]
@@ -181,18 +195,23 @@ class MXFP4GroupedGEMM(torch.autograd.Function):
             groups = groups_from_offsets(offsets)
         torch._check(M_buf % 32 == 0)
         x = inputs if inputs.is_contiguous() else inputs.contiguous()
-        a_q, a_s, a_qm, a_sm = quantize_rowcol(x, False, hadamard=hadamard_transform, clip_mode=clip_mode, use_uos=use_uos, pad_codes=True)
-        # weights: one pass gives the K-packed codes (forward) and the N-packed codes (dX)
+        if use_2dblock_x:   # one 2D-block quantisation, both packings: K-packed for the forward, token-packed for dW
+            a_q, a_s, a_qm, a_sm = quantize_rowcol(x, True, use_uos=use_uos, pad_codes=True)
+        else:               # row copy for the forward; Hadamard + clip on the token-axis copy saved for dW
+            a_q, a_s, a_qm, a_sm = quantize_rowcol(x, False, hadamard=hadamard_transform, clip_mode=clip_mode, use_uos=use_uos, pad_codes=True)
+        # weights: codes packed along K [E, N, K/2] for the forward, packed along N [E, K, N/2] for dX
         w = expert_weights if trans_weights else expert_weights.transpose(1, 2)   # logical [E, N, K]
         if w.stride(2) == 1:
-            wq_nk, ws_nk, wq_kn, ws_kn = _quantize_experts(expert_weights, w, use_uos)   # [E,N,K/2], [E,N/32,K/32], [E,K,N/2], [E,K/32,N/32]
+            wq_nk, ws_nk, wq_kn, ws_kn = _quantize_experts(expert_weights, w, use_2dblock_w, use_uos)
         else:                                                                     # stored [E, K, N]: same pass, roles swapped
-            wq_kn, ws_kn, wq_nk, ws_nk = _quantize_experts(expert_weights, w.transpose(1, 2), use_uos)
-        out = grouped_forward(a_q, a_s, wq_nk, ws_nk, groups, False, True, original_dtype)
+            wq_kn, ws_kn, wq_nk, ws_nk = _quantize_experts(expert_weights, w.transpose(1, 2), use_2dblock_w, use_uos)
+        out = grouped_forward(a_q, a_s, wq_nk, ws_nk, groups, use_2dblock_x, use_2dblock_w, original_dtype)
         ctx.save_for_backward(a_qm, a_sm, wq_kn, ws_kn, groups.offs, groups.expert)
         ctx.num_groups = groups.n
         ctx.trans_weights = trans_weights
         ctx.original_dtype = original_dtype
+        ctx.use_2dblock_x = bool(use_2dblock_x)
+        ctx.use_2dblock_w = bool(use_2dblock_w)
         ctx.use_sr_grad = use_sr_grad
         ctx.hadamard_transform = hadamard_transform
         ctx.clip_mode = clip_mode
@@ -209,22 +228,27 @@ class MXFP4GroupedGEMM(torch.autograd.Function):
         sr = bool(ctx.use_sr_grad)
         # random words: made inside the quantizer (Philox) unless a source of explicit words is installed
         rand = rt.draw_rand_bits(go.shape, go.device) if (sr and not rt.philox_in_kernel()) else None
-        go_q, go_s, go_qm, go_sm = quantize_rowcol(go, False, use_sr=sr, rand_bits=rand, hadamard=ctx.hadamard_transform,
-                                                   clip_mode=ctx.clip_mode, use_uos=ctx.use_uos, pad_codes=True)
-        grad_inputs = grouped_forward(go_q, go_s, wq_kn, ws_kn, groups, False, True, ctx.original_dtype)
+        if ctx.use_2dblock_x:
+            go_q, go_s, go_qm, go_sm = quantize_rowcol(go, True, use_sr=sr, rand_bits=rand, use_uos=ctx.use_uos, pad_codes=True)
+        else:
+            go_q, go_s, go_qm, go_sm = quantize_rowcol(go, False, use_sr=sr, rand_bits=rand, hadamard=ctx.hadamard_transform,
+                                                       clip_mode=ctx.clip_mode, use_uos=ctx.use_uos, pad_codes=True)
+        grad_inputs = grouped_forward(go_q, go_s, wq_kn, ws_kn, groups, ctx.use_2dblock_x, ctx.use_2dblock_w, ctx.original_dtype)
         grad_weights = grouped_dw(go_qm.transpose(0, 1), go_sm.transpose(0, 1), a_qm.transpose(0, 1), a_sm.transpose(0, 1),
                                   groups, ctx.num_experts, ctx.original_dtype, ctx.trans_weights,
-                                  _wgrad_scale(ctx.clip_mode, ctx.use_dge))
+                                  _wgrad_scale(ctx.clip_mode, ctx.use_dge), is_2d=ctx.use_2dblock_x)
         return (grad_inputs, grad_weights) + (None,) * 11
 
 
-def _quantize_experts(owner: torch.Tensor, w: torch.Tensor, use_uos: bool):
-    """w [E, R, C] (unit stride along C; ``owner`` or a transposed view of it) -> codes packed along C [E,R,C/2], 2D scales
-    [E,R/32,C/32], codes packed along R [E,C,R/2] and the same scales stored transposed [E,C/32,R/32] (each operand of a
-    GEMM wants unit stride along its K).  The cache entry belongs to ``owner``, the tensor object the caller keeps."""
+def _quantize_experts(owner: torch.Tensor, w: torch.Tensor, is_2d: bool, use_uos: bool):
+    """w [E, R, C] (unit stride along C; ``owner`` or a transposed view of it) -> codes packed along C [E,R,C/2] with
+    their scales, and codes packed along R [E,C,R/2] with theirs (each operand of a GEMM wants unit stride along its
+    reduction dim).  2D blocks: one quantisation, scales [E,R/32,C/32] and the same values stored transposed
+    [E,C/32,R/32].  1D blocks: two quantisations (blocks along C: scales [E,R,C/32]; blocks along R: [E,C,R/32]), still one
+    pass over the weights.  The cache entry belongs to ``owner``, the tensor object the caller keeps."""
     from .quantization import _prep, _quantize_call
-    return cached_weight_quantisation(owner, ("experts2d", bool(use_uos), tuple(w.shape), tuple(w.stride())),
-                                      lambda: _quantize_call(_prep(w), True, True, True, False, None, None, 0, use_uos, True))
+    return cached_weight_quantisation(owner, ("experts", bool(is_2d), bool(use_uos), tuple(w.shape), tuple(w.stride())),
+                                      lambda: _quantize_call(_prep(w), True, True, bool(is_2d), False, None, None, 0, use_uos, True))
 
 
 def mxfp4_grouped_gemm(inputs, expert_weights, expert_indices, *, trans_weights=True, use_2dblock_x=False, use_2dblock_w=True,

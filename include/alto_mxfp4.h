@@ -221,7 +221,8 @@ int64_t alto_mxfp4_grouped_gemm_workspace_bytes(int64_t M_total, int num_groups)
 /*
  * Grouped weight gradient: dW[e][N][K] = sum over the rows r of every group of expert e of dY[r][:]^T . X[r][:],
  * operands packed along the token dim:  go [N][M_total/2], x [K][M_total/2] with
- * scales [N][M_total/32], [K][M_total/32] (1D along tokens; strides given).
+ * scales [N][M_total/32], [K][M_total/32] (1D along tokens; strides given), or with go_is_2d / x_is_2d one scale per
+ * 32 x 32 block: [N/32][M_total/32], [K/32][M_total/32] (the use_2dblock_go / use_2dblock_x operands of cg_backward.py:398-497).
  * Replaces _kernel_mxfp4_grouped_gemm_backward_dw (cg_backward.py:213-395); with group_expert == NULL the
  * expert's row range comes from offs directly instead of a scan over all groups.  Every boundary between the
  * token ranges of two experts must be a multiple of 32 (the reference requires 128, cg_backward.py:443-447): an MX
@@ -230,8 +231,8 @@ int64_t alto_mxfp4_grouped_gemm_workspace_bytes(int64_t M_total, int num_groups)
  * dW of experts with no tokens is written with zeros.  Element (e, n, k) lands at
  * dw[e * dw_stride_e + n * dw_stride_n + k * dw_stride_k].
  */
-int alto_mxfp4_grouped_gemm_dw(const uint8_t* go, int64_t ld_go, const uint8_t* go_scales, int64_t gs_r, int64_t gs_k,
-                               const uint8_t* x, int64_t ld_xq, const uint8_t* x_scales, int64_t xs_r, int64_t xs_k,
+int alto_mxfp4_grouped_gemm_dw(const uint8_t* go, int64_t ld_go, const uint8_t* go_scales, int64_t gs_r, int64_t gs_k, int go_is_2d,
+                               const uint8_t* x, int64_t ld_xq, const uint8_t* x_scales, int64_t xs_r, int64_t xs_k, int x_is_2d,
                                const int32_t* offs, const int32_t* group_expert, int num_groups, int num_experts,
                                int64_t M_total, int64_t N, int64_t K,
                                void* dw, int dw_dtype, int64_t dw_stride_e, int64_t dw_stride_n, int64_t dw_stride_k,

@@ -438,37 +438,37 @@ def rel_frobenius(got: torch.Tensor, ref: torch.Tensor) -> float:
 
 
 # --------------------------------------------------------------------------- linear (Q8)
-def linear_forward_ref(x, w, use_2dblock_x=False, use_2dblock_w=True, hadamard=None, clip_mode="none", dtype=torch.float64):
+def linear_forward_ref(x, w, use_2dblock_x=False, use_2dblock_w=True, hadamard=None, clip_mode="none", dtype=torch.float64, use_uos=False):
     """Forward of MXFP4LinearFunction (mxfp_linear.py:265-422) on its dequantize-and-matmul branch.
 
     Returns (y, saved) where saved holds the operands backward needs:
     the token-axis (axis 0) quantisation of H.x and the weight codes/scales.
     """
     x2 = x.reshape(-1, x.shape[-1])
-    xq, xs = quantize(x2, axis=-1, is_2d_block=use_2dblock_x)
-    wq, ws = quantize(w, axis=-1, is_2d_block=use_2dblock_w)
+    xq, xs = quantize(x2, axis=-1, is_2d_block=use_2dblock_x, use_uos=use_uos)
+    wq, ws = quantize(w, axis=-1, is_2d_block=use_2dblock_w, use_uos=use_uos)
     y = gemm_ref(xq, xs, wq, ws, use_2dblock_x, use_2dblock_w, trans_b=True, dtype=dtype)
     saved = {}
     if not use_2dblock_w:
-        wq, ws = quantize(w, axis=0, is_2d_block=False)
+        wq, ws = quantize(w, axis=0, is_2d_block=False, use_uos=use_uos)
     if not use_2dblock_x:
         xh = rht_left(x2, *hadamard) if hadamard is not None else x2
-        xq, xs = quantize(xh, axis=0, is_2d_block=False, clip_mode=clip_mode)
+        xq, xs = quantize(xh, axis=0, is_2d_block=False, clip_mode=clip_mode, use_uos=use_uos)
     saved.update(x_q=xq, x_s=xs, w_q=wq, w_s=ws)
     return y, saved
 
 
 def linear_backward_ref(grad_out, saved, use_2dblock_x=False, use_2dblock_w=True, use_sr_grad=False, rand_bits=None,
-                        hadamard=None, clip_mode="none", dtype=torch.float64):
+                        hadamard=None, clip_mode="none", dtype=torch.float64, use_uos=False):
     """Backward of MXFP4LinearFunction (mxfp_linear.py:424-570): returns (dX, dW) in ``dtype``."""
     g2 = grad_out.reshape(-1, grad_out.shape[-1])
     if use_2dblock_x:
-        gq, gs = quantize(g2, axis=-1, is_2d_block=True, use_sr=use_sr_grad, rand_bits=rand_bits)
+        gq, gs = quantize(g2, axis=-1, is_2d_block=True, use_sr=use_sr_grad, rand_bits=rand_bits, use_uos=use_uos)
         gq_m, gs_m = gq, gs
     else:
-        gq, gs = quantize(g2, axis=-1, is_2d_block=False, use_sr=use_sr_grad, rand_bits=rand_bits)
+        gq, gs = quantize(g2, axis=-1, is_2d_block=False, use_sr=use_sr_grad, rand_bits=rand_bits, use_uos=use_uos)
         gh = rht_left(g2, *hadamard) if hadamard is not None else g2
-        gq_m, gs_m = quantize(gh, axis=0, is_2d_block=False, use_sr=use_sr_grad, rand_bits=rand_bits, clip_mode=clip_mode)
+        gq_m, gs_m = quantize(gh, axis=0, is_2d_block=False, use_sr=use_sr_grad, rand_bits=rand_bits, clip_mode=clip_mode, use_uos=use_uos)
     dx = gemm_ref(gq, gs, saved["w_q"], saved["w_s"], use_2dblock_x, use_2dblock_w, k_pack_b=not use_2dblock_w, dtype=dtype)
     dw = gemm_ref(gq_m, gs_m, saved["x_q"], saved["x_s"], use_2dblock_x, use_2dblock_x, trans_a=True,
                   k_pack_a=not use_2dblock_x, k_pack_b=not use_2dblock_x, dtype=dtype)

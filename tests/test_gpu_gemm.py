@@ -91,20 +91,11 @@ def test_gemm_shape_errors(m):
         m.blockwise_mxfp4_gemm(aq, s, torch.zeros(32, 32, dtype=torch.uint8, device=DEV), torch.zeros(32, 2, dtype=torch.uint8, device=DEV), trans_b=True)
 
 
-@pytest.mark.parametrize("shape", [(1, 512, 384, 128), (4, 256, 512, 1024)])
-@pytest.mark.parametrize("use_2dblock_x,use_2dblock_w", [(False, True), (False, False), (True, True)])
-@pytest.mark.parametrize("use_sr", [False, True])
-@pytest.mark.parametrize("use_h", [False, True])
-@pytest.mark.parametrize("clip_mode", ["none", "static"])
-def test_linear_autograd(m, shape, use_2dblock_x, use_2dblock_w, use_sr, use_h, clip_mode):
-    """MXFP4LinearFunction fwd/bwd: equals the oracle's restatement of the reference flow, and meets the reference's SNR
-    floors against the high-precision linear (tests/unittest/mxfp4/test_mxfp_linear.py:105-197)."""
-    if use_2dblock_x and use_h:
-        pytest.skip("Hadamard transform is applied only if 1D block is used for activations.")
+def _linear_autograd_case(m, shape, use_2dblock_x, use_2dblock_w, use_sr, use_h, clip_mode, dtype, use_uos, floors=True):
     B, M, N, K = shape
-    x = randn_outliers((B, M, K), torch.bfloat16, seed=1234)
-    w = randn_outliers((N, K), torch.bfloat16, seed=1235)
-    target = randn_outliers((B, M, N), torch.bfloat16, seed=1236)
+    x = randn_outliers((B, M, K), dtype, seed=1234)
+    w = randn_outliers((N, K), dtype, seed=1235)
+    target = randn_outliers((B, M, N), dtype, seed=1236)
     signs, perm = hadamard_from_seed(1234)
     had = (signs, perm) if use_h else None
     r = rand_bits((B * M, N), seed=77)
@@ -113,18 +104,22 @@ def test_linear_autograd(m, shape, use_2dblock_x, use_2dblock_w, use_sr, use_h, 
         xg = x.to(DEV).requires_grad_(True)
         wg = w.to(DEV).requires_grad_(True)
         h = m.HadamardTransform(signs, perm) if use_h else None
-        y = m.MXFP4LinearFunction.apply(xg, wg, use_2dblock_x, use_2dblock_w, use_sr, False, clip_mode, False, h, False)
+        y = m.MXFP4LinearFunction.apply(xg, wg, use_2dblock_x, use_2dblock_w, use_sr, False, clip_mode, False, h, use_uos)
         y.retain_grad()
         torch.nn.functional.mse_loss(y, target.to(DEV)).backward()     # the reference test's loss (test_mxfp_linear.py:160-161)
         go = y.grad.cpu()
     finally:
         m.set_rand_bits_source(None)
-    y_ref, saved = O.linear_forward_ref(x, w, use_2dblock_x, use_2dblock_w, hadamard=had, clip_mode=clip_mode)
-    dx_ref, dw_ref = O.linear_backward_ref(go, saved, use_2dblock_x, use_2dblock_w, use_sr_grad=use_sr, rand_bits=r, hadamard=had, clip_mode=clip_mode)
-    assert y.shape == (B, M, N) and xg.grad.shape == x.shape and wg.grad.shape == w.shape
-    assert O.rel_frobenius(y.detach().cpu().reshape(-1, N), y_ref) < 4e-3
-    assert O.rel_frobenius(xg.grad.cpu().reshape(-1, K), dx_ref) < 4e-3
-    assert O.rel_frobenius(wg.grad.cpu(), dw_ref) < 4e-3
+    y_ref, saved = O.linear_forward_ref(x, w, use_2dblock_x, use_2dblock_w, hadamard=had, clip_mode=clip_mode, use_uos=use_uos)
+    dx_ref, dw_ref = O.linear_backward_ref(go, saved, use_2dblock_x, use_2dblock_w, use_sr_grad=use_sr, rand_bits=r, hadamard=had, clip_mode=clip_mode,
+                                           use_uos=use_uos)
+    assert y.shape == (B, M, N) and y.dtype == dtype and xg.grad.shape == x.shape and wg.grad.shape == w.shape
+    tol = TOL[dtype]
+    assert O.rel_frobenius(y.detach().cpu().reshape(-1, N), y_ref) < tol
+    assert O.rel_frobenius(xg.grad.cpu().reshape(-1, K), dx_ref) < tol
+    assert O.rel_frobenius(wg.grad.cpu(), dw_ref) < tol
+    if not floors:
+        return
     # accuracy floors vs the unquantized linear
     xf, wf, gf = x.double().reshape(-1, K), w.double(), go.double().reshape(-1, N)
     floor = 6.0 if clip_mode == "static" else (6.9 if use_sr else 8.4)
@@ -134,6 +129,32 @@ def test_linear_autograd(m, shape, use_2dblock_x, use_2dblock_w, use_sr, use_h, 
         # with 2D activation blocks the reference never clips (no clip_mode on those calls, mxfp_linear.py:434-446) yet still
         # rescales dW by 16/9 (:543-544); the kernels reproduce that (parity above), so no accuracy floor applies there
         assert snr_db(gf.T @ xf, wg.grad) > floor
+
+
+@pytest.mark.parametrize("shape", [(1, 512, 384, 128), (4, 256, 512, 1024)])
+@pytest.mark.parametrize("use_2dblock_x", [False, True])
+@pytest.mark.parametrize("use_2dblock_w", [False, True])
+@pytest.mark.parametrize("use_sr", [False, True])
+@pytest.mark.parametrize("use_h", [False, True])
+@pytest.mark.parametrize("clip_mode,use_uos", [("none", False), ("static", False), ("none", True)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_linear_autograd(m, shape, use_2dblock_x, use_2dblock_w, use_sr, use_h, clip_mode, use_uos, dtype):
+    """MXFP4LinearFunction fwd/bwd: equals the oracle's restatement of the reference flow, and meets the reference's SNR
+    floors against the high-precision linear (tests/unittest/mxfp4/test_mxfp_linear.py:105-197): every block-layout
+    combination, bf16 and fp32 tensors, stochastic rounding, Hadamard, static clip, UOS."""
+    if use_2dblock_x and use_h:
+        pytest.skip("Hadamard transform is applied only if 1D block is used for activations.")
+    if dtype == torch.float32 and shape[0] != 1:
+        pytest.skip("fp32 tensors run on the first shape and on the large one below")
+    _linear_autograd_case(m, shape, use_2dblock_x, use_2dblock_w, use_sr, use_h, clip_mode, dtype, use_uos, floors=not use_uos)
+
+
+@pytest.mark.parametrize("use_2dblock_x,use_2dblock_w", [(False, True), (False, False), (True, True), (True, False)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_linear_autograd_large_shape(m, use_2dblock_x, use_2dblock_w, dtype):
+    """The reference's second shape, (4, 1024, 1024, 2048) (test_mxfp_linear.py:105), with stochastic rounding and, for 1D
+    activation blocks, the Hadamard transform."""
+    _linear_autograd_case(m, (4, 1024, 1024, 2048), use_2dblock_x, use_2dblock_w, True, not use_2dblock_x, "none", dtype, False)
 
 
 @pytest.mark.parametrize("use_sr", [False, True])
@@ -352,3 +373,93 @@ def test_grouped_dw_misaligned_boundaries_are_poisoned(m, tiled):
                        groups, 2, torch.float32)
     idx2 = torch.cat([torch.ones(128 * scale, dtype=torch.int32), torch.zeros(128 * scale, dtype=torch.int32)])
     assert O.rel_frobenius(dw2.cpu(), O.grouped_gemm_dw_ref(gqm, gsm, aqm, asm, idx2, 2)) < 1e-5
+
+
+@pytest.mark.parametrize("use_2dblock_x", [False, True])
+@pytest.mark.parametrize("use_2dblock_w", [False, True])
+@pytest.mark.parametrize("trans_weights", [False, True])
+@pytest.mark.parametrize("contiguous", [False, True])
+@pytest.mark.parametrize("use_h", [False, True])
+@pytest.mark.parametrize("clip_mode", ["none", "static", "dynamic"])
+@pytest.mark.parametrize("use_uos", [False, True])
+def test_grouped_gemm_flag_matrix(m, use_2dblock_x, use_2dblock_w, trans_weights, contiguous, use_h, clip_mode, use_uos):
+    """The reference's own sweep (tests/unittest/mxfp4/test_mxfp_grouped_gemm.py:20-44) on (1024, 512, 512, 8): every block
+    layout of activations and weights, both weight orientations, transposed storage, Hadamard, the clip modes and UOS, with
+    stochastic rounding of the gradient on explicit words; forward, dX and dW against the oracle's restatement of the flow."""
+    if use_2dblock_x and use_h:
+        pytest.skip("Hadamard transform is applied only if 1D block is used for activations.")
+    if clip_mode == "dynamic" and not use_h:
+        pytest.skip("Dynamic clip mode is not supported without Hadamard transform.")
+    if use_uos and clip_mode != "none":
+        pytest.skip("UOS is not supported with clip mode.")
+    M_total, N, K, E = 1024, 512, 512, 8
+    a = randn_outliers((M_total, K), torch.bfloat16, seed=140)
+    w = randn_outliers((E, N, K), torch.bfloat16, seed=141) * 0.02          # logical [E, N, K]
+    g = torch.Generator().manual_seed(142)
+    idx = torch.randint(0, E, (M_total // 128,), generator=g, dtype=torch.int32).repeat_interleave(128)
+    go = randn_outliers((M_total, N), torch.bfloat16, seed=143) / (M_total * N)
+    r = rand_bits((M_total, N), seed=144)
+    signs, perm = hadamard_from_seed(1234)
+    # storage: [E, N, K] for trans_weights else [E, K, N]; "not contiguous" = the transposed storage behind a view
+    w_log = w if trans_weights else w.transpose(1, 2)
+    w_dev = (w_log.contiguous() if contiguous else w_log.transpose(1, 2).contiguous().transpose(1, 2)).to(DEV).requires_grad_(True)
+    a_dev = (a if contiguous else a.t().contiguous().t()).to(DEV).requires_grad_(True)
+    assert w_dev.is_contiguous() == contiguous and a_dev.is_contiguous() == contiguous
+    m.set_rand_bits_source(lambda shp, d: r.to(d))
+    m.HadamardFactory.configure(seed=1234)
+    try:
+        out = m.mxfp4_grouped_gemm(a_dev, w_dev, idx.to(DEV), trans_weights=trans_weights, use_2dblock_x=use_2dblock_x,
+                                   use_2dblock_w=use_2dblock_w, use_sr_grad=True, use_hadamard=use_h, clip_mode=clip_mode, use_uos=use_uos)
+        out.backward(go.to(DEV))
+    finally:
+        m.set_rand_bits_source(None)
+    # the oracle's flow (cg_backward.py:605-930)
+    aq, as_ = O.quantize(a, is_2d_block=use_2dblock_x, use_uos=use_uos)
+    wq, ws = O.quantize(w, axis=-1, is_2d_block=use_2dblock_w, use_uos=use_uos)
+    ref = O.grouped_gemm_ref(aq, as_, wq, ws, idx, use_2dblock_x=use_2dblock_x, use_2dblock_w=use_2dblock_w)
+    assert O.rel_frobenius(out.detach().cpu(), ref) < 4e-3
+    if use_2dblock_x:
+        gq, gs = O.quantize(go, is_2d_block=True, use_sr=True, rand_bits=r, use_uos=use_uos)
+        gqm, gsm, aqm, asm = gq, gs, aq, as_
+    else:
+        gq, gs = O.quantize(go, use_sr=True, rand_bits=r, use_uos=use_uos)
+        gh, ah = (O.rht_left(go, signs, perm), O.rht_left(a, signs, perm)) if use_h else (go, a)
+        gqm, gsm = O.quantize(gh, axis=0, use_sr=True, rand_bits=r, clip_mode=clip_mode, use_uos=use_uos)
+        aqm, asm = O.quantize(ah, axis=0, clip_mode=clip_mode, use_uos=use_uos)
+    if use_2dblock_w:
+        dx_ref = O.grouped_gemm_dx_ref(gq, gs, wq, ws, idx, use_2dblock_x=use_2dblock_x, use_2dblock_w=True, k_pack_w=False)
+    else:   # 1D weight blocks: a second quantisation along N serves dX
+        wq2, ws2 = O.quantize(w, axis=-2, use_uos=use_uos)
+        dx_ref = O.grouped_gemm_dx_ref(gq, gs, wq2, ws2, idx, use_2dblock_x=use_2dblock_x, use_2dblock_w=False, k_pack_w=True)
+    assert O.rel_frobenius(a_dev.grad.cpu(), dx_ref) < 4e-3
+    dw_ref = O.grouped_gemm_dw_ref(gqm, gsm, aqm, asm, idx, E, use_2dblock_x=use_2dblock_x, trans_weights=trans_weights)
+    if clip_mode == "static":
+        dw_ref = dw_ref * (16.0 / 9.0)
+    assert w_dev.grad.shape == w_dev.shape
+    assert O.rel_frobenius(w_dev.grad.cpu(), dw_ref) < 4e-3
+    # the reference's accuracy floor on the forward result (its dX / dW floors are stated for round-to-nearest gradients)
+    o_hp = torch.cat([a.double()[i:i + 128] @ w.double()[int(idx[i])].T for i in range(0, M_total, 128)])
+    assert snr_db(o_hp, out.detach()) > 10
+
+
+def test_grouped_backward_weights_operand_forms(m):
+    """mxfp4_grouped_gemm_backward_weights (cg_backward.py:398-497) with operands packed along the tokens (k_pack) or along
+    the features, 1D or 2D scales: all four give the oracle's dW."""
+    M_total, N, K, E = 512, 256, 384, 4
+    go = randn_outliers((M_total, N), torch.bfloat16, seed=150) / 100
+    a = randn_outliers((M_total, K), torch.bfloat16, seed=151)
+    idx = torch.tensor([2, 0, 0, 3], dtype=torch.int32).repeat_interleave(128)
+    for is_2d in (False, True):
+        if is_2d:
+            gq, gs = O.quantize(go, is_2d_block=True)            # [M, N/2], [M/32, N/32]
+            xq, xs = O.quantize(a, is_2d_block=True)
+            forms = [(gq, xq, False), (O.pack_nibbles(O.unpack_nibbles(gq).t().contiguous()).t(), O.pack_nibbles(O.unpack_nibbles(xq).t().contiguous()).t(), True)]
+        else:
+            gq, gs = O.quantize(go, axis=0)                      # [M/2, N] over [N][M/2] memory, [M/32, N]
+            xq, xs = O.quantize(a, axis=0)
+            forms = [(gq, xq, True), (O.pack_nibbles(O.unpack_nibbles(gq.t().contiguous()).t().contiguous()), O.pack_nibbles(O.unpack_nibbles(xq.t().contiguous()).t().contiguous()), False)]
+        ref = O.grouped_gemm_dw_ref(gq, gs, xq, xs, idx, E, use_2dblock_x=is_2d)
+        for g_codes, x_codes, k_pack in forms:
+            dw = m.mxfp4_grouped_gemm_backward_weights(g_codes.to(DEV), x_codes.to(DEV), idx.to(DEV), E, gs.to(DEV), xs.to(DEV), True, is_2d, is_2d,
+                                                       k_pack, k_pack, torch.float32)
+            assert O.rel_frobenius(dw.cpu(), ref) < 1e-5, (is_2d, k_pack)
