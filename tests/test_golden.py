@@ -112,3 +112,64 @@ def test_hip_attention_and_dynamic_clip_vectors(m):
     q, s = m.convert_to_mxfp4(bf16("rne_x_bf16bits").cuda(), clip_mode="dynamic")
     assert_bytes_equal(q, t("dyn_codes"), "dynamic-clip codes")
     assert_bytes_equal(s, t("dyn_scales"), "dynamic-clip scales")
+
+
+# ---------------------------------------------------------------------------------------------- vectors made by the reference
+def _ref_vectors():
+    return np.load(os.path.join(os.path.dirname(__file__), "golden", "reference_vectors.npz"))
+
+
+@pytest.mark.parametrize("name,kw", [("row", dict(axis=-1)), ("col", dict(axis=-2)), ("2d", dict(axis=-1, is_2d_block=True))])
+def test_dynamic_clip_equals_the_reference_twin(name, kw):
+    """clip_mode="dynamic" on fp32 data: the oracle reproduces, byte for byte, the codes, scales and dequantised values
+    that the reference's PyTorch twin computed (tests/golden/make_reference_vectors.py) -- the function its own test holds
+    bit-equal to the Triton kernel for fp32 tensors (tests/unittest/mxfp4/test_mxfp_quantization.py:62-75)."""
+    d = _ref_vectors()
+    x = torch.from_numpy(d["dyn_x"])
+    q, s = O.quantize(x, clip_mode="dynamic", **kw)
+    assert torch.equal(s.contiguous(), torch.from_numpy(d[f"dyn_{name}_scales"]))
+    assert torch.equal(q.contiguous(), torch.from_numpy(d[f"dyn_{name}_codes"]))
+    dq = O.dequantize(q, s, torch.float32, clip_mode="dynamic", **kw)
+    assert torch.equal(dq.contiguous(), torch.from_numpy(d[f"dyn_{name}_dq"]))
+
+
+@pytest.mark.parametrize("name", ["a", "b", "c"])
+def test_attention_model_equals_the_reference_cpu_model(name):
+    """The oracle's MXFP4 attention recurrence gives the reference CPU model's outputs (test_mxfp_pnq.py:87-149) bit for
+    bit with natural exponentials, and within one bf16 rounding with the kernel's exp2 formulation."""
+    from oracle.attention_oracle import attention_fwd_ref
+    d = _ref_vectors()
+    q, k, v = (torch.from_numpy(d[f"attn_{name}_{t}"]).view(torch.bfloat16) for t in "qkv")
+    exp = torch.from_numpy(d[f"attn_{name}_out"]).view(torch.bfloat16)
+    out, _ = attention_fwd_ref(q, k, v, causal=bool(d[f"attn_{name}_causal"]), use_exp2=False)
+    assert torch.equal(out.view(torch.int16), exp.view(torch.int16))
+    out2, _ = attention_fwd_ref(q, k, v, causal=bool(d[f"attn_{name}_causal"]), use_exp2=True)
+    assert float((out2.float() - exp.float()).norm() / exp.float().norm()) < 4e-3
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name,kw", [("row", dict(axis=-1)), ("col", dict(axis=-2)), ("2d", dict(axis=-1, is_2d_block=True))])
+def test_hip_dynamic_clip_equals_the_reference_twin(name, kw):
+    """The HIP quantizer with clip_mode="dynamic" reproduces the reference twin's fp32 vectors byte for byte."""
+    import alto_amd.mxfp4 as m
+    d = _ref_vectors()
+    x = torch.from_numpy(d["dyn_x"]).cuda()
+    q, s = m.convert_to_mxfp4(x, clip_mode="dynamic", **kw)
+    assert_bytes_equal(s.contiguous(), torch.from_numpy(d[f"dyn_{name}_scales"]), f"dynamic {name} scales")
+    assert_bytes_equal(q.contiguous(), torch.from_numpy(d[f"dyn_{name}_codes"]), f"dynamic {name} codes")
+    dq = m.convert_from_mxfp4(q, s, torch.float32, clip_mode="dynamic", **kw)
+    assert torch.equal(dq.contiguous().cpu(), torch.from_numpy(d[f"dyn_{name}_dq"]))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", ["a", "b", "c"])
+def test_hip_attention_close_to_the_reference_cpu_model(name):
+    """The HIP attention kernel on the fixture's Q, K, V against the reference CPU model's output: relative L2 <= 4e-3
+    (exp2 formulation and v_exp_f32 against libm's exp: a probability can cross an E2M1 rounding boundary)."""
+    import alto_amd.mxfp4 as m
+    d = _ref_vectors()
+    q, k, v = (torch.from_numpy(d[f"attn_{name}_{t}"]).view(torch.bfloat16).cuda() for t in "qkv")
+    exp = torch.from_numpy(d[f"attn_{name}_out"]).view(torch.bfloat16)
+    out = m.triton_attention_mxfp4(q, k, v, causal=bool(d[f"attn_{name}_causal"]))
+    out = out[0] if isinstance(out, (tuple, list)) else out
+    assert float((out.float().cpu() - exp.float()).norm() / exp.float().norm()) < 4e-3

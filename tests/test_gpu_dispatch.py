@@ -3,6 +3,7 @@
 import pytest
 import torch
 
+import oracle as O
 from tests.helpers import rand_bits, randn_outliers
 
 pytestmark = pytest.mark.gpu
@@ -84,23 +85,26 @@ def test_grouped_mm_through_wrapper(m):
 @pytest.mark.parametrize("is_2d", [True, False])
 @pytest.mark.parametrize("use_uos", [False, True])
 def test_fused_qdq_equals_quantize_then_dequantize(m, dtype, is_2d, use_uos):
-    """One launch == convert_from_mxfp4(convert_to_mxfp4(w)) bit for bit (the de-oscillation hook, optimizer.py:123-168)."""
-    w = (randn_outliers((3, 96, 320), dtype, seed=11) * 0.02).to(DEV)
+    """One launch == the oracle's dequantize(quantize(w)) bit for bit (the de-oscillation hook, optimizer.py:123-168), and
+    therefore also the two separate HIP launches."""
+    w_cpu = randn_outliers((3, 96, 320), dtype, seed=11) * 0.02
+    w = w_cpu.to(DEV)
+    bits = torch.int16 if dtype == torch.bfloat16 else torch.int32
     for axis in (-1, -2):
-        q, s = m.convert_to_mxfp4(w, axis=axis, is_2d_block=is_2d, use_uos=use_uos)
-        ref = m.convert_from_mxfp4(q, s, output_dtype=dtype, axis=axis, is_2d_block=is_2d)
+        exp = O.dequantize(*O.quantize(w_cpu, axis=axis, is_2d_block=is_2d, use_uos=use_uos), dtype, axis=axis, is_2d_block=is_2d)
         got = m.quantize_dequantize(w, axis=axis, is_2d_block=is_2d, use_uos=use_uos)
         assert got.dtype == dtype and got.shape == w.shape
-        assert torch.equal(got.view(torch.int16 if dtype == torch.bfloat16 else torch.int32),
-                           ref.contiguous().view(torch.int16 if dtype == torch.bfloat16 else torch.int32)), (axis, is_2d)
+        assert torch.equal(got.cpu().view(bits), exp.contiguous().view(bits)), (axis, is_2d)
+        q, s = m.convert_to_mxfp4(w, axis=axis, is_2d_block=is_2d, use_uos=use_uos)
+        ref = m.convert_from_mxfp4(q, s, output_dtype=dtype, axis=axis, is_2d_block=is_2d)
+        assert torch.equal(got.view(bits), ref.contiguous().view(bits)), (axis, is_2d)
     # the recipe-level closure, with a row count that is not a multiple of 32 (padded as the reference does)
     cfg = m.TrainingOpConfig(use_2dblock_w=is_2d, use_uos=use_uos)
-    w2 = (randn_outliers((100, 256), dtype, seed=12) * 0.02).to(DEV)
-    got = m._make_qdq_fn_for(cfg)(w2, -1)
-    wp = torch.nn.functional.pad(w2, (0, 0, 0, 28))
-    q, s = m.convert_to_mxfp4(wp, axis=-1, is_2d_block=is_2d, use_uos=use_uos)
-    ref = m.convert_from_mxfp4(q, s, output_dtype=dtype, axis=-1, is_2d_block=is_2d)[:100]
-    assert got.shape == (100, 256) and torch.equal(got, ref)
+    w2_cpu = randn_outliers((100, 256), dtype, seed=12) * 0.02
+    got = m._make_qdq_fn_for(cfg)(w2_cpu.to(DEV), -1)
+    wp = torch.nn.functional.pad(w2_cpu, (0, 0, 0, 28))
+    exp = O.dequantize(*O.quantize(wp, axis=-1, is_2d_block=is_2d, use_uos=use_uos), dtype, axis=-1, is_2d_block=is_2d)[:100]
+    assert got.shape == (100, 256) and torch.equal(got.cpu(), exp)
 
 
 def test_weight_cache_reuses_until_weight_changes(m):
@@ -146,6 +150,14 @@ def test_dge_scales_the_weight_gradient(m, clip_mode):
     # one rounding in the GEMM epilogue (acc * (16/9 * 0.2)) versus the reference's two: within a few fp32 ulps
     torch.testing.assert_close(grads[True][2], grads[False][2] * f, rtol=4e-7, atol=0)
     assert grads[False][2].abs().max() > 0
+    # against the oracle: its dW times dge_bwd evaluated element by element at the quantised weight's grid values
+    xc, wc, gc = x.cpu(), w.cpu(), go.cpu()
+    _, saved = O.linear_forward_ref(xc, wc, False, True, clip_mode=clip_mode)
+    _, dw_ref = O.linear_backward_ref(gc, saved, False, True, clip_mode=clip_mode)
+    wq, _ = O.quantize(wc, is_2d_block=True)
+    factor = O.dge_bwd_ref(O.weight_grid_values(wq))
+    assert factor.shape == wc.shape and float((factor - 0.2).abs().max()) < 1e-6
+    assert O.rel_frobenius(grads[True][2].cpu(), dw_ref * factor.double()) < 1e-5
 
 
 def test_dge_grouped_weight_gradient(m):
@@ -163,6 +175,13 @@ def test_dge_grouped_weight_gradient(m):
     assert torch.equal(grads[True][0], grads[False][0])
     torch.testing.assert_close(grads[True][1], grads[False][1] * 0.2, rtol=4e-7, atol=0)
     assert grads[False][1].abs().max() > 0
+    # against the oracle's flow times dge_bwd at the grid values of the quantised expert weights
+    xc, wc, gc, ic = x.cpu(), w.cpu(), go.cpu(), idx.cpu()
+    gqm, gsm = O.quantize(gc, axis=0)
+    aqm, asm = O.quantize(xc, axis=0)
+    dw_ref = O.grouped_gemm_dw_ref(gqm, gsm, aqm, asm, ic, E)
+    wq, _ = O.quantize(wc, is_2d_block=True)
+    assert O.rel_frobenius(grads[True][1].cpu(), dw_ref * O.dge_bwd_ref(O.weight_grid_values(wq)).double()) < 1e-5
 
 
 def test_registered_torch_ops_run_the_hip_kernels(m):

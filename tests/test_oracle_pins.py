@@ -414,3 +414,42 @@ def test_philox4x32_10_known_answers():
     big = random_bits(4 * 1500, seed=3, offset=2 ** 64 - 700)
     assert np.array_equal(big[:4 * 600], random_bits(4 * 600, seed=3, offset=2 ** 64 - 700))
     assert np.array_equal(big[4 * 700:4 * 704], random_bits(16, seed=3, offset=2 ** 64))
+
+
+# ------------------------------------------------------------------------------------------------ dynamic clip, estimator
+def test_dynamic_clip_scale_known_answers():
+    """clip_mode="dynamic" (mxfp_quantization.py:54-59,65-70): max_abs = (2.92247856 / 6) std + 1e-8 with the population
+    standard deviation of the block, exponent after rounding to one mantissa bit, no "-2".  Closed forms:
+    a constant block (and an all-zero one) has std 0, so max_abs = 1e-8 = 0x322BCC77 -> byte 100; a block of +-a has mean 0
+    and std a, so +-1.5 gives 0.7306... -> byte 126, +-2^k gives 0.4870... 2^k -> byte 127 + k - 1 (1.948 rounds up to the
+    next binade: 0.487 = 1.948 2^-2, and 1.948 + 0.25 >= 2)."""
+    for dtype in (torch.float32,):
+        x = torch.zeros(8, 32, dtype=dtype)
+        x[0] = 3.0
+        x[2] = torch.tensor([1.5, -1.5] * 16)
+        x[3] = torch.tensor([4.0, -4.0] * 16)
+        x[4] = torch.tensor([2.0 ** -10, -(2.0 ** -10)] * 16)
+        s = O.block_scales(x, False, clip_mode="dynamic")
+        assert s[:5, 0].tolist() == [100, 100, 126, 127 + 2 - 1, 127 - 10 - 1]
+        # 2D: one statistic over the 32 x 32 block
+        y = torch.zeros(32, 64, dtype=dtype)
+        y[:, 32:] = torch.tensor([1.5, -1.5] * 16)
+        assert O.block_scales(y, True, clip_mode="dynamic").tolist() == [[100, 126]]
+
+
+def test_dge_multiplier_is_the_derivative_of_the_estimator():
+    """dge_bwd (alto/kernels/dge/dge.py:80-93) against what the mathematics fixes: at every E2M1 grid value the two powers
+    cancel and leave 1/k; inside an interval it is the derivative of dge_fwd (:62-77), whose end points are fixed points, so
+    it integrates to the interval's width; next to the mid point it is clamped at 3."""
+    k = 5.0
+    grid = torch.tensor([0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0, -0.5, -1.0, -1.5, -2.0, -3.0, -4.0, -6.0])
+    assert float((O.dge_bwd_ref(grid, k) - 1 / k).abs().max()) < 1e-6
+    for lo, hi in ((1.0, 1.5), (2.0, 3.0), (-6.0, -4.0), (4.0, 6.0)):
+        half, mid = (hi - lo) / 2, (lo + hi) / 2
+        # substitute x = mid + half u^k (u in [0, 1]): the integrand of the upper half becomes half, a constant
+        u = torch.linspace(0, 1, 20001, dtype=torch.float64)[1:]
+        x = (mid + half * u ** k).float()
+        unclamped_region = O.dge_bwd_ref(x, k) < 3.0
+        integrand = O.dge_bwd_ref(x, k).double() * (half * k * u ** (k - 1))
+        assert bool(((integrand[unclamped_region] - half).abs() < 1e-3 * half).all())
+    assert float(O.dge_bwd_ref(torch.tensor([1.25 + 1e-6, 2.5 - 1e-7]), k).min()) == 3.0
