@@ -34,13 +34,15 @@ def _laplace(shape, scale, device, gen):
 
 
 def _time_steps(fn, steps, warmup):
-    """Average milliseconds per call of fn, HIP events on the current stream bracketing exactly `steps` calls."""
+    """HIP events on the launch stream (torch's current stream, which every entry point is given) bracket exactly `steps`
+    back-to-back calls of fn: that is the reported time.  A second pass of `steps` calls with an event between consecutive
+    calls gives the spread (the markers cost a couple of microseconds each, so they stay out of the first pass).
+    Returns (mean ms per step of the bracket, host wall ms per step, sorted per-step ms of the second pass)."""
     import torch
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
-    e0 = torch.cuda.Event(enable_timing=True)
-    e1 = torch.cuda.Event(enable_timing=True)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
     e0.record()
     for _ in range(steps):
@@ -48,7 +50,14 @@ def _time_steps(fn, steps, warmup):
     e1.record()
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3 / steps
-    return e0.elapsed_time(e1) / steps, wall_ms
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
+    ev[0].record()
+    for i in range(steps):
+        fn()
+        ev[i + 1].record()
+    torch.cuda.synchronize()
+    per = sorted(ev[i].elapsed_time(ev[i + 1]) for i in range(steps))
+    return e0.elapsed_time(e1) / steps, wall_ms, per
 
 
 # ------------------------------------------------------------------------------------------------ workloads
@@ -440,12 +449,18 @@ class MfmaProbe(Workload):
         from alto_amd.mxfp4 import _runtime as rt
         self.rt, self.stream = rt, rt.stream_ptr(dev)
         self.sink = torch.zeros(512, dtype=torch.float32, device=dev)
+        self.ticks = torch.zeros(2, dtype=torch.int64, device=dev)
         self.iters, self.wgs = 4000, torch.cuda.get_device_properties(dev).multi_processor_count
         self.work = 2.0 * 32 * 32 * 64 * 8 * self.iters * 8 * self.wgs
 
     def step(self):
-        code = self.rt.lib().alto_mxfp4_probe_mfma(self.random, self.iters, self.wgs, self.sink.data_ptr(), self.stream)
+        code = self.rt.lib().alto_mxfp4_probe_mfma(self.random, self.iters, self.wgs, self.sink.data_ptr(), self.ticks.data_ptr(), self.stream)
         assert code == 0, code
+
+    def extra(self):
+        """The clock the chip held during the last launch: shader-clock cycles per tick of the constant 100 MHz counter."""
+        cycles, ticks = (int(v) for v in self.ticks.cpu())
+        return {"clock_mhz": round(100.0 * cycles / ticks, 1) if ticks > 0 else None}
 
     def cpu_sample(self):
         raise NotImplementedError("the probe has no CPU counterpart")
@@ -487,13 +502,25 @@ def measure(w, dev, gen, steps, warmup):
     import torch
     w.setup(dev, gen)
     torch.cuda.synchronize()
-    ms, wall_ms = _time_steps(w.step, steps, warmup)
+    ms, wall_ms, per = _time_steps(w.step, steps, warmup)
     if w.bound == "mfma":
         achieved, peak, unit = w.work / (ms * 1e-3) / 1e12, PEAK_MXFP4_TFLOPS, "TFLOP/s"
     else:
         achieved, peak, unit = w.work / (ms * 1e-3) / 1e9, PEAK_HBM_GBS, "GB/s"
-    return {"workload": w.name, "kernel": w.kernel, "ms": ms, "wall_ms": wall_ms, "achieved": achieved, "peak": peak, "unit": unit,
-            "bound": w.bound, "frac": achieved / peak}
+    res = {"workload": w.name, "kernel": w.kernel, "ms": ms, "wall_ms": wall_ms, "achieved": achieved, "peak": peak, "unit": unit,
+           "bound": w.bound, "frac": achieved / peak, "ms_median": per[len(per) // 2], "ms_min": per[0], "ms_max": per[-1]}
+    if hasattr(w, "extra"):
+        res.update(w.extra())
+    return res
+
+
+def _brief(r):
+    """The fields of a measurement that go into "others"."""
+    out = {"workload": r["workload"], "ms": round(r["ms"], 4), "ms_median": round(r["ms_median"], 4), "ms_min": round(r["ms_min"], 4),
+           "ms_max": round(r["ms_max"], 4), "achieved": round(r["achieved"], 2), "unit": r["unit"], "bound": r["bound"], "frac": round(r["frac"], 4)}
+    if "clock_mhz" in r:
+        out["clock_mhz"] = r["clock_mhz"]
+    return out
 
 
 def cpu_baseline(w):
@@ -552,14 +579,16 @@ def main():
         print(f"bench.py: no cpu_baseline for {args.workload}: {e}", file=sys.stderr)
         cpu = None
     others = {}
+    clock_observed = None
     if not args.only:
         for key, w in wl.items():
             if key == args.workload or key == "copy_calib":
                 continue
-            if key.startswith("mfma_probe"):   # the pipe's own rate, reported beside the published peak
+            if key.startswith("mfma_probe"):   # the pipe's own rate and clock, reported beside the published peak
                 r = measure(w, dev, gen, 3, 1)
-                others[key] = {"workload": r["workload"], "ms": round(r["ms"], 4), "achieved": round(r["achieved"], 2), "unit": r["unit"],
-                               "bound": r["bound"], "frac": round(r["frac"], 4)}
+                others[key] = _brief(r)
+                if key == "mfma_probe_random":
+                    clock_observed = r.get("clock_mhz")
                 continue
             primary_mem_release = None  # noqa: F841
             try:
@@ -570,8 +599,10 @@ def main():
                         raise
                     others[key] = {"workload": w.name, "error": str(e)[:200]}
                     continue
-                others[key] = {"workload": r["workload"], "ms": round(r["ms"], 4), "achieved": round(r["achieved"], 2), "unit": r["unit"],
-                               "bound": r["bound"], "frac": round(r["frac"], 4)}
+                others[key] = _brief(r)
+                if key == "cfg2_quant":   # the metric names the quantizer too: its own traffic figure and CPU leg
+                    others[key]["traffic"] = load_traffic(key)
+                    others[key]["cpu_baseline"] = None if args.no_cpu else cpu_baseline(w)
             finally:
                 for attr in list(vars(w)):
                     if attr not in ("name", "work"):
@@ -591,8 +622,10 @@ def main():
         "vs_baseline": None,
         "dtype": "mxfp4 (e2m1 codes, e8m0 scales), fp32 accumulate" if res["bound"] == "mfma" else "bf16 -> e2m1/e8m0 (u8 bit ops, fp32 transform)",
         "data": "synthetic",
-        "config": {"workload": res["workload"], "device": props.name, "cus": props.multi_processor_count,
-                   "clock_mhz": props.clock_rate // 1000 if hasattr(props, "clock_rate") else None},
+        # clock_mhz: what the chip held under a register-only loop of FP4 MFMAs on random operands in this run (shader
+        # cycles per tick of the constant 100 MHz counter); null with --only, which skips that probe
+        "config": {"workload": res["workload"], "device": props.name, "cus": props.multi_processor_count, "clock_mhz": clock_observed},
+        "ms_median": round(res["ms_median"], 5), "ms_min": round(res["ms_min"], 5), "ms_max": round(res["ms_max"], 5),
         "roofline": {"bound": res["bound"], "achieved": round(res["achieved"], 3), "peak": res["peak"], "unit": res["unit"],
                      "frac": round(res["frac"], 4), "traffic": load_traffic(args.workload), "kernel": res["kernel"], "kernel_ms": round(res["ms"], 5)},
         "cpu_baseline": cpu,

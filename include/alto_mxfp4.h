@@ -283,9 +283,11 @@ int alto_mxfp4_random_bits(uint32_t* out, int64_t n, uint64_t seed, uint64_t off
  * (8 per iteration and wave, 8 waves per workgroup, `workgroups` workgroups; 2*32*32*64 FLOP each),
  * with constant (random_operands = 0) or pseudo-random FP4 operands.  bench.py times it to report
  * the rate the matrix pipe itself sustains on this part next to the published peak.
- * `sink` is device memory for 512 floats (practically never written).
+ * `sink` is device memory for 512 floats (practically never written).  `ticks` is NULL or device memory for two uint64:
+ * the shader-clock cycles and the ticks of the constant 100 MHz counter that the loop of workgroup 0 took, whose ratio is
+ * the clock the chip held under this load.
  */
-int alto_mxfp4_probe_mfma(int random_operands, int iters, int workgroups, float* sink, void* stream);
+int alto_mxfp4_probe_mfma(int random_operands, int iters, int workgroups, float* sink, uint64_t* ticks, void* stream);
 
 #ifdef __cplusplus
 }
