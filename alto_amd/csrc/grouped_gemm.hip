@@ -214,15 +214,45 @@ struct PassWalk {
 
 constexpr int PLAN_THREADS = 256;
 
-// one workgroup: thread t owns the bands [t nb, (t + 1) nb); counts their passes, then writes them at the offset an
-// exclusive scan of the counts gives, so the list is in band order
+// One workgroup.  Two ways to cut the rows into passes, same list format:
+//  * groups in expert order (group_expert == NULL, the sorted form of torch._grouped_mm): every group is tiled from its
+//    own first row in steps of 256, so an expert has at most one partial tile (about E / 2 partial tiles in all, where
+//    cutting fixed 256-row bands at the expert boundaries gives one extra pass per boundary); the rows before the first
+//    and after the last group are tiled the same way as zero-fill passes.  Item i of the walk: 0 = head, 1..G = groups,
+//    G + 1 = tail; thread t owns a block of consecutive items.
+//  * per-group expert ids (the reference's form, one id per aligned 128-row group, any order): thread t owns the bands
+//    [t nb, (t + 1) nb) and emits, per band, one pass per run of groups of the same expert.
+// Either way a thread counts its passes, an exclusive scan of the counts gives its offset, and it writes them there,
+// so the list is in row order.
 __global__ __launch_bounds__(PLAN_THREADS) void grouped_plan_kernel(PassWalk wk, int tiles_m, int32_t* ws, int max_pass) {
   __shared__ int scan[PLAN_THREADS];
   const int t = threadIdx.x;
-  const int nb = (tiles_m + PLAN_THREADS - 1) / PLAN_THREADS;
-  const int b0 = t * nb, b1 = (b0 + nb) < tiles_m ? (b0 + nb) : tiles_m;
+  const bool sorted = wk.group_expert == nullptr;
+  const int items = sorted ? wk.num_groups + 2 : tiles_m;
+  const int per = (items + PLAN_THREADS - 1) / PLAN_THREADS;
+  const int i0 = t * per, i1 = (i0 + per) < items ? (i0 + per) : items;
+  const int Mt = (int)wk.M_total;
+  // row range and expert of item i of the sorted form
+  auto item = [&](int i, int& lo, int& hi, int& e) {
+    if (i == 0) { lo = 0; hi = wk.off_at(0); e = -1; }
+    else if (i == wk.num_groups + 1) { lo = wk.off_at(wk.num_groups); hi = Mt; e = -1; }
+    else { lo = wk.off_at(i - 1); hi = wk.off_at(i); e = (i - 1) < wk.num_experts ? i - 1 : -1; }
+    if (i > 0 && lo < wk.off_at(0)) lo = wk.off_at(0);   // offsets that go backwards never make two passes own a row
+    if (hi < lo) hi = lo;
+  };
+  auto walk = [&](auto&& emit) {
+    for (int i = i0; i < i1; ++i) {
+      if (sorted) {
+        int lo, hi, e;
+        item(i, lo, hi, e);
+        for (int r = lo; r < hi; r += GT_TM) emit(r, r, r + GT_TM < hi ? r + GT_TM : hi, e);
+      } else {
+        wk.band(i, [&](int lo, int hi, int e) { emit(i * GT_TM, lo, hi, e); });
+      }
+    }
+  };
   int cnt = 0;
-  for (int tm = b0; tm < b1; ++tm) wk.band(tm, [&](int, int, int) { ++cnt; });
+  walk([&](int, int, int, int) { ++cnt; });
   scan[t] = cnt;
   __syncthreads();
   for (int d = 1; d < PLAN_THREADS; d <<= 1) {   // inclusive scan
@@ -233,11 +263,10 @@ __global__ __launch_bounds__(PLAN_THREADS) void grouped_plan_kernel(PassWalk wk,
   }
   int at = scan[t] - cnt;
   int4* list = reinterpret_cast<int4*>(ws + 4);
-  for (int tm = b0; tm < b1; ++tm)
-    wk.band(tm, [&](int lo, int hi, int e) {
-      if (at < max_pass) list[at] = make_int4(tm * GT_TM, lo, hi, e);
-      ++at;
-    });
+  walk([&](int row0, int lo, int hi, int e) {
+    if (at < max_pass) list[at] = make_int4(row0, lo, hi, e);
+    ++at;
+  });
   if (t == PLAN_THREADS - 1) ws[0] = scan[t] < max_pass ? scan[t] : max_pass;
 }
 
