@@ -33,11 +33,24 @@ def _laplace(shape, scale, device, gen):
     return (-scale * torch.sign(u) * torch.log1p(-2 * u.abs())).bfloat16()
 
 
-def _time_steps(fn, steps, warmup):
-    """HIP events on the launch stream (torch's current stream, which every entry point is given) bracket exactly `steps`
-    back-to-back calls of fn: that is the reported time.  A second pass of `steps` calls with an event between consecutive
-    calls gives the spread (the markers cost a couple of microseconds each, so they stay out of the first pass).
-    Returns (mean ms per step of the bracket, host wall ms per step, sorted per-step ms of the second pass)."""
+def _settle(fn, settle_ms):
+    """Runs fn back to back, untimed, for settle_ms of wall time.  From idle the part's power management needs some 60 ms
+    of sustained load to reach the clock it then holds (the first launches of a burst run 20 to 60 % slower); a training
+    step sees the settled clock, so that is the state the timed steps are taken in.  Returns the number of calls made."""
+    import torch
+    n = 0
+    t0 = time.perf_counter()
+    while (time.perf_counter() - t0) * 1e3 < settle_ms:
+        for _ in range(8):
+            fn()
+        torch.cuda.synchronize()
+        n += 8
+    return n
+
+
+def _bracket(fn, steps, warmup):
+    """`warmup` untimed calls, then HIP events on the launch stream (torch's current stream, which every entry point is
+    given) around exactly `steps` back-to-back calls.  Returns (mean ms per step, host wall ms per step)."""
     import torch
     for _ in range(warmup):
         fn()
@@ -49,7 +62,16 @@ def _time_steps(fn, steps, warmup):
         fn()
     e1.record()
     torch.cuda.synchronize()
-    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    return e0.elapsed_time(e1) / steps, (time.perf_counter() - t0) * 1e3 / steps
+
+
+def _time_steps(fn, steps, warmup, settle_ms):
+    """Settling calls, then the bracket of `_bracket`: that is the reported time.  A second pass of `steps` calls with an
+    event between consecutive calls gives the spread (the markers cost a couple of microseconds each, so they stay out of
+    the first pass).  Returns (mean ms per step of the bracket, host wall ms per step, sorted per-step ms of the second pass)."""
+    import torch
+    _settle(fn, settle_ms)
+    ms, wall_ms = _bracket(fn, steps, warmup)
     ev = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
     ev[0].record()
     for i in range(steps):
@@ -57,7 +79,7 @@ def _time_steps(fn, steps, warmup):
         ev[i + 1].record()
     torch.cuda.synchronize()
     per = sorted(ev[i].elapsed_time(ev[i + 1]) for i in range(steps))
-    return e0.elapsed_time(e1) / steps, wall_ms, per
+    return ms, wall_ms, per
 
 
 # ------------------------------------------------------------------------------------------------ workloads
@@ -498,17 +520,25 @@ def make_workloads():
     }
 
 
-def measure(w, dev, gen, steps, warmup):
+def measure(w, dev, gen, steps, warmup, settle_ms, from_idle=False):
+    """from_idle: also time `steps` calls after `warmup` calls BEFORE the settling phase, after half a second without
+    work, i.e. what a short burst on an idle device sees (reported beside the settled figure, never as the value)."""
     import torch
     w.setup(dev, gen)
     torch.cuda.synchronize()
-    ms, wall_ms, per = _time_steps(w.step, steps, warmup)
+    idle_ms = None
+    if from_idle:
+        time.sleep(0.5)
+        idle_ms, _ = _bracket(w.step, steps, warmup)
+    ms, wall_ms, per = _time_steps(w.step, steps, warmup, settle_ms)
     if w.bound == "mfma":
         achieved, peak, unit = w.work / (ms * 1e-3) / 1e12, PEAK_MXFP4_TFLOPS, "TFLOP/s"
     else:
         achieved, peak, unit = w.work / (ms * 1e-3) / 1e9, PEAK_HBM_GBS, "GB/s"
     res = {"workload": w.name, "kernel": w.kernel, "ms": ms, "wall_ms": wall_ms, "achieved": achieved, "peak": peak, "unit": unit,
            "bound": w.bound, "frac": achieved / peak, "ms_median": per[len(per) // 2], "ms_min": per[0], "ms_max": per[-1]}
+    if idle_ms is not None:
+        res["from_idle_ms"] = idle_ms
     if hasattr(w, "extra"):
         res.update(w.extra())
     return res
@@ -547,6 +577,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--settle-ms", type=float, default=150.0,
+                    help="untimed back-to-back calls of each workload for this long before its warm-up and timed steps (clock settling)")
     ap.add_argument("--workload", default="cfg3_fprop", help="primary workload; one of " + ", ".join(make_workloads()))
     ap.add_argument("--only", action="store_true", help="measure the primary workload only (for profiling runs)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -572,7 +604,7 @@ def main():
         print(f"unknown workload {args.workload}", file=sys.stderr)
         sys.exit(2)
     primary = wl[args.workload]
-    res = measure(primary, dev, gen, args.steps, args.warmup)
+    res = measure(primary, dev, gen, args.steps, args.warmup, args.settle_ms, from_idle=not args.only)
     try:
         cpu = None if args.no_cpu else cpu_baseline(primary)
     except NotImplementedError as e:   # a composite workload without a CPU leg of its own
@@ -585,7 +617,7 @@ def main():
             if key == args.workload or key == "copy_calib":
                 continue
             if key.startswith("mfma_probe"):   # the pipe's own rate and clock, reported beside the published peak
-                r = measure(w, dev, gen, 3, 1)
+                r = measure(w, dev, gen, 3, 1, args.settle_ms)
                 others[key] = _brief(r)
                 if key == "mfma_probe_random":
                     clock_observed = r.get("clock_mhz")
@@ -593,7 +625,7 @@ def main():
             primary_mem_release = None  # noqa: F841
             try:
                 try:
-                    r = measure(w, dev, gen, max(5, args.steps // 2), max(2, args.warmup // 2))
+                    r = measure(w, dev, gen, max(5, args.steps // 2), max(2, args.warmup // 2), args.settle_ms)
                 except (RuntimeError, AttributeError, NotImplementedError) as e:
                     if key != "cfg3_fprop_vendor":
                         raise
@@ -609,6 +641,11 @@ def main():
                         setattr(w, attr, None)
                 torch.cuda.empty_cache()
 
+    if "from_idle_ms" in res:   # the same K steps on a device that was idle: the clock is still on its way up
+        t = res["from_idle_ms"]
+        rate = primary.work / (t * 1e-3) / (1e12 if res["bound"] == "mfma" else 1e9)
+        others[args.workload + "_from_idle"] = {"workload": res["workload"] + ", after 0.5 s without work, no settling calls", "ms": round(t, 4),
+                                                "achieved": round(rate, 2), "unit": res["unit"], "bound": res["bound"], "frac": round(rate / res["peak"], 4)}
     line = {
         "metric": METRIC,
         "value": round(res["achieved"], 3),
@@ -624,7 +661,9 @@ def main():
         "data": "synthetic",
         # clock_mhz: what the chip held under a register-only loop of FP4 MFMAs on random operands in this run (shader
         # cycles per tick of the constant 100 MHz counter); null with --only, which skips that probe
-        "config": {"workload": res["workload"], "device": props.name, "cus": props.multi_processor_count, "clock_mhz": clock_observed},
+        # settle_ms: every workload is first run untimed for this long, so that the timed steps see the clock of sustained load
+        "config": {"workload": res["workload"], "device": props.name, "cus": props.multi_processor_count, "clock_mhz": clock_observed,
+                   "settle_ms": args.settle_ms},
         "ms_median": round(res["ms_median"], 5), "ms_min": round(res["ms_min"], 5), "ms_max": round(res["ms_max"], 5),
         "roofline": {"bound": res["bound"], "achieved": round(res["achieved"], 3), "peak": res["peak"], "unit": res["unit"],
                      "frac": round(res["frac"], 4), "traffic": load_traffic(args.workload), "kernel": res["kernel"], "kernel_ms": round(res["ms"], 5)},
