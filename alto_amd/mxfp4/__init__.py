@@ -10,7 +10,7 @@ from .linear import (MXFP4LinearFunction, _to_mxfp4_then_scaled_mm, blockwise_mx
 from .ops import register_torch_ops
 from .qdq import _make_qdq_fn_for, quantize_dequantize
 from .quantization import BLOCK_SIZE_DEFAULT, convert_from_mxfp4, convert_to_mxfp4, hadamard_left, quantize_rowcol
-from ._runtime import set_rand_bits_source
+from ._runtime import enable_device_philox_state, set_rand_bits_source
 from .tensor import MXFP4TrainingWeightWrapperTensor, TrainingWeightWrapperBaseTensor, swap_params
 
 __all__ = (
@@ -35,6 +35,7 @@ __all__ = (
     "hadamard_left",
     "transpose_codes",
     "set_rand_bits_source",
+    "enable_device_philox_state",
     "MXFP4TrainingWeightWrapperTensor",
     "TrainingWeightWrapperBaseTensor",
     "swap_params",

@@ -65,6 +65,45 @@ def philox_seed_offset(seed: Optional[int], offset: Optional[int]):
     return int(seed) & (2 ** 64 - 1), int(offset or 0) & (2 ** 64 - 1)
 
 
+# A Philox stream whose (key, counter) pair lives in DEVICE memory: the quantizer reads it there and a one-thread kernel
+# moves the counter on after every use.  Nothing about the random words is then a kernel argument, so a HIP graph that
+# captured a stochastic-rounding quantizer draws fresh words on every replay (a host-side seed would be frozen into it).
+_device_states: dict = {}
+_device_state_on = False
+
+
+def enable_device_philox_state(on: bool = True, seed: Optional[int] = None, device=None) -> None:
+    """Switch the default source of stochastic-rounding words (calls that pass neither ``rand_bits`` nor ``philox_seed``)
+    to a device-resident Philox state.  Call it BEFORE capturing a HIP graph: the state of ``device`` (default: the current
+    one) is created here, with key ``seed`` (default: 63 bits from torch's CPU generator) and counter 0, because creating it
+    copies from the host.  ``on=False`` returns to per-call host seeds and drops the states."""
+    global _device_state_on
+    _device_state_on = bool(on)
+    _device_states.clear()
+    if on:
+        dev = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
+        key, _ = philox_seed_offset(seed, 0)
+        _device_states[dev.index or 0] = torch.tensor([key - (1 << 64) if key >= (1 << 63) else key, 0], dtype=torch.int64, device=dev)
+
+
+def philox_device_state(device: torch.device) -> Optional[torch.Tensor]:
+    """The int64[2] tensor {key, counter} of ``device`` when the device-resident stream is enabled, else None."""
+    if not _device_state_on:
+        return None
+    idx = device.index if device.index is not None else torch.cuda.current_device()
+    st = _device_states.get(idx)
+    if st is None:   # first use on another device: created now (not capturable; enable per device before capturing)
+        key, _ = philox_seed_offset(None, 0)
+        st = _device_states[idx] = torch.tensor([key, 0], dtype=torch.int64, device=torch.device("cuda", idx))
+    return st
+
+
+def philox_advance(state: torch.Tensor, words: int) -> None:
+    """Enqueue the counter update of ``state`` past ``words`` random words on the current stream."""
+    from .._lib import check
+    check(lib().alto_mxfp4_philox_advance(state.data_ptr(), int(words), stream_ptr(state.device)), "alto_mxfp4_philox_advance")
+
+
 def draw_rand_bits(shape, device, seed: Optional[int] = None, offset: Optional[int] = None) -> torch.Tensor:
     """32 random bits per element for stochastic rounding (int32 tensor of ``shape`` on ``device``).
 

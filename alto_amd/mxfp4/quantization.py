@@ -53,7 +53,9 @@ def _quantize_call(x3: torch.Tensor, want_row: bool, want_col: bool, is_2d: bool
     """x3: [B, M, C] with unit stride along C and uniform row / batch strides. Returns the outputs (or None): dense, or
     with ``pad_codes`` code tensors whose rows are padded to whole 128-byte cache lines (for GEMM operands).
     ``philox = (seed, offset)`` with ``use_sr`` and no ``rand3``: the kernel makes the random words itself, element
-    (b, i, j) taking word (b M + i) C + j of the stream ``alto_mxfp4_random_bits(.., seed, offset)`` writes."""
+    (b, i, j) taking word (b M + i) C + j of the stream ``alto_mxfp4_random_bits(.., seed, offset)`` writes.
+    ``philox`` = an int64[2] device tensor {key, counter}: the same, with key and counter read on the device and the
+    counter moved past the B M C words afterwards (nothing about the draw is a kernel argument: safe under graph capture)."""
     B, M, C = x3.shape
     dev = x3.device
     row_codes = row_scales = col_codes = col_scales = None
@@ -72,13 +74,17 @@ def _quantize_call(x3: torch.Tensor, want_row: bool, want_col: bool, is_2d: bool
         bs_r = rand3.stride(0) if B > 1 else M * ld_r
     if use_sr and rand3 is None:
         assert philox is not None, "stochastic rounding needs rand_bits or a Philox (seed, offset)"
+        state = philox if isinstance(philox, torch.Tensor) else None
+        seed, offset = (0, 0) if state is not None else (philox[0] & (2 ** 64 - 1), philox[1] & (2 ** 64 - 1))
         rc = rt.lib().alto_mxfp4_quantize_sr_philox(
             x3.data_ptr(), rt.dtype_code(x3.dtype), B, M, C, ld_x, bs_x,
             rt.ptr(row_codes), rt.ptr(row_scales), rt.ptr(col_codes), rt.ptr(col_scales),
             row_codes.stride(1) if want_row else 0, col_codes.stride(1) if want_col else 0,
-            int(is_2d), philox[0] & (2 ** 64 - 1), philox[1] & (2 ** 64 - 1), None,
+            int(is_2d), seed, offset, rt.ptr(state),
             had, sp, pp, clip, int(use_uos), rt.stream_ptr(dev))
         check(rc, "alto_mxfp4_quantize_sr_philox")
+        if state is not None:
+            rt.philox_advance(state, B * M * C)
         return row_codes, row_scales, col_codes, col_scales
     rc = rt.lib().alto_mxfp4_quantize_pitched(
         x3.data_ptr(), rt.dtype_code(x3.dtype), B, M, C, ld_x, bs_x,
@@ -155,7 +161,9 @@ def convert_to_mxfp4(
     if use_sr:
         if rand_bits is None and ax >= nd - 2 and clip_mode != "dynamic" and data_hp.shape[-1] < 2 ** 26 and rt.philox_in_kernel():
             # the kernel makes the words itself: same bytes as rand_bits = draw_rand_bits(shape, seed, offset), no tensor
-            philox = rt.philox_seed_offset(philox_seed, philox_offset)
+            state = rt.philox_device_state(data_hp.device) if philox_seed is None else None
+            direct = ax == nd - 1 or data_hp.shape[-1] % 8 == 0   # the paths that hand the stream to the kernel
+            philox = state if (state is not None and direct) else rt.philox_seed_offset(philox_seed, philox_offset)
         else:
             if rand_bits is None:
                 rand_bits = rt.draw_rand_bits(data_hp.shape, data_hp.device, philox_seed, philox_offset)
@@ -264,7 +272,10 @@ def quantize_rowcol(
     philox = None
     if use_sr and rand_bits is None:
         if clip_mode != "dynamic" and C < 2 ** 26 and rt.philox_in_kernel():
-            philox = rt.philox_seed_offset(None, None)   # the kernel makes the words: no tensor, no fill launch
+            # the kernel makes the words: no tensor, no fill launch
+            philox = rt.philox_device_state(x.device)
+            if philox is None:
+                philox = rt.philox_seed_offset(None, None)
         else:
             rand_bits = rt.draw_rand_bits(x.shape, x.device)
     if clip_mode == "dynamic":   # the row pair is never clipped; the column pair takes the plain path

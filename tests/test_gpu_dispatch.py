@@ -242,3 +242,45 @@ def test_forward_replays_from_a_hip_graph(m):
         ref = eager if i != 1 else m._to_mxfp4_then_scaled_mm(x * 2, w, False, True, False, False, "none", False)
         assert torch.equal(static_y, ref), f"replay {i}"
         (x.float() @ w.float().T).sum().item()   # unrelated eager work and a host sync between replays
+
+
+def test_captured_stochastic_rounding_draws_fresh_words_on_every_replay(m):
+    """With the device-resident Philox state nothing about the random words is a kernel argument: a captured SR
+    quantizer (fused row + column copies with the Hadamard transform) draws new words on every replay, and every replay
+    equals the eager call keyed with the (key, counter) the state held before it."""
+    import alto_amd.mxfp4._runtime as rt
+    x = randn_outliers((128, 512), torch.bfloat16, seed=63).to(DEV)
+    from tests.helpers import hadamard_from_seed
+    had = m.HadamardTransform(*hadamard_from_seed(5))
+    rt.enable_device_philox_state(True, seed=1234)
+    try:
+        state = rt.philox_device_state(x.device)
+        assert state.tolist() == [1234, 0]
+        static_x = x.clone()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):   # warm-up on the capture stream; it also moves the counter on
+            m.quantize_rowcol(static_x, False, True, hadamard=had)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        words = x.numel()
+        assert state.tolist() == [1234, (words + 3) // 4]
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            outs = m.quantize_rowcol(static_x, False, True, hadamard=had)
+        seen = []
+        for i in range(3):
+            key, counter = state.tolist()
+            assert counter == (i + 1) * ((words + 3) // 4)
+            g.replay()
+            torch.cuda.synchronize()
+            got = [o.clone() for o in outs]
+            bits = rt.draw_rand_bits(x.shape, x.device, key, counter)   # eager twin: the same words as a tensor
+            want = m.quantize_rowcol(x, False, True, hadamard=had, rand_bits=bits)
+            for a, b in zip(got, want):
+                assert torch.equal(a, b), f"replay {i}"
+            seen.append(got[0])
+            (x.float() @ x.float().T).sum().item()
+        assert not torch.equal(seen[0], seen[1]) and not torch.equal(seen[1], seen[2])
+    finally:
+        rt.enable_device_philox_state(False)
