@@ -305,11 +305,23 @@ template <typename OutT>
 __global__ __launch_bounds__(GT_THREADS) void grouped_dw_tiled_kernel(OperandView P, OperandView Q, int64_t NP, int64_t NQ,
                                                                       const int32_t* offs, const int32_t* group_expert, int num_groups,
                                                                       int64_t M_total, OutT* dw, int64_t s_e, int64_t ld, float out_scale,
-                                                                      int tiles_p, int tiles_q) {
+                                                                      int tiles_p, int tiles_q, int xq_log2) {
   extern __shared__ __align__(16) uint8_t smem[];
   const int e = blockIdx.y;
   int tm, tn;
-  if (!grouped_tile_coords(blockIdx.x, tiles_p, tiles_q, tm, tn)) return;
+  {
+    // Each XCD (blockIdx.x % 8) owns one rectangular block of every expert's tile grid, the XCDs forming a
+    // (8 >> xq_log2) x (1 << xq_log2) arrangement: its ~32 resident workgroups then share the P and Q bands of one
+    // expert's token range through its L2, and each band is fetched by few XCDs.
+    const int k = blockIdx.x & 7, j = blockIdx.x >> 3;
+    const int xq = 1 << xq_log2, xp = 8 >> xq_log2;
+    const int bp = (tiles_p + xp - 1) / xp, bq = (tiles_q + xq - 1) / xq;
+    const int p0 = (k >> xq_log2) * bp, q0 = (k & (xq - 1)) * bq;
+    const int np = tiles_p - p0 < bp ? tiles_p - p0 : bp, nq = tiles_q - q0 < bq ? tiles_q - q0 : bq;
+    if (np <= 0 || nq <= 0 || j >= np * nq) return;
+    tm = p0 + j / nq;
+    tn = q0 + j % nq;
+  }
   TileAcc acc;
   gemm_tile_zero(acc);
   const int64_t p_bytes = (NP - 1) * P.ld + M_total / 2, q_bytes = (NQ - 1) * Q.ld + M_total / 2;
@@ -432,8 +444,20 @@ int launch_dw_tiled(const OperandView& P, const OperandView& Q, int64_t NP, int6
   std::call_once(once, [&] { attr_rc = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, GT_DW_LDS_BYTES); });
   if (attr_rc != hipSuccess) return -1;
   const int tiles_p = (int)((NP + GT_TM - 1) / GT_TM), tiles_q = (int)((NQ + GT_TN - 1) / GT_TN);
-  hipLaunchKernelGGL(kern, dim3((unsigned)grouped_grid_size(tiles_p, tiles_q), (unsigned)num_experts), dim3(GT_THREADS), GT_DW_LDS_BYTES, st, P, Q, NP, NQ, offs,
-                     group_expert, num_groups, M_total, (OutT*)dw, s_e, ld, out_scale, tiles_p, tiles_q);
+  // split of the 8 XCDs over the tile grid: the smallest blocks (least idle workgroups), then the smallest perimeter
+  int xq_log2 = 0;
+  int64_t best_area = -1, best_per = 0;
+  for (int l = 0; l < 4; ++l) {
+    const int xq = 1 << l, xp = 8 >> l;
+    const int64_t bp = (tiles_p + xp - 1) / xp, bq = (tiles_q + xq - 1) / xq;
+    if (best_area < 0 || bp * bq < best_area || (bp * bq == best_area && bp + bq < best_per)) {
+      best_area = bp * bq;
+      best_per = bp + bq;
+      xq_log2 = l;
+    }
+  }
+  hipLaunchKernelGGL(kern, dim3((unsigned)(8 * best_area), (unsigned)num_experts), dim3(GT_THREADS), GT_DW_LDS_BYTES, st, P, Q, NP, NQ, offs,
+                     group_expert, num_groups, M_total, (OutT*)dw, s_e, ld, out_scale, tiles_p, tiles_q, xq_log2);
   return 0;
 }
 
