@@ -76,7 +76,9 @@ def enable_device_philox_state(on: bool = True, seed: Optional[int] = None, devi
     """Switch the default source of stochastic-rounding words (calls that pass neither ``rand_bits`` nor ``philox_seed``)
     to a device-resident Philox state.  Call it BEFORE capturing a HIP graph: the state of ``device`` (default: the current
     one) is created here, with key ``seed`` (default: 63 bits from torch's CPU generator) and counter 0, because creating it
-    copies from the host.  ``on=False`` returns to per-call host seeds and drops the states."""
+    copies from the host.  ``on=False`` returns to per-call host seeds and drops the states.  Calls the kernel cannot serve
+    with its own words (``clip_mode="dynamic"``, quantisation axes other than the last two) still fill a tensor from a
+    host-side seed, which a captured graph would repeat."""
     global _device_state_on
     _device_state_on = bool(on)
     _device_states.clear()
