@@ -47,6 +47,30 @@ def test_argument_validation_needs_no_gpu():
     assert rc == -1 and b"permutation" in lib.alto_mxfp4_last_error()
 
 
+def test_argument_validation_of_the_philox_and_grouped_entry_points():
+    """Rejected before any HIP call: dynamic clip with in-kernel random words, a grouped GEMM without (or with too small a)
+    workspace; and the size the workspace query promises."""
+    from alto_amd import _lib
+    lib = _lib.load()
+    buf = ctypes.create_string_buffer(1 << 16)
+    p = ctypes.addressof(buf)
+    p += (-p) % 16
+    rc = lib.alto_mxfp4_quantize_sr_philox(p, 0, 1, 32, 32, 32, 1024, p, p, None, None, 16, 0, 0, 1, 0, None, 0, None, None, 2, 0, None)
+    assert rc == -3 and b"dynamic" in lib.alto_mxfp4_last_error()
+    rc = lib.alto_mxfp4_quantize_sr_philox(None, 0, 1, 32, 32, 32, 1024, p, p, None, None, 16, 0, 0, 1, 0, None, 0, None, None, 0, 0, None)
+    assert rc == -1 and b"NULL" in lib.alto_mxfp4_last_error()
+    M, N, K, E = 512, 256, 512, 2
+    need = lib.alto_mxfp4_grouped_gemm_workspace_bytes(M, E)
+    assert need == 16 + 16 * (M // 256 + E + 2)
+    args = [p, K // 2, p, K // 32, 1, 0, p, N * K // 2, K // 2, p, (N // 32) * (K // 32), K // 32, 1, 1, p, None, E, E, M, N, K, p, 0, N]
+    rc = lib.alto_mxfp4_grouped_gemm(*args, None, 0, None)
+    assert rc == -1 and b"workspace" in lib.alto_mxfp4_last_error()
+    rc = lib.alto_mxfp4_grouped_gemm(*args, p, need - 16, None)
+    assert rc == -1 and b"too small" in lib.alto_mxfp4_last_error()
+    rc = lib.alto_mxfp4_grouped_gemm_dw(None, 0, p, 1, 1, 0, p, 0, p, 1, 1, 0, p, None, E, E, M, N, K, p, 0, N * K, K, 1, 1.0, None)
+    assert rc == -1 and b"NULL" in lib.alto_mxfp4_last_error()
+
+
 def test_ops_refuse_cpu_tensors():
     import alto_amd.mxfp4 as m
     with pytest.raises(RuntimeError, match="no CPU fallback"):
