@@ -236,3 +236,23 @@ def test_weight_cache_is_keyed_by_object_identity():
         assert L.weight_cache_stats()["entries"] == 0, "entries must die with their weight"
     finally:
         L.enable_weight_cache(False)
+
+
+def test_product_never_imports_the_oracle_and_bench_refuses_more_than_one_gpu():
+    """The oracle is the checker: nothing under the package may import it, and bench.py only inside its cpu_sample legs.
+    bench.py measures one GPU and says so when asked for more."""
+    import subprocess
+    import sys
+    pkg = os.path.join(ROOT, "alto_amd")
+    for base, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".h", ".cpp")):
+                text = open(os.path.join(base, f), errors="replace").read()
+                assert not re.search(r"^\s*(import|from)\s+oracle\b", text, flags=re.M), f"{f} imports the oracle"
+    bench = open(os.path.join(ROOT, "bench.py")).read()
+    for m in re.finditer(r"^(\s*)(import|from)\s+oracle\b", bench, flags=re.M):
+        head = bench[:m.start()]
+        last_def = head.rfind("\n    def ")
+        assert last_def >= 0 and head[last_def:].lstrip().startswith("def cpu_sample"), "bench.py imports the oracle outside a cpu_sample leg"
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert r.returncode != 0 and "one GPU" in r.stderr
