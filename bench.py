@@ -644,8 +644,11 @@ def main():
     if "from_idle_ms" in res:   # the same K steps on a device that was idle: the clock is still on its way up
         t = res["from_idle_ms"]
         rate = primary.work / (t * 1e-3) / (1e12 if res["bound"] == "mfma" else 1e9)
-        others[args.workload + "_from_idle"] = {"workload": res["workload"] + ", after 0.5 s without work, no settling calls", "ms": round(t, 4),
-                                                "achieved": round(rate, 2), "unit": res["unit"], "bound": res["bound"], "frac": round(rate / res["peak"], 4)}
+        from_idle = {"workload": res["workload"] + ", after 0.5 s without work, no settling calls", "ms": round(t, 4),
+                     "achieved": round(rate, 2), "unit": res["unit"], "bound": res["bound"], "frac": round(rate / res["peak"], 4)}
+        others[args.workload + "_from_idle"] = from_idle
+    else:
+        from_idle = None
     line = {
         "metric": METRIC,
         "value": round(res["achieved"], 3),
@@ -668,6 +671,8 @@ def main():
         "roofline": {"bound": res["bound"], "achieved": round(res["achieved"], 3), "peak": res["peak"], "unit": res["unit"],
                      "frac": round(res["frac"], 4), "traffic": load_traffic(args.workload), "kernel": res["kernel"], "kernel_ms": round(res["ms"], 5)},
         "cpu_baseline": cpu,
+        # the same steps on a device that had been idle (its clock still rising): beside `value`, never instead of it
+        "from_idle": from_idle,
         "others": others,
     }
     print(json.dumps(line))
