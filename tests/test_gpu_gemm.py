@@ -343,6 +343,33 @@ def test_grouped_many_groups_sorted_runs(m):
     assert bool((wg.grad[3] == 0).all())
 
 
+def test_grouped_ascending_expert_ids_equal_the_offset_form(m):
+    """Per-group expert ids in ascending order (tokens sorted by expert, 128-row groups; experts 1 and 4 unused, the last
+    group carries an id beyond the expert range and must come out as zeros).  The passes are cut differently than for
+    the offsets form (256-row bands cut at expert changes, against tiles that start at each expert's first row), but the
+    result must equal it bit for bit (a row's dot products do not depend on where its tile starts), and the oracle within
+    the GEMM tolerance."""
+    M_total, N, K, E = 3072, 384, 640, 6
+    a, w = _grouped_inputs(M_total, N, K, E, seed=85)
+    sizes = [5, 0, 3, 9, 0, 6]                       # groups of 128 rows per expert; one more group with id 6 (invalid)
+    ids = torch.tensor(sum([[e] * n for e, n in enumerate(sizes)], []) + [E], dtype=torch.int32)
+    assert ids.numel() * 128 == M_total
+    idx = ids.repeat_interleave(128)
+    aq, as_ = m.convert_to_mxfp4(a.to(DEV), axis=-1)
+    wq, ws = m.convert_to_mxfp4(w.to(DEV), axis=-1, is_2d_block=True)
+    out_ids = m.mxfp4_grouped_gemm_forward(aq, wq, idx.to(DEV), as_, ws, trans_weights=True)
+    from alto_amd.mxfp4.grouped_gemm import grouped_forward, groups_from_offsets
+    ends = torch.tensor([0] + sizes, dtype=torch.int32).cumsum(0).to(torch.int32) * 128
+    out_offs = grouped_forward(aq, as_, wq, ws, groups_from_offsets(ends.to(DEV)), False, True, torch.bfloat16)
+    assert torch.equal(out_ids[: ends[-1]], out_offs[: ends[-1]])
+    assert bool((out_ids[ends[-1]:] == 0).all()) and bool((out_offs[ends[-1]:] == 0).all())
+    oq, os_ = O.quantize(a)
+    owq, ows = O.quantize(w, axis=-1, is_2d_block=True)
+    ref = O.grouped_gemm_ref(oq, os_, owq, ows, idx.clamp(max=E - 1))
+    ref[ends[-1]:] = 0
+    assert O.rel_frobenius(out_ids.cpu(), ref) < 4e-3
+
+
 @pytest.mark.parametrize("tiled", [False, True])
 def test_grouped_dw_misaligned_boundaries_are_poisoned(m, tiled):
     """The weight gradient reduces whole MX blocks of 32 tokens per expert.  Offsets that split a block between two
