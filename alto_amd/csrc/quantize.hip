@@ -44,6 +44,7 @@ struct QuantParams {
 __device__ __forceinline__ int packed_byte(const uint32_t (&t)[8], int k) { return (int)((t[k >> 2] >> (8 * (k & 3))) & 0xFFu); }
 
 typedef unsigned short us2_t __attribute__((ext_vector_type(2)));
+typedef float f2_t __attribute__((ext_vector_type(2)));
 typedef unsigned int v4u_t __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ uint32_t pk_max_u16(uint32_t a, uint32_t b) {
@@ -78,7 +79,23 @@ __device__ __forceinline__ float round_to_T(float v) {
   return v;
 }
 
-// SR: 0 = round to nearest even, 1 = stochastic with supplied random words, 2 = stochastic with Philox words made here.
+// SR: 0 = round to nearest even, 1 = stochastic with supplied random words, 2 = stochastic with Philox words made here,
+// 3 = stochastic with the hardware converts v_cvt_scalef32_sr_pk_fp4_{bf16,f32} (one random dword per PAIR of
+// neighbouring elements along the quantisation axis, as the reference's gfx950 path has it,
+// mxfp_quantization.py:133-182), dwords cut from Philox words made here.  What the instruction does with the dword
+// (measured on the instruction itself): the element in the low half is rounded by adding the dword's top bits under
+// the kept mantissa bit and truncating -- bits 31..10 for an fp32 source, bits 31..26 for a bf16 source -- and the
+// element in the high half by the same rule with the dword shifted left by one.  A bf16 pair therefore consumes
+// the top 7 bits of its dword only, and four pairs share one Philox word (pair k of the four gets word << 8 k).
+// Which word belongs to which pair is a function of (batch, row, column) alone:
+//   nb = ceil(M / 32) row bands; row-copy calls R = batch nb C (bf16) or 4 batch nb C (fp32);
+//   row copy, element (b, i, j):  bf16  call ((b nb + i/32) (C/8) + j/8) 8 + i%8, word (i%32)/8, shift 8 ((j%8)/2)
+//                                 fp32  call that * 4 + (i%32)/8,              word (j%8)/2
+//   column copy, rows (2p, 2p+1) of band i/32, column j (after the Hadamard transform, in output row order):
+//                                 bf16  call R + (b nb + i/32) C + j,  word (p%16)/4, shift 8 (p%4)
+//                                 fp32  call R + ((b nb + i/32) C + j) 4 + (p%16)/4,  word p%4
+//   where "call c" is the Philox4x32-10 block with the 128-bit counter offset + c.  A 2D-block quantisation has one
+//   set of codes: its column packing holds the codes of the row copy.
 // Memory is addressed through buffer descriptors that start at the tile (32-bit per-lane offsets, row steps as scalar
 // offsets; an offset with bit 31 set is out of range: such a load returns zeros and such a store is dropped, which is
 // how rows past M and columns past C are masked).
@@ -92,8 +109,15 @@ __global__ __launch_bounds__(256) void quant_kernel(const QuantParams p) {
   // LDS: making them twice would cost more than the occupancy.
   constexpr bool EARLY = DO_COL && SR == 1;
   constexpr bool STASH = DO_COL && SR == 2;
+  constexpr bool HW = SR == 3;
+  constexpr bool XCODES = HW && B2D && DO_COL;   // 2D blocks: the column packing takes the row phase's codes through LDS
   constexpr int OOB = (int)0x80000000;
-  __shared__ __align__(16) T tile[DO_COL ? 32 * TILE_C : 8];
+  // the column phase of the hardware mode brings its transformed values back to row order through a private strip per
+  // thread (17 dwords of bf16 pairs or 33 dwords of fp32: odd pitches, conflict-free), which reuses the tile's memory
+  constexpr int STRIP = BF ? 17 : 33;
+  constexpr int TILE_ELEMS = !DO_COL ? 8 : ((HW && RHT) ? (256 * STRIP * 4 + (int)sizeof(T) - 1) / (int)sizeof(T) : 32 * TILE_C);
+  __shared__ __align__(16) T tile[TILE_ELEMS];
+  __shared__ __align__(8) uint8_t xcodes[XCODES ? 32 * TILE_C : 8];
   __shared__ __align__(16) uint32_t stash[STASH ? 32 * TILE_C : 4];
   __shared__ uint32_t blkmax[8];
   __shared__ uint8_t sperm[32];
@@ -123,18 +147,36 @@ __global__ __launch_bounds__(256) void quant_kernel(const QuantParams p) {
   // Philox: element (b, i, j) consumes word ((b M + i) C + j) of the stream, i.e. word j % 4 of the block with the
   // counter ctr0 + ((b M + i) C + j) / 4.  A lane owns 8 consecutive elements of a row = two blocks.
   uint64_t key = 0, ctr0 = 0, qbase = 0;
-  if constexpr (SR == 2) {
+  if constexpr (SR == 2 || HW) {
     key = p.philox_state ? p.philox_state[0] : p.seed;
     ctr0 = p.philox_state ? p.philox_state[1] : p.ctr0;
     qbase = ctr0 + (((uint64_t)b * (uint64_t)M + (uint64_t)row0) * (uint64_t)C >> 2);
   }
+  const uint64_t band = (uint64_t)b * gridDim.y + blockIdx.y;   // hardware mode: index of this 32-row band
 
   // ------------------------------------------------------------------ row phase
   const int chunk = tid & 31, rsub = tid >> 5;
   const int c = col0 + chunk * 8;
   const bool cok = c < C;
   uint32_t w[4][BF ? 4 : 8];
-  uint32_t rr[4][(SR != 0 && (DO_ROW || STASH)) ? 8 : 1];
+  uint32_t rr[4][((SR == 1 || SR == 2) && (DO_ROW || STASH)) ? 8 : 1];
+  constexpr bool ROW_CODES = DO_ROW || XCODES;   // the row phase encodes (and stores, when DO_ROW)
+  uint32_t hw_row[4][(HW && ROW_CODES) ? (BF ? 1 : 4) : 1];
+  if constexpr (HW && ROW_CODES) {
+    const uint64_t call = (band * (uint64_t)(C >> 3) + (uint64_t)((col0 >> 3) + (tid & 31))) * 8 + (uint64_t)(tid >> 5);
+    if constexpr (BF) {
+      const uint64_t q = ctr0 + call;
+      const uint4 a = philox4x32_10(q, q < ctr0 ? 1ull : 0ull, key);
+      hw_row[0][0] = a.x; hw_row[1][0] = a.y; hw_row[2][0] = a.z; hw_row[3][0] = a.w;
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const uint64_t q = ctr0 + call * 4 + (uint64_t)i;
+        const uint4 a = philox4x32_10(q, q < ctr0 ? 1ull : 0ull, key);
+        hw_row[i][0] = a.x; hw_row[i][1] = a.y; hw_row[i][2] = a.z; hw_row[i][3] = a.w;
+      }
+    }
+  }
   uint32_t amax_i[4];
   bool valid[4];
 #pragma unroll
@@ -206,7 +248,7 @@ __global__ __launch_bounds__(256) void quant_kernel(const QuantParams p) {
   }
   if (B2D || DO_COL) __syncthreads();
 
-  if (DO_ROW || B2D) {
+  if (ROW_CODES || B2D) {
     // descriptors of the row outputs start at the tile's first row
     const __amdgpu_buffer_rsrc_t rsrc_rc = __builtin_amdgcn_make_buffer_rsrc(
         DO_ROW ? p.row_codes + (b * M + row0) * p.ld_rc : nullptr, 0, DO_ROW ? 0x7FFFFFFF : 0, 0x00020000);
@@ -227,7 +269,7 @@ __global__ __launch_bounds__(256) void quant_kernel(const QuantParams p) {
         if (DO_ROW) p.row_scales[(b * (M / 32) + blockIdx.y) * (C / 32) + (c >> 5)] = (uint8_t)s;
         if (DO_COL) p.col_scales[(b * (C / 32) + (c >> 5)) * (M / 32) + blockIdx.y] = (uint8_t)s;
       }
-      if constexpr (DO_ROW) {
+      if constexpr (ROW_CODES) {
       const float scale_f = u2f(s << 23);
       float v[8];
 #pragma unroll
@@ -242,6 +284,18 @@ __global__ __launch_bounds__(256) void quant_kernel(const QuantParams p) {
         out = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(out, v[2], v[3], scale_f, 1);
         out = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(out, v[4], v[5], scale_f, 2);
         out = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(out, v[6], v[7], scale_f, 3);
+      } else if constexpr (HW) {
+        uint32_t by[4];   // byte 0 of each result holds the pair's two codes; the other bytes are not defined
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          if constexpr (BF) {
+            const uint32_t src = (GEN && p.clip_row) ? pack_bf16x2(v[2 * e], v[2 * e + 1]) : w[i][e];
+            by[e] = __builtin_amdgcn_cvt_scalef32_sr_pk_fp4_bf16(0u, __builtin_bit_cast(bf16x2_t, src), hw_row[i][0] << (8 * e), scale_f, 0);
+          } else {
+            by[e] = __builtin_amdgcn_cvt_scalef32_sr_pk_fp4_f32(0u, f2_t{v[2 * e], v[2 * e + 1]}, hw_row[i][e], scale_f, 0);
+          }
+        }
+        out = __builtin_amdgcn_perm(by[1], by[0], 0x0C0C0400u) | __builtin_amdgcn_perm(by[3], by[2], 0x04000C0Cu);
       } else {
         const float inv = u2f((254u - s) << 23);
 #pragma unroll
@@ -251,7 +305,14 @@ __global__ __launch_bounds__(256) void quant_kernel(const QuantParams p) {
           out |= code << (4 * e);
         }
       }
-      __builtin_amdgcn_raw_buffer_store_b32(out, rsrc_rc, valid[i] ? rsub * ldrc + (c >> 1) : OOB, 8 * i * ldrc, 0);
+      if constexpr (DO_ROW) __builtin_amdgcn_raw_buffer_store_b32(out, rsrc_rc, valid[i] ? rsub * ldrc + (c >> 1) : OOB, 8 * i * ldrc, 0);
+      if constexpr (XCODES) {   // one code per byte, in column order, for the column packing
+        const uint32_t ev = out & 0x0F0F0F0Fu, od = (out >> 4) & 0x0F0F0F0Fu;
+        uint2 two;
+        two.x = __builtin_amdgcn_perm(od, ev, 0x05010400u);
+        two.y = __builtin_amdgcn_perm(od, ev, 0x07030602u);
+        *reinterpret_cast<uint2*>(&xcodes[(rsub + 8 * i) * TILE_C + chunk * 8]) = two;
+      }
       }
     }
   }
@@ -318,6 +379,67 @@ __global__ __launch_bounds__(256) void quant_kernel(const QuantParams p) {
     const float scale_f = u2f(s << 23);
     const float inv = u2f((254u - s) << 23);
     uint32_t codes[32];
+    uint32_t out[4];
+    if constexpr (HW && B2D) {
+      // 2D blocks have one set of codes: the row phase left them in LDS, one per byte
+      __syncthreads();
+#pragma unroll
+      for (int k = 0; k < 32; ++k) codes[k] = xcodes[k * TILE_C + tid];
+    } else if constexpr (HW) {
+      // transformed values back to row order (a private strip in LDS undoes the permutation), then one hardware
+      // convert per pair of rows
+      if (GEN && p.clip_col) {
+#pragma unroll
+        for (int k = 0; k < 32; ++k) z[k] = round_to_T<T>(z[k] * 0.75f);
+      }
+      uint32_t* strip = reinterpret_cast<uint32_t*>(tile) + tid * STRIP;
+      const uint64_t nrow = (uint64_t)gridDim.z * gridDim.y * (uint64_t)C;   // calls of the row copy: batch * bands * C
+      uint32_t by[16];
+      if constexpr (BF) {
+        uint32_t pr[16];
+#pragma unroll
+        for (int j = 0; j < 16; ++j) pr[j] = pack_bf16x2(z[2 * j], z[2 * j + 1]);
+        if (RHT) {
+          unsigned short* s16 = reinterpret_cast<unsigned short*>(strip);
+#pragma unroll
+          for (int j = 0; j < 16; ++j) {
+            s16[packed_byte(p.pinv4, 2 * j)] = (unsigned short)pr[j];
+            s16[packed_byte(p.pinv4, 2 * j + 1)] = (unsigned short)(pr[j] >> 16);
+          }
+          asm volatile("" ::: "memory");   // same thread reads what it wrote: LDS ops of one wave complete in order
+#pragma unroll
+          for (int j = 0; j < 16; ++j) pr[j] = strip[j];
+        }
+        const uint64_t q = ctr0 + nrow + band * (uint64_t)C + (uint64_t)cc;
+        const uint4 a = philox4x32_10(q, q < ctr0 ? 1ull : 0ull, key);
+        const uint32_t wd[4] = {a.x, a.y, a.z, a.w};
+#pragma unroll
+        for (int j = 0; j < 16; ++j)
+          by[j] = __builtin_amdgcn_cvt_scalef32_sr_pk_fp4_bf16(0u, __builtin_bit_cast(bf16x2_t, pr[j]), wd[j >> 2] << (8 * (j & 3)), scale_f, 0);
+      } else {
+        if (RHT) {
+          float* sf = reinterpret_cast<float*>(strip);
+#pragma unroll
+          for (int k = 0; k < 32; ++k) sf[packed_byte(p.pinv4, k)] = z[k];
+          asm volatile("" ::: "memory");
+#pragma unroll
+          for (int k = 0; k < 32; ++k) z[k] = sf[k];
+        }
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const uint64_t q = ctr0 + 4 * nrow + (band * (uint64_t)C + (uint64_t)cc) * 4 + (uint64_t)g;
+          const uint4 a = philox4x32_10(q, q < ctr0 ? 1ull : 0ull, key);
+          const uint32_t wd[4] = {a.x, a.y, a.z, a.w};
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            by[4 * g + e] = __builtin_amdgcn_cvt_scalef32_sr_pk_fp4_f32(0u, f2_t{z[8 * g + 2 * e], z[8 * g + 2 * e + 1]}, wd[e], scale_f, 0);
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        out[j] = __builtin_amdgcn_perm(by[4 * j + 1], by[4 * j], 0x0C0C0400u) | __builtin_amdgcn_perm(by[4 * j + 3], by[4 * j + 2], 0x04000C0Cu);
+    }
+    if constexpr (!HW) {
 #pragma unroll
     for (int k = 0; k < 32; ++k) {
       float v = z[k];
@@ -332,8 +454,10 @@ __global__ __launch_bounds__(256) void quant_kernel(const QuantParams p) {
         codes[k] = e2m1_sr_mag(q, r) | ((f2u(q) >> 28) & 8u);
       }
     }
-    uint32_t out[4];
-    if (RHT) {
+    }
+    if constexpr (HW && !B2D) {
+      // out[] is complete
+    } else if (RHT) {
       // undo the permutation: position k belongs to row perm_inv[k]; a private byte scratch in LDS does the indexing
       uint32_t* stage = reinterpret_cast<uint32_t*>(tile);
       uint8_t* sb = reinterpret_cast<uint8_t*>(stage + tid * STAGE_PITCH);
@@ -445,11 +569,13 @@ void dispatch_mode(const QuantParams& p, dim3 grid, hipStream_t st, bool do_row,
 template <typename T>
 void dispatch(const QuantParams& p, dim3 grid, hipStream_t st, bool do_row, bool do_col, bool rht, bool b2d, int sr, bool gen) {
   if (gen) {
-    if (sr == 2) dispatch_mode<T, 2, true>(p, grid, st, do_row, do_col, rht, b2d);
+    if (sr == 3) dispatch_mode<T, 3, true>(p, grid, st, do_row, do_col, rht, b2d);
+    else if (sr == 2) dispatch_mode<T, 2, true>(p, grid, st, do_row, do_col, rht, b2d);
     else if (sr == 1) dispatch_mode<T, 1, true>(p, grid, st, do_row, do_col, rht, b2d);
     else dispatch_mode<T, 0, true>(p, grid, st, do_row, do_col, rht, b2d);
   } else {
-    if (sr == 2) dispatch_mode<T, 2, false>(p, grid, st, do_row, do_col, rht, b2d);
+    if (sr == 3) dispatch_mode<T, 3, false>(p, grid, st, do_row, do_col, rht, b2d);
+    else if (sr == 2) dispatch_mode<T, 2, false>(p, grid, st, do_row, do_col, rht, b2d);
     else if (sr == 1) dispatch_mode<T, 1, false>(p, grid, st, do_row, do_col, rht, b2d);
     else dispatch_mode<T, 0, false>(p, grid, st, do_row, do_col, rht, b2d);
   }
@@ -464,7 +590,8 @@ namespace {
 // one-thread kernel: moves the counter of a device-resident Philox state past the blocks a quantizer call consumed
 __global__ void philox_advance_kernel(uint64_t* state, uint64_t blocks) { state[1] += blocks; }
 
-// sr_mode: 0 round to nearest even, 1 stochastic with the words in rand_bits, 2 stochastic with Philox words made in the kernel
+// sr_mode: 0 round to nearest even, 1 stochastic with the words in rand_bits, 2 stochastic with Philox words made in the kernel,
+// 3 stochastic with the hardware converts (dwords cut from Philox words made in the kernel)
 int quantize_impl(const void* x, int dtype, int64_t batch, int64_t M, int64_t C, int64_t ld_x, int64_t bs_x,
                   uint8_t* row_codes, uint8_t* row_scales, uint8_t* col_codes, uint8_t* col_scales,
                   int64_t ld_row_codes, int64_t ld_col_codes, int is_2d, int sr_mode,
@@ -502,7 +629,7 @@ int quantize_impl(const void* x, int dtype, int64_t batch, int64_t M, int64_t C,
   if (clip_mode == ALTO_CLIP_DYNAMIC) {   // std-based scale: separate plain kernel, quantisation along the contiguous dim
     ALTO_REQUIRE(do_row && !do_col && !hadamard && !use_uos,
                  "quantize: clip_mode=dynamic gives the row output only (no column output, Hadamard or UOS); transpose on the host");
-    if (sr_mode == 2) {
+    if (sr_mode >= 2) {
       set_error("quantize: clip_mode=dynamic takes its random words from a tensor (fill one with alto_mxfp4_random_bits)");
       return ALTO_MXFP4_ENOTIMPL;
     }
@@ -575,6 +702,23 @@ extern "C" int alto_mxfp4_quantize_sr_philox(const void* x, int dtype, int64_t b
   ALTO_REQUIRE((reinterpret_cast<uintptr_t>(philox_state) & 7) == 0, "quantize_sr_philox: philox_state must be 8-byte aligned");
   return quantize_impl(x, dtype, batch, M, C, ld_x, bs_x, row_codes, row_scales, col_codes, col_scales, ld_row_codes, ld_col_codes, is_2d,
                        2, nullptr, 0, 0, seed, offset, philox_state, hadamard, signs, perm, clip_mode, use_uos, stream);
+}
+
+extern "C" int alto_mxfp4_quantize_sr_hw(const void* x, int dtype, int64_t batch, int64_t M, int64_t C, int64_t ld_x, int64_t bs_x,
+                                         uint8_t* row_codes, uint8_t* row_scales, uint8_t* col_codes, uint8_t* col_scales,
+                                         int64_t ld_row_codes, int64_t ld_col_codes, int is_2d,
+                                         uint64_t seed, uint64_t offset, const uint64_t* philox_state,
+                                         int hadamard, const int8_t* signs, const uint8_t* perm,
+                                         int clip_mode, int use_uos, void* stream) {
+  using namespace alto;
+  ALTO_REQUIRE((reinterpret_cast<uintptr_t>(philox_state) & 7) == 0, "quantize_sr_hw: philox_state must be 8-byte aligned");
+  return quantize_impl(x, dtype, batch, M, C, ld_x, bs_x, row_codes, row_scales, col_codes, col_scales, ld_row_codes, ld_col_codes, is_2d,
+                       3, nullptr, 0, 0, seed, offset, philox_state, hadamard, signs, perm, clip_mode, use_uos, stream);
+}
+
+extern "C" int64_t alto_mxfp4_quantize_sr_hw_words(int dtype, int64_t batch, int64_t M, int64_t C) {
+  const int64_t nb = (M + 31) / 32;
+  return 4 * (dtype == ALTO_DT_BF16 ? 2 : 8) * batch * nb * C;
 }
 
 extern "C" int alto_mxfp4_philox_advance(uint64_t* philox_state, uint64_t words, void* stream) {

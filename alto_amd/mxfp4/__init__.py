@@ -10,7 +10,7 @@ from .linear import (MXFP4LinearFunction, _to_mxfp4_then_scaled_mm, blockwise_mx
 from .ops import register_torch_ops
 from .qdq import _make_qdq_fn_for, quantize_dequantize
 from .quantization import BLOCK_SIZE_DEFAULT, convert_from_mxfp4, convert_to_mxfp4, hadamard_left, quantize_rowcol
-from ._runtime import enable_device_philox_state, set_rand_bits_source
+from ._runtime import enable_device_philox_state, set_rand_bits_source, use_hardware_stochastic_rounding
 from .tensor import MXFP4TrainingWeightWrapperTensor, TrainingWeightWrapperBaseTensor, swap_params
 
 __all__ = (
@@ -36,6 +36,7 @@ __all__ = (
     "transpose_codes",
     "set_rand_bits_source",
     "enable_device_philox_state",
+    "use_hardware_stochastic_rounding",
     "MXFP4TrainingWeightWrapperTensor",
     "TrainingWeightWrapperBaseTensor",
     "swap_params",

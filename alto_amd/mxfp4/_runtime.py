@@ -52,6 +52,22 @@ def set_rand_bits_source(fn: Optional[Callable[[torch.Size, torch.device], torch
     _rand_source = fn
 
 
+# The reference picks the gfx950 hardware converts whenever ``use_asm`` is left at None (mxfp_quantization.py:426-427).
+# Here None means the exact software rule unless this switch is on; ``use_asm=True`` / ``False`` always win.
+_hw_rounding_default = False
+
+
+def use_hardware_stochastic_rounding(on: bool = True) -> None:
+    """Make stochastic rounding with ``use_asm=None`` (what the autograd functions pass) use the hardware converts
+    (``v_cvt_scalef32_sr_pk_fp4_*``, one random dword per pair of elements) instead of the software rule."""
+    global _hw_rounding_default
+    _hw_rounding_default = bool(on)
+
+
+def hardware_stochastic_rounding(use_asm: Optional[bool] = None) -> bool:
+    return _hw_rounding_default if use_asm is None else bool(use_asm)
+
+
 def philox_in_kernel() -> bool:
     """True when the quantizer may draw its random words itself (no source installed with ``set_rand_bits_source``)."""
     return _rand_source is None

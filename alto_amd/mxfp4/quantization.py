@@ -49,13 +49,14 @@ def _code_buffer(B: int, R: int, nbytes: int, dev, pad: bool) -> torch.Tensor:
 
 def _quantize_call(x3: torch.Tensor, want_row: bool, want_col: bool, is_2d: bool, use_sr: bool,
                    rand3: Optional[torch.Tensor], hadamard: Optional[HadamardTransform], clip: int, use_uos: bool,
-                   pad_codes: bool = False, philox: Optional[Tuple[int, int]] = None):
+                   pad_codes: bool = False, philox: Optional[Tuple[int, int]] = None, hw_sr: bool = False):
     """x3: [B, M, C] with unit stride along C and uniform row / batch strides. Returns the outputs (or None): dense, or
     with ``pad_codes`` code tensors whose rows are padded to whole 128-byte cache lines (for GEMM operands).
     ``philox = (seed, offset)`` with ``use_sr`` and no ``rand3``: the kernel makes the random words itself, element
     (b, i, j) taking word (b M + i) C + j of the stream ``alto_mxfp4_random_bits(.., seed, offset)`` writes.
     ``philox`` = an int64[2] device tensor {key, counter}: the same, with key and counter read on the device and the
-    counter moved past the B M C words afterwards (nothing about the draw is a kernel argument: safe under graph capture)."""
+    counter moved past the B M C words afterwards (nothing about the draw is a kernel argument: safe under graph capture).
+    ``hw_sr``: round with the hardware's stochastic converts (``alto_mxfp4_quantize_sr_hw``; needs ``philox``)."""
     B, M, C = x3.shape
     dev = x3.device
     row_codes = row_scales = col_codes = col_scales = None
@@ -76,6 +77,17 @@ def _quantize_call(x3: torch.Tensor, want_row: bool, want_col: bool, is_2d: bool
         assert philox is not None, "stochastic rounding needs rand_bits or a Philox (seed, offset)"
         state = philox if isinstance(philox, torch.Tensor) else None
         seed, offset = (0, 0) if state is not None else (philox[0] & (2 ** 64 - 1), philox[1] & (2 ** 64 - 1))
+        if hw_sr:
+            rc = rt.lib().alto_mxfp4_quantize_sr_hw(
+                x3.data_ptr(), rt.dtype_code(x3.dtype), B, M, C, ld_x, bs_x,
+                rt.ptr(row_codes), rt.ptr(row_scales), rt.ptr(col_codes), rt.ptr(col_scales),
+                row_codes.stride(1) if want_row else 0, col_codes.stride(1) if want_col else 0,
+                int(is_2d), seed, offset, rt.ptr(state),
+                had, sp, pp, clip, int(use_uos), rt.stream_ptr(dev))
+            check(rc, "alto_mxfp4_quantize_sr_hw")
+            if state is not None:
+                rt.philox_advance(state, rt.lib().alto_mxfp4_quantize_sr_hw_words(rt.dtype_code(x3.dtype), B, M, C))
+            return row_codes, row_scales, col_codes, col_scales
         rc = rt.lib().alto_mxfp4_quantize_sr_philox(
             x3.data_ptr(), rt.dtype_code(x3.dtype), B, M, C, ld_x, bs_x,
             rt.ptr(row_codes), rt.ptr(row_scales), rt.ptr(col_codes), rt.ptr(col_scales),
@@ -143,8 +155,13 @@ def convert_to_mxfp4(
     the results are computed densely in that orientation and returned transposed back, so ``axis=-2`` on
     ``[M, C]`` yields logical ``[M/2, C]`` codes backed by ``[C][M/2]`` memory.
 
-    ``use_asm`` is accepted for signature compatibility and ignored (there is one implementation).
-    ``use_sr`` consumes ``rand_bits`` (int32/uint32, same shape as ``data_hp``; element ``[i, j]`` uses
+    ``use_asm`` selects the rounding hardware of ``use_sr`` (round-to-nearest always runs on the hardware convert, whose
+    results equal the software rule bit for bit): ``True`` rounds with ``v_cvt_scalef32_sr_pk_fp4_{bf16,f32}``, one random
+    dword per pair of neighbouring elements, cut from the Philox stream ``(philox_seed, philox_offset)`` inside the kernel
+    (mxfp_quantization.py:133-182; ``rand_bits`` cannot be given, ``clip_mode="dynamic"`` is not offered); ``False`` runs
+    the software rule of triton_fp4_ops.py:49-61 with 32 random bits per element; ``None`` (the reference: hardware on
+    gfx950) follows ``use_hardware_stochastic_rounding()``, off by default.
+    ``use_sr`` (software rule) consumes ``rand_bits`` (int32/uint32, same shape as ``data_hp``; element ``[i, j]`` uses
     ``rand_bits[i, j]``); when omitted they come from the library's Philox4x32-10 fill kernel (key and
     counter start ``philox_seed``/``philox_offset`` if given, else a draw from torch's CPU generator).  ``hadamard`` fuses ``hadamard(x, left_mul=True)`` in front of
     an ``axis=-2`` quantisation of a 2D tensor.
@@ -158,7 +175,18 @@ def convert_to_mxfp4(
     nd = data_hp.dim()
     ax = axis % nd
     philox = None
-    if use_sr:
+    hw_sr = bool(use_sr) and rt.hardware_stochastic_rounding(use_asm)
+    if hw_sr and (clip_mode == "dynamic" or rand_bits is not None):
+        # the hardware path has neither; an explicit use_asm=True says so, the session-wide default steps aside
+        if use_asm and clip_mode == "dynamic":
+            raise NotImplementedError("clip_mode='dynamic' with the hardware stochastic rounding is not implemented")
+        if use_asm:
+            raise ValueError("the hardware stochastic rounding draws its random dwords from the Philox stream: pass philox_seed/offset, not rand_bits")
+        hw_sr = False
+    if hw_sr:
+        state = rt.philox_device_state(data_hp.device) if philox_seed is None else None
+        philox = state if state is not None else rt.philox_seed_offset(philox_seed, philox_offset)
+    elif use_sr:
         if rand_bits is None and ax >= nd - 2 and clip_mode != "dynamic" and data_hp.shape[-1] < 2 ** 26 and rt.philox_in_kernel():
             # the kernel makes the words itself: same bytes as rand_bits = draw_rand_bits(shape, seed, offset), no tensor
             state = rt.philox_device_state(data_hp.device) if philox_seed is None else None
@@ -189,7 +217,7 @@ def convert_to_mxfp4(
         if use_sr and philox is None:
             r3 = rand_bits.expand_as(data_hp)
             r3 = _batched_view(r3 if r3.is_contiguous() else r3.contiguous())
-        _, _, cc, cs = _quantize_call(x3, False, True, is_2d_block, use_sr, r3, hadamard, clip, use_uos, philox=philox)
+        _, _, cc, cs = _quantize_call(x3, False, True, is_2d_block, use_sr, r3, hadamard, clip, use_uos, philox=philox, hw_sr=hw_sr)
         lead = data_hp.shape[:-2]
         M, C = data_hp.shape[-2], data_hp.shape[-1]
         codes = cc.reshape(*lead, C, M // 2).transpose(-1, -2)
@@ -199,7 +227,7 @@ def convert_to_mxfp4(
     # general case: move the axis last (view), then quantise along the contiguous dim
     xt = data_hp.transpose(ax, -1)
     shp = xt.shape
-    if philox is not None and ax != nd - 1:   # (only the last-axis case reaches here with Philox; other axes take a tensor)
+    if philox is not None and ax != nd - 1 and not hw_sr:   # (only the last-axis case reaches here with Philox; other axes take a tensor)
         rand_bits = _as_i32(rt.draw_rand_bits(data_hp.shape, data_hp.device, philox[0], philox[1]))
         philox = None
     rtens = rand_bits.transpose(ax, -1) if (use_sr and philox is None) else None
@@ -208,7 +236,7 @@ def convert_to_mxfp4(
         r3 = None
         if use_sr and philox is None:
             r3 = _batched_view(rtens.contiguous())
-        rcodes, rscales, _, _ = _quantize_call(x3, True, False, True, use_sr, r3, None, clip, use_uos, philox=philox)
+        rcodes, rscales, _, _ = _quantize_call(x3, True, False, True, use_sr, r3, None, clip, use_uos, philox=philox, hw_sr=hw_sr)
         codes = rcodes.reshape(*shp[:-1], shp[-1] // 2)
         scales = rscales.reshape(*shp[:-2], shp[-2] // 32, shp[-1] // 32)
     else:
@@ -218,7 +246,7 @@ def convert_to_mxfp4(
         r3 = None
         if use_sr and philox is None:
             r3 = rtens.reshape(-1, shp[-1]).contiguous().unsqueeze(0)
-        rcodes, rscales, _, _ = _quantize_call(x2.unsqueeze(0), True, False, False, use_sr, r3, None, clip, use_uos, philox=philox)
+        rcodes, rscales, _, _ = _quantize_call(x2.unsqueeze(0), True, False, False, use_sr, r3, None, clip, use_uos, philox=philox, hw_sr=hw_sr)
         codes = rcodes.reshape(*shp[:-1], shp[-1] // 2)
         scales = rscales.reshape(*shp[:-1], shp[-1] // 32)
     return codes.transpose(ax, -1), scales.transpose(ax, -1)
@@ -255,6 +283,7 @@ def quantize_rowcol(
     clip_mode: str = "none",
     use_uos: bool = False,
     pad_codes: bool = False,
+    use_asm: Optional[bool] = None,
 ):
     """One pass over a 2D ``x [M, C]`` producing BOTH quantisations the linear layer needs.
 
@@ -270,7 +299,12 @@ def quantize_rowcol(
     torch._check(M % 32 == 0 and C % 32 == 0)
     clip = _clip_code(clip_mode)
     philox = None
-    if use_sr and rand_bits is None:
+    hw_sr = bool(use_sr) and rand_bits is None and clip_mode != "dynamic" and rt.hardware_stochastic_rounding(use_asm)
+    if hw_sr:
+        philox = rt.philox_device_state(x.device)
+        if philox is None:
+            philox = rt.philox_seed_offset(None, None)
+    elif use_sr and rand_bits is None:
         if clip_mode != "dynamic" and C < 2 ** 26 and rt.philox_in_kernel():
             # the kernel makes the words: no tensor, no fill launch
             philox = rt.philox_device_state(x.device)
@@ -289,7 +323,7 @@ def quantize_rowcol(
         assert rand_bits.shape == x.shape
         r3 = _as_i32(rand_bits)
         r3 = _batched_view(r3 if r3.stride(-1) == 1 and r3.stride(0) % 4 == 0 and r3.data_ptr() % 16 == 0 else r3.contiguous())
-    rc, rs, cc, cs = _quantize_call(x3, True, True, is_2d_block, use_sr, r3, hadamard, clip, use_uos, pad_codes, philox=philox)
+    rc, rs, cc, cs = _quantize_call(x3, True, True, is_2d_block, use_sr, r3, hadamard, clip, use_uos, pad_codes, philox=philox, hw_sr=hw_sr)
     return rc[0], rs[0], cc[0].transpose(0, 1), cs[0].transpose(0, 1)
 
 

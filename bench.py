@@ -170,6 +170,20 @@ class FusedGradQuantPhilox(FusedGradQuant):
         raise NotImplementedError("the CPU leg is the supplied-words workload's")
 
 
+class FusedGradQuantHw(FusedGradQuantPhilox):
+    """The same pass with the hardware's stochastic-rounding converts (what the reference runs on gfx950 with use_asm left
+    at its default): one v_cvt_scalef32_sr_pk_fp4_bf16 per pair, dwords cut from Philox words made in the kernel."""
+    name = "cfg2_fused_rht_sr_quantizer[8192x4096], hardware SR converts, random words made in the kernel"
+    kernel = "quant_kernel<bf16, row+col, SR hardware, RHT>"
+
+    def step(self):
+        rt, (rc, rs, cc, cs) = self.rt, self.out
+        code = rt.lib().alto_mxfp4_quantize_sr_hw(self.x.data_ptr(), rt.dtype_code(self.x.dtype), 1, self.M, self.C, self.C, self.M * self.C,
+                                                  rc.data_ptr(), rs.data_ptr(), cc.data_ptr(), cs.data_ptr(), 0, 0, 0, 1234, 0, None,
+                                                  1, self.h.signs.data_ptr(), self.h.perm.data_ptr(), 0, 0, self.stream)
+        assert code == 0, code
+
+
 class RneQuant(Workload):
     """Config 1: bf16 [4096, 4096] ~ N(0,1) with 1% x50 outliers, 1D-32 blocks, RNE, no Hadamard."""
     name = "cfg1_rne_quantizer[4096x4096]"
@@ -401,9 +415,10 @@ class LinearStep(Workload):
     kernel = "gemm"
     M, K, N = 8192, 4096, 14336
 
-    def __init__(self, cached):
+    def __init__(self, cached, hw_sr=False):
         self.cached = cached
-        self.name = f"cfg3+4_linear_fwd_bwd[8192x4096->14336,{'cached' if cached else 'requantized'} weight]"
+        self.hw_sr = hw_sr
+        self.name = f"cfg3+4_linear_fwd_bwd[8192x4096->14336,{'cached' if cached else 'requantized'} weight{', hardware SR converts' if hw_sr else ''}]"
         self.work = 3 * 2.0 * self.M * self.K * self.N
 
     def setup(self, dev, gen):
@@ -420,11 +435,13 @@ class LinearStep(Workload):
     def step(self):
         m = self.m
         m.enable_weight_cache(self.cached)
+        m.use_hardware_stochastic_rounding(self.hw_sr)
         try:   # the random words of the stochastic rounding are drawn inside the step (Philox fill kernel), as in training
             self.x.grad = self.w.grad = None
             y = m.MXFP4LinearFunction.apply(self.x, self.w, False, True, True, False, "none", False, self.h, False)
             y.backward(self.go)
         finally:
+            m.use_hardware_stochastic_rounding(False)
             if not self.cached:
                 m.enable_weight_cache(False)
         return y
@@ -504,6 +521,7 @@ def make_workloads():
                                         "act", "weight"),
         "cfg2_quant": FusedGradQuant(),
         "cfg2_quant_philox": FusedGradQuantPhilox(),
+        "cfg2_quant_hw_sr": FusedGradQuantHw(),
         "cfg1_quant": RneQuant(),
         # config 4: dgrad dX[8192,14336] = dY[8192,4096] . W^T-packed[14336,4096]; wgrad dW[4096,14336] over 8192 tokens
         "cfg4_dgrad": Gemm("cfg4_dgrad_gemm[8192x14336x4096]", 8192, 14336, 4096, False, True, "grad", "weight"),
@@ -514,6 +532,8 @@ def make_workloads():
         "attn_fwd": AttentionFwd(),
         "linear_step": LinearStep(False),
         "linear_step_cached": LinearStep(True),
+        "linear_step_hw_sr": LinearStep(False, hw_sr=True),
+        "linear_step_cached_hw_sr": LinearStep(True, hw_sr=True),
         "copy_calib": CopyCalibration(),
         "mfma_probe_const": MfmaProbe(False),
         "mfma_probe_random": MfmaProbe(True),

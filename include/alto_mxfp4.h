@@ -120,6 +120,36 @@ int alto_mxfp4_quantize_sr_philox(const void* x, int dtype, int64_t batch, int64
                                   int clip_mode, int use_uos, void* stream);
 
 /*
+ * The same quantizer with the stochastic rounding of the gfx950 hardware converts: one v_cvt_scalef32_sr_pk_fp4_bf16
+ * (or _f32) per PAIR of neighbouring elements along the quantisation axis, one random dword per pair.  This is what the
+ * reference runs on gfx950 when use_asm is left at its default (alto/kernels/fp4/mxfp4/mxfp_quantization.py:133-182,
+ * USE_ASM = is_cdna4() at :426-427).  The dwords are cut from the Philox4x32-10 stream (key = seed, 128-bit counter
+ * starting at offset), made inside the kernel.  With nb = ceil(M / 32) and "call c" = the Philox block with counter
+ * offset + c:
+ *   row output, pair (elements 2p, 2p+1) of x[b][i][.], j = 2p:
+ *     bf16: dword = word (i%32)/8 of call ((b nb + i/32) (C/8) + j/8) 8 + i%8, shifted left by 8 ((j%8)/2)
+ *     fp32: dword = word (j%8)/2 of call (((b nb + i/32) (C/8) + j/8) 8 + i%8) 4 + (i%32)/8
+ *   column output, pair (rows 2p, 2p+1 of the transformed matrix) of column j, band i/32 = 2p/32, R = batch nb C:
+ *     bf16: dword = word (p%16)/4 of call R + (b nb + i/32) C + j, shifted left by 8 (p%4)
+ *     fp32: dword = word p%4 of call 4 R + ((b nb + i/32) C + j) 4 + (p%16)/4
+ *   (the instruction reads the top 7 bits of the dword for a bf16 pair and the top 23 for an fp32 pair, so four bf16 pairs
+ *   share one Philox word).  With is_2d both packings hold the codes of the row rule.
+ * A call consumes alto_mxfp4_quantize_sr_hw_words(dtype, batch, M, C) words of the stream whatever outputs it writes.
+ * philox_state as in alto_mxfp4_quantize_sr_philox.  clip_mode = dynamic is not offered here (ALTO_MXFP4_ENOTIMPL).
+ * Results differ from ALTO_ROUND_SR's (the software rule of triton_fp4_ops.py:49-61): the instruction never moves an
+ * exactly representable value and looks at fewer random bits.
+ */
+int alto_mxfp4_quantize_sr_hw(const void* x, int dtype, int64_t batch, int64_t M, int64_t C, int64_t ld_x, int64_t bs_x,
+                              uint8_t* row_codes, uint8_t* row_scales, uint8_t* col_codes, uint8_t* col_scales,
+                              int64_t ld_row_codes, int64_t ld_col_codes, int is_2d,
+                              uint64_t seed, uint64_t offset, const uint64_t* philox_state,
+                              int hadamard, const int8_t* signs, const uint8_t* perm,
+                              int clip_mode, int use_uos, void* stream);
+
+/* Random words one alto_mxfp4_quantize_sr_hw call of these sizes takes from its stream (a multiple of 4). */
+int64_t alto_mxfp4_quantize_sr_hw_words(int dtype, int64_t batch, int64_t M, int64_t C);
+
+/*
  * Moves the counter of a device-resident Philox state {key, counter} past `words` random words (counter += ceil(words / 4)),
  * enqueued on `stream` after the quantizer call that consumed them.  A one-thread kernel; it can be captured together
  * with that call.  No counterpart in the reference (its Philox offsets are host integers).

@@ -1,0 +1,157 @@
+"""GPU parity of the hardware stochastic-rounding mode (``use_asm=True``: v_cvt_scalef32_sr_pk_fp4_*).
+
+Bit parity is against ``oracle/hw_sr.py`` -- a bit model of the instruction pinned by raw outputs of the instruction
+(tests/golden/hw_sr_vectors.npz) plus the Philox addressing of the random dwords -- and the reference's own acceptance
+test of its hardware path is run as well (tests/unittest/mxfp4/test_mxfp_quantization.py:76-82: scales equal, every code
+within one code of the round-to-nearest result).
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle as O
+from oracle import hw_sr as H
+from tests.helpers import assert_bytes_equal, hadamard_from_seed, laplace, randn_outliers
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+SEED, OFFSET = 0x1234_5678_9ABC, 77
+
+
+@pytest.fixture(scope="module")
+def m():
+    import alto_amd.mxfp4 as mod
+    assert torch.cuda.is_available(), "GPU tests need an MI355X"
+    return mod
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("shape", [(128, 64), (96, 544), (96, 520), (3, 64, 256)])
+@pytest.mark.parametrize("axis", [-1, -2])
+@pytest.mark.parametrize("is_2d", [False, True])
+def test_codes_equal_the_instruction_model(m, dtype, shape, axis, is_2d):
+    if shape[-1] % 32 and (is_2d or axis == -1):
+        pytest.skip("520 columns: only a 1D quantisation along the rows exists")
+    x = randn_outliers(shape, dtype, seed=4321)
+    got = m.convert_to_mxfp4(x.to(DEV), axis=axis, is_2d_block=is_2d, use_sr=True, use_asm=True, philox_seed=SEED, philox_offset=OFFSET)
+    x3 = x.reshape(-1, shape[-2], shape[-1])
+    codes, scales = H.quantize_sr_hw(x3, "row" if axis == -1 else "col", is_2d, SEED, OFFSET)
+    lead = shape[:-2]
+    if axis == -1:
+        exp_c, exp_s = codes.reshape(*lead, *codes.shape[1:]), scales.reshape(*lead, *scales.shape[1:])
+    else:   # column output: logical [.., M/2, C] views over [C][M/2] memory
+        exp_c = codes.reshape(*lead, *codes.shape[1:]).transpose(-1, -2)
+        exp_s = scales.reshape(*lead, *scales.shape[1:]).transpose(-1, -2)
+    assert_bytes_equal(got[1], exp_s, "scales")
+    assert_bytes_equal(got[0], exp_c, "codes")
+    # the scales are those of the round-to-nearest oracle, and every code is within one code of it (the reference's test)
+    rne_c, rne_s = O.quantize(x, axis=axis, is_2d_block=is_2d)
+    assert_bytes_equal(got[1], rne_s, "scales vs the software oracle")
+    g, r = got[0].cpu().to(torch.int16), rne_c.to(torch.int16)
+    assert int(((g & 0xF) - (r & 0xF)).abs().max()) <= 1 and int(((g >> 4) - (r >> 4)).abs().max()) <= 1
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("clip_mode,use_uos", [("none", False), ("static", False), ("none", True)])
+@pytest.mark.parametrize("use_perm,C", [(True, 320), (False, 320), (True, 328)])
+def test_fused_row_and_hadamard_column_output(m, lib, dtype, clip_mode, use_uos, use_perm, C):
+    """The pass the backward of the linear layer runs over dY: row codes + transformed column codes, through the C ABI
+    (C = 328 is not a multiple of 32: column output only, last tile ragged)."""
+    M = 160
+    x = laplace((M, C), 1e-3, dtype, seed=5)
+    signs, perm = hadamard_from_seed(1234)
+    if not use_perm:
+        perm = None
+    xd = x.to(DEV)
+    rc = torch.empty((M, C // 2), dtype=torch.uint8, device=DEV)
+    rs = torch.empty((M, C // 32), dtype=torch.uint8, device=DEV) if C % 32 == 0 else None
+    cc = torch.empty((C, M // 2), dtype=torch.uint8, device=DEV); cs = torch.empty((C, M // 32), dtype=torch.uint8, device=DEV)
+    sg = signs.to(torch.int8).contiguous(); pm = None if perm is None else perm.to(torch.uint8).contiguous()
+    clip = {"none": 0, "static": 1}[clip_mode]
+    want_row = rs is not None
+    err = lib.alto_mxfp4_quantize_sr_hw(xd.data_ptr(), 0 if dtype == torch.bfloat16 else 1, 1, M, C, C, M * C,
+                                        rc.data_ptr() if want_row else None, rs.data_ptr() if want_row else None, cc.data_ptr(), cs.data_ptr(), 0, 0, 0,
+                                        SEED, OFFSET, None, 1, sg.data_ptr(), None if pm is None else pm.data_ptr(), clip, int(use_uos),
+                                        torch.cuda.current_stream().cuda_stream)
+    assert err == 0, lib.alto_mxfp4_last_error()
+    torch.cuda.synchronize()
+    ec, es = H.quantize_sr_hw(x[None], "col", False, SEED, OFFSET, signs=signs, perm=perm, clip_mode=clip_mode, use_uos=use_uos)
+    assert_bytes_equal(cs, es[0], "column scales")
+    assert_bytes_equal(cc, ec[0], "column codes")
+    if want_row:
+        er, ers = H.quantize_sr_hw(x[None], "row", False, SEED, OFFSET, use_uos=use_uos)   # the row output of a fused pass is never clipped
+        assert_bytes_equal(rs, ers[0], "row scales")
+        assert_bytes_equal(rc, er[0], "row codes")
+
+
+def test_fused_pass_with_row_output(m):
+    """quantize_rowcol with the hardware rounding: both outputs against the model, seeds taken from torch's generator."""
+    M, C = 256, 512
+    x = laplace((M, C), 1e-3, torch.bfloat16, seed=6)
+    signs, perm = hadamard_from_seed(99)
+    h = m.HadamardTransform(signs, perm)
+    torch.manual_seed(2024)
+    seed = int(torch.randint(0, 2 ** 63 - 1, (1,), dtype=torch.int64).item())
+    torch.manual_seed(2024)
+    rc, rs, cc, cs = m.quantization.quantize_rowcol(x.to(DEV), False, use_sr=True, hadamard=h, use_asm=True)
+    er, ers = H.quantize_sr_hw(x[None], "row", False, seed, 0)
+    ec, ecs = H.quantize_sr_hw(x[None], "col", False, seed, 0, signs=signs, perm=perm)
+    assert_bytes_equal(rs, ers[0], "row scales"); assert_bytes_equal(rc, er[0], "row codes")
+    assert_bytes_equal(cs.transpose(0, 1), ecs[0], "column scales"); assert_bytes_equal(cc.transpose(0, 1), ec[0], "column codes")
+
+
+def test_grid_values_never_move_and_rounding_is_unbiased(m):
+    """Exactly representable inputs come back unchanged; elsewhere the result is one of the two neighbours and the mean
+    over many draws approaches the input (bf16 pairs see 6 random bits: the expectation is exact for bf16 inputs whose
+    fraction of the grid step has 6 bits, which these have)."""
+    grid = torch.tensor([0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0])
+    vals = torch.cat([grid, -grid[1:], torch.tensor([0.625, 1.25, 2.5, 5.0, 0.125, -0.375, 3.5, -4.5])])
+    x = vals.repeat(4096 * 32 // vals.numel() + 1)[: 4096 * 32].reshape(4096, 32).to(torch.bfloat16)
+    x[:, 0] = 6.0   # every block's maximum: scale 1
+    codes, scales = m.convert_to_mxfp4(x.to(DEV), use_sr=True, use_asm=True, philox_seed=5, philox_offset=0)
+    dq = m.convert_from_mxfp4(codes, scales, torch.float32).cpu()
+    xf = x.float()
+    on_grid = (xf.abs().unsqueeze(-1) == grid).any(-1)
+    assert torch.equal(dq[on_grid], xf[on_grid])
+    lo = torch.tensor([0.5, 1.0, 2.0, 4.0, 0.0, -0.5, 3.0, -6.0]); hi = torch.tensor([1.0, 1.5, 3.0, 6.0, 0.5, 0.0, 4.0, -4.0])
+    for v, a, b in zip([0.625, 1.25, 2.5, 5.0, 0.125, -0.375, 3.5, -4.5], lo.tolist(), hi.tolist()):
+        sel = xf == v
+        got = dq[sel]
+        assert bool(((got == a) | (got == b)).all()), v
+        assert abs(float(got.mean()) - v) < 0.05 * (b - a) + 4 * (b - a) / (2 * got.numel() ** 0.5), (v, float(got.mean()), got.numel())
+
+
+def test_explicit_use_asm_rejects_what_the_hardware_path_lacks(m):
+    x = torch.randn(64, 64, device=DEV)
+    with pytest.raises(ValueError):
+        m.convert_to_mxfp4(x, use_sr=True, use_asm=True, rand_bits=torch.zeros(64, 64, dtype=torch.int32, device=DEV))
+    with pytest.raises(NotImplementedError):
+        m.convert_to_mxfp4(x, use_sr=True, use_asm=True, clip_mode="dynamic")
+    # round to nearest is the hardware convert either way: same bytes
+    a = m.convert_to_mxfp4(x, use_asm=True); b = m.convert_to_mxfp4(x, use_asm=False)
+    assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
+
+
+def test_session_default_routes_the_autograd_function(m):
+    """use_hardware_stochastic_rounding(): the linear function's backward quantizes dY with the hardware converts (same
+    scales as the software path, codes within one code of round-to-nearest) and draws from the device-resident stream."""
+    torch.manual_seed(0)
+    x = torch.randn(256, 512, device=DEV, dtype=torch.bfloat16, requires_grad=True)
+    w = (0.02 * torch.randn(384, 512, device=DEV, dtype=torch.bfloat16)).requires_grad_()
+    go = laplace((256, 384), 1e-3, torch.bfloat16, seed=3).to(DEV)
+    h = m.HadamardTransform(*hadamard_from_seed(7))
+    outs = {}
+    for hw in (False, True):
+        m.use_hardware_stochastic_rounding(hw)
+        try:
+            y = m.MXFP4LinearFunction.apply(x, w, False, True, True, False, "none", False, h, False)
+            gx, gw = torch.autograd.grad(y, (x, w), go)
+        finally:
+            m.use_hardware_stochastic_rounding(False)
+        outs[hw] = (gx.float(), gw.float())
+    ref_gx = go.float() @ w.float().detach()
+    ref_gw = go.float().t() @ x.float().detach()
+    for hw in (False, True):
+        gx, gw = outs[hw]
+        assert float((gx - ref_gx).norm() / ref_gx.norm()) < 0.25 and float((gw - ref_gw).norm() / ref_gw.norm()) < 0.25
+    assert not torch.equal(outs[False][0], outs[True][0])
