@@ -22,6 +22,7 @@ c_f32 = ctypes.c_float
 SIGNATURES = {
     "alto_mxfp4_version": (c_int, []),
     "alto_mxfp4_last_error": (ctypes.c_char_p, []),
+    "alto_mxfp4_init": (c_int, []),
     "alto_mxfp4_quantize": (c_int, [c_vp, c_int, c_i64, c_i64, c_i64, c_i64, c_i64,
                                     c_vp, c_vp, c_vp, c_vp,
                                     c_int, c_int, c_vp, c_i64, c_i64,

@@ -232,19 +232,38 @@ __global__ __launch_bounds__(PLAN_THREADS) void grouped_plan_kernel(PassWalk wk,
   const int per = (items + PLAN_THREADS - 1) / PLAN_THREADS;
   const int i0 = t * per, i1 = (i0 + per) < items ? (i0 + per) : items;
   const int Mt = (int)wk.M_total;
-  // row range and expert of item i of the sorted form
-  auto item = [&](int i, int& lo, int& hi, int& e) {
-    if (i == 0) { lo = 0; hi = wk.off_at(0); e = -1; }
-    else if (i == wk.num_groups + 1) { lo = wk.off_at(wk.num_groups); hi = Mt; e = -1; }
-    else { lo = wk.off_at(i - 1); hi = wk.off_at(i); e = (i - 1) < wk.num_experts ? i - 1 : -1; }
-    if (i > 0 && lo < wk.off_at(0)) lo = wk.off_at(0);   // offsets that go backwards never make two passes own a row
-    if (hi < lo) hi = lo;
+  // Sorted form: item i ends at E(i) = offs[i] (head: offs[0]; tail: M_total) and starts at the running maximum of the
+  // ends before it, so the items tile [0, M_total) without overlap whatever the offsets are: a group whose end lies
+  // below an earlier end is empty, one that starts below it is cut (the fallback kernel's row search does the same).
+  auto item_end = [&](int i) { return i == wk.num_groups + 1 ? Mt : wk.off_at(i); };
+  int start = 0;   // running maximum of the ends before item i0
+  if (sorted) {
+    int lm = 0;
+    for (int i = i0; i < i1; ++i) { const int v = item_end(i); lm = v > lm ? v : lm; }
+    scan[t] = lm;
+    __syncthreads();
+    for (int d = 1; d < PLAN_THREADS; d <<= 1) {   // inclusive max scan
+      const int v = t >= d ? scan[t - d] : 0;
+      __syncthreads();
+      scan[t] = v > scan[t] ? v : scan[t];
+      __syncthreads();
+    }
+    start = t > 0 ? scan[t - 1] : 0;
+    __syncthreads();
+  }
+  auto item = [&](int i, int& run, int& lo, int& hi, int& e) {   // `run` carries the running maximum along the thread's items
+    e = (i >= 1 && i <= wk.num_groups && (i - 1) < wk.num_experts) ? i - 1 : -1;
+    lo = run;
+    const int end = item_end(i);
+    hi = end > lo ? end : lo;
+    run = hi;
   };
   auto walk = [&](auto&& emit) {
+    int run = start;
     for (int i = i0; i < i1; ++i) {
       if (sorted) {
         int lo, hi, e;
-        item(i, lo, hi, e);
+        item(i, run, lo, hi, e);
         for (int r = lo; r < hi; r += GT_TM) emit(r, r, r + GT_TM < hi ? r + GT_TM : hi, e);
       } else {
         wk.band(i, [&](int lo, int hi, int e) { emit(i * GT_TM, lo, hi, e); });
@@ -574,6 +593,12 @@ int scratch_of_current_device(void** out) {
 }
 }  // namespace
 }  // namespace alto
+
+extern "C" int alto_mxfp4_init(void) {
+  using namespace alto;
+  void* p = nullptr;
+  return scratch_of_current_device(&p);
+}
 
 extern "C" int alto_mxfp4_grouped_gemm_noalloc(const uint8_t* a, int64_t lda, const uint8_t* a_scales, int64_t a_ss_r, int64_t a_ss_k, int a_is_2d,
                                                const uint8_t* w, int64_t w_stride_e, int64_t ldw,

@@ -322,6 +322,7 @@ __global__ __launch_bounds__(256) void quant_kernel(const QuantParams p) {
     const int cc = col0 + tid;
     const bool cvalid = cc < C;
     float z[32];
+    uint32_t zp[(BF && RHT) ? 16 : 1];   // the transformed column as packed bf16 pairs
 #pragma unroll
     for (int k = 0; k < 32; ++k) {
       if (BF) z[k] = u2f((uint32_t)reinterpret_cast<const unsigned short*>(tile)[k * TILE_C + tid] << 16);
@@ -342,6 +343,8 @@ __global__ __launch_bounds__(256) void quant_kernel(const QuantParams p) {
       }
       // z * (+-1) / float32(sqrt(32)), correctly rounded: quotient estimate, one FMA correction, both with the sign
       // folded into the (wave-uniform) constants; the sign bit is taken from the estimate so that -0 stays -0.
+      // (Taking the block's absmax before the division and dropping the guard for columns without an infinity was
+      // measured: the second copy of the loop costs more than the 32 guards save.)
 #pragma unroll
       for (int k = 0; k < 32; ++k) {
         const uint32_t flip = ((p.sign_mask >> k) & 1u) << 31;   // scalar: the constants stay in scalar registers
@@ -355,9 +358,9 @@ __global__ __launch_bounds__(256) void quant_kernel(const QuantParams p) {
       if constexpr (BF) {   // round to bf16 two at a time
 #pragma unroll
         for (int k = 0; k < 32; k += 2) {
-          const uint32_t w2 = pack_bf16x2(z[k], z[k + 1]);
-          z[k] = u2f(w2 << 16);
-          z[k + 1] = u2f(w2 & 0xFFFF0000u);
+          zp[k >> 1] = pack_bf16x2(z[k], z[k + 1]);   // the hardware convert takes the packed pairs as they are
+          z[k] = u2f(zp[k >> 1] << 16);
+          z[k + 1] = u2f(zp[k >> 1] & 0xFFFF0000u);
         }
       }
     }
@@ -398,7 +401,7 @@ __global__ __launch_bounds__(256) void quant_kernel(const QuantParams p) {
       if constexpr (BF) {
         uint32_t pr[16];
 #pragma unroll
-        for (int j = 0; j < 16; ++j) pr[j] = pack_bf16x2(z[2 * j], z[2 * j + 1]);
+        for (int j = 0; j < 16; ++j) pr[j] = (RHT && !(GEN && p.clip_col)) ? zp[RHT ? j : 0] : pack_bf16x2(z[2 * j], z[2 * j + 1]);
         if (RHT) {
           unsigned short* s16 = reinterpret_cast<unsigned short*>(strip);
 #pragma unroll

@@ -4,6 +4,8 @@ from __future__ import annotations
 from dataclasses import dataclass
 from typing import Literal
 
+import torch
+
 
 @dataclass(unsafe_hash=True, kw_only=True, slots=True)
 class TrainingOpConfig:
@@ -22,3 +24,6 @@ class TrainingOpConfig:
             raise ValueError(f"this build implements precision='mxfp4' only, got {self.precision!r}")
         if self.clip_mode not in ("none", "static", "dynamic"):
             raise ValueError(f"Invalid clip mode: {self.clip_mode}")
+
+
+torch.serialization.add_safe_globals([TrainingOpConfig])   # dispatch/config.py:57

@@ -183,6 +183,7 @@ class MXFP4GroupedGEMM(torch.autograd.Function):
                 hadamard_transform: Optional[HadamardTransform] = None, use_uos: bool = False, offsets: Optional[torch.Tensor] = None):
         assert not use_macro_block_scaling, "Macro block scaling is not supported in real MXFP4 kernels"
         original_dtype = inputs.dtype
+        weights_owner = expert_weights   # the object the caller keeps: cache entries belong to it, not to the alias below
         expert_weights = unwrap_weight_wrapper(expert_weights)
         E = expert_weights.shape[0]
         M_buf = inputs.shape[0]
@@ -202,9 +203,9 @@ class MXFP4GroupedGEMM(torch.autograd.Function):
         # weights: codes packed along K [E, N, K/2] for the forward, packed along N [E, K, N/2] for dX
         w = expert_weights if trans_weights else expert_weights.transpose(1, 2)   # logical [E, N, K]
         if w.stride(2) == 1:
-            wq_nk, ws_nk, wq_kn, ws_kn = _quantize_experts(expert_weights, w, use_2dblock_w, use_uos)
+            wq_nk, ws_nk, wq_kn, ws_kn = _quantize_experts(weights_owner, w, use_2dblock_w, use_uos)
         else:                                                                     # stored [E, K, N]: same pass, roles swapped
-            wq_kn, ws_kn, wq_nk, ws_nk = _quantize_experts(expert_weights, w.transpose(1, 2), use_2dblock_w, use_uos)
+            wq_kn, ws_kn, wq_nk, ws_nk = _quantize_experts(weights_owner, w.transpose(1, 2), use_2dblock_w, use_uos)
         out = grouped_forward(a_q, a_s, wq_nk, ws_nk, groups, use_2dblock_x, use_2dblock_w, original_dtype)
         ctx.save_for_backward(a_qm, a_sm, wq_kn, ws_kn, groups.offs, groups.expert)
         ctx.num_groups = groups.n

@@ -62,7 +62,8 @@ def cached_weight_quantisation(weight: torch.Tensor, tag, make):
     if not _WEIGHT_CACHE_ENABLED:
         return make()
     key = (id(weight), tag)
-    stamp = (weight._version, weight.data_ptr(), tuple(weight.shape), tuple(weight.stride()), weight.dtype, weight.device)
+    inner = getattr(weight, "_data", weight)   # a wrapper subclass keeps the tensor that in-place updates touch in _data
+    stamp = (inner._version, inner.data_ptr(), tuple(inner.shape), tuple(inner.stride()), inner.dtype, inner.device)
     hit = _WEIGHT_CACHE.get(key)
     if hit is not None and hit[0]() is weight and hit[1] == stamp:
         _WEIGHT_CACHE_STATS["hits"] += 1
@@ -75,9 +76,13 @@ def cached_weight_quantisation(weight: torch.Tensor, tag, make):
     return out
 
 
-def _quantize_weight_2d(weight: torch.Tensor, use_uos: bool):
-    """(w_q, w_s, w_qt, w_st) of a 2D-block quantisation, from the cache when the weight is unchanged."""
-    return cached_weight_quantisation(weight, ("linear2d", bool(use_uos)), lambda: quantize_rowcol(weight, True, use_uos=use_uos, pad_codes=True))
+def _quantize_weight_2d(weight: torch.Tensor, use_uos: bool, owner: Optional[torch.Tensor] = None):
+    """(w_q, w_s, w_qt, w_st) of a 2D-block quantisation, from the cache when the weight is unchanged.  ``owner`` is the
+    object the CALLER keeps alive (the ``nn.Parameter`` or wrapper tensor): ``weight`` itself may be a plain-tensor alias
+    made for this call only (``unwrap_weight_wrapper`` of a Parameter is a new object every time), on which an entry
+    would never be found again.  The alias shares the owner's storage and version counter."""
+    return cached_weight_quantisation(weight if owner is None else owner, ("linear2d", bool(use_uos)),
+                                      lambda: quantize_rowcol(weight, True, use_uos=use_uos, pad_codes=True))
 
 
 def transpose_codes(codes: torch.Tensor) -> torch.Tensor:
@@ -193,6 +198,7 @@ class MXFP4LinearFunction(torch.autograd.Function):
     def forward(ctx, x, weight, use_2dblock_x, use_2dblock_w, use_sr_grad, use_dge, clip_mode,
                 use_macro_block_scaling, hadamard_transform: Optional[HadamardTransform] = None, use_uos: bool = False):
         assert not use_macro_block_scaling, "Macro block scaling is not supported in real MXFP4 kernels"
+        weight_owner = weight
         weight = unwrap_weight_wrapper(weight)
         original_shape = x.shape
         original_dtype = x.dtype
@@ -210,7 +216,7 @@ class MXFP4LinearFunction(torch.autograd.Function):
                 x_qm, x_sm = convert_to_mxfp4(x2, axis=0, clip_mode=clip_mode, use_uos=use_uos, hadamard=hadamard_transform)
 
         if use_2dblock_w:
-            w_q, w_s, w_qt, w_st = _quantize_weight_2d(weight, use_uos)
+            w_q, w_s, w_qt, w_st = _quantize_weight_2d(weight, use_uos, owner=weight_owner)
             # [N/2, K] view over [K][N/2] memory; scales [N/32, K/32] as a view over [K/32][N/32] memory (same values as
             # w_s, stored so that the dgrad GEMM reads them with unit stride along its reduction dim N)
             w_bwd, w_bwd_s = w_qt, w_st

@@ -184,3 +184,7 @@ def swap_params(module: nn.Module, *, module_filter_fn: Optional[Callable[[nn.Mo
 
     visit(module, "")
     return module
+
+
+# checkpoints written with wrapped weights load under torch.load(weights_only=True) (dispatch/tensor.py:499-503)
+torch.serialization.add_safe_globals([MXFP4TrainingWeightWrapperTensor])

@@ -237,8 +237,18 @@ int alto_mxfp4_grouped_gemm(const uint8_t* a, int64_t lda, const uint8_t* a_scal
  * the call allocates nothing; it serves M_total / 256 + num_groups + 2 <= 65535 and rejects larger problems with
  * ALTO_MXFP4_EINVAL.  Every call on a GPU shares that GPU's array: calls that overlap in time on one GPU (two streams,
  * two host threads) race on it and must use alto_mxfp4_grouped_gemm with separate workspaces instead.  Same results as
- * alto_mxfp4_grouped_gemm, bit for bit.
+ * alto_mxfp4_grouped_gemm, bit for bit.  The array used is that of the CURRENT device, which must be the device `stream`
+ * belongs to.  Its address is looked up on the first use on a device (a runtime query that may load the code object):
+ * call alto_mxfp4_init() on every device beforehand when the first call would otherwise fall inside a stream capture.
  */
+/*
+ * Per-device set-up that the entry points otherwise do on first use: resolves, for the CURRENT device, the address of the
+ * library's built-in pass-list array.  Call it once per device (with that device current) before capturing a HIP graph
+ * that contains alto_mxfp4_grouped_gemm_noalloc.  Idempotent, thread-safe, allocates nothing.  No counterpart in the
+ * reference.
+ */
+int alto_mxfp4_init(void);
+
 int alto_mxfp4_grouped_gemm_noalloc(const uint8_t* a, int64_t lda, const uint8_t* a_scales, int64_t a_ss_r, int64_t a_ss_k, int a_is_2d,
                                     const uint8_t* w, int64_t w_stride_e, int64_t ldw,
                                     const uint8_t* w_scales, int64_t ws_stride_e, int64_t ws_r, int64_t ws_k, int w_is_2d,

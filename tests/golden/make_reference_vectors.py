@@ -53,6 +53,24 @@ def main():
         dq = ref_utils.convert_from_mxfp4_pytorch(q, s, output_dtype=torch.float32, clip_mode="dynamic", **kw)
         out[f"dyn_{name}_dq"] = dq.contiguous().numpy().copy()
 
+    # ---- the twin's other modes (clip none / static, the UOS scale rule), bf16 and fp32: they pin the scale rule, the
+    # round-to-nearest encode and the packing by bytes the reference wrote, beside the closed-form pins of the oracle.
+    # The twin rounds to nearest only (no stochastic rounding), so these are RNE vectors.
+    xt = randn_outliers((64, 128), torch.float32, seed=503)
+    xt[5, 32:64] = 0.0
+    xt[6, :32] = torch.tensor([6.0, -6.0, 5.0, 7.0] * 8)         # at and around the top of the grid
+    xt[7, :32] = 2.0 ** -130                                     # below the smallest scale
+    for dt_name, dt in (("f32", torch.float32), ("bf16", torch.bfloat16)):
+        xx = xt.to(dt)
+        out[f"twin_{dt_name}_x"] = xx.numpy().copy() if dt == torch.float32 else bits16(xx)
+        for mode, mkw in (("none", dict(clip_mode="none")), ("static", dict(clip_mode="static")), ("uos", dict(clip_mode="none", use_uos=True))):
+            for name, kw in (("row", dict(axis=-1)), ("col", dict(axis=-2)), ("2d", dict(axis=-1, is_2d_block=True))):
+                q, s = ref_utils.convert_to_mxfp4_pytorch(xx, **mkw, **kw)
+                out[f"twin_{dt_name}_{mode}_{name}_codes"] = q.contiguous().numpy().copy()
+                out[f"twin_{dt_name}_{mode}_{name}_scales"] = s.contiguous().numpy().copy()
+                dq = ref_utils.convert_from_mxfp4_pytorch(q, s, output_dtype=dt, clip_mode=mkw["clip_mode"], **kw)
+                out[f"twin_{dt_name}_{mode}_{name}_dq"] = dq.contiguous().numpy().copy() if dt == torch.float32 else bits16(dq.contiguous())
+
     # ---- attention: grouped-query heads, a partial last key block, head dims 64 and 128, non-causal with Sq != Sk.
     # (Causal cases keep Sq = Sk: the CPU model ends its key loop at the unshifted query end, test_mxfp_pnq.py:125, which
     # departs from the kernel's bottom-right aligned mask, triton_flash_attention_mxfp4.py:286-294, when Sq != Sk.)

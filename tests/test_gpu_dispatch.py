@@ -107,9 +107,12 @@ def test_fused_qdq_equals_quantize_then_dequantize(m, dtype, is_2d, use_uos):
     assert got.shape == (100, 256) and torch.equal(got.cpu(), exp)
 
 
-def test_weight_cache_reuses_until_weight_changes(m):
+@pytest.mark.parametrize("as_parameter", [False, True])
+def test_weight_cache_reuses_until_weight_changes(m, as_parameter):
     x = randn_outliers((64, 256), torch.bfloat16, seed=13).to(DEV)
     w = (randn_outliers((128, 256), torch.bfloat16, seed=14) * 0.02).to(DEV).requires_grad_(True)
+    if as_parameter:   # what a module holds: the kernels see a fresh plain-tensor alias of it in every forward
+        w = torch.nn.Parameter(w.detach())
     args = (False, True, False, False, "none", False)
     y0 = m._to_mxfp4_then_scaled_mm(x, w, *args)
     m.enable_weight_cache(True)

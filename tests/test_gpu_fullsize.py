@@ -142,13 +142,17 @@ def test_cfg4_backward_full_size(m):
     go_q, go_s, go_qm, go_sm = m.quantize_rowcol(go, False, use_sr=True, rand_bits=r, hadamard=h)
     _, _, x_qm, x_sm = m.quantize_rowcol(xd, False, hadamard=h)
     w_q, w_s, w_qt, w_st = m.quantize_rowcol(wd, True)
-    # quantizer outputs of sampled token bands, bit for bit: row copy (SR, no transform) and Hadamard column copy (SR)
-    for r0 in _bands(M, 4):
-        gb, rb = go[r0:r0 + 256].cpu(), r[r0:r0 + 256].cpu()
+    # the whole of dY, bit for bit: row copy (SR, no transform) and Hadamard column copy (SR), in slabs of 1024 tokens
+    go_c, r_c = go.cpu(), r.cpu()
+    gq_c, gs_c, gqm_c, gsm_c = go_q.cpu(), go_s.cpu(), go_qm.cpu(), go_sm.cpu()
+    for r0 in range(0, M, 1024):
+        gb, rb = go_c[r0:r0 + 1024], r_c[r0:r0 + 1024]
         eq, es = O.quantize(gb, use_sr=True, rand_bits=rb)
-        assert torch.equal(go_q[r0:r0 + 256].cpu(), eq) and torch.equal(go_s[r0:r0 + 256].cpu(), es), f"dY rows {r0}"
+        assert torch.equal(gq_c[r0:r0 + 1024], eq) and torch.equal(gs_c[r0:r0 + 1024], es), f"dY rows {r0}"
         eq, es = O.quantize(O.rht_left(gb, signs, perm), axis=0, use_sr=True, rand_bits=rb)
-        assert torch.equal(go_qm[r0 // 2:r0 // 2 + 128].cpu(), eq) and torch.equal(go_sm[r0 // 32:r0 // 32 + 8].cpu(), es), f"H.dY rows {r0}"
+        assert torch.equal(gqm_c[r0 // 2:r0 // 2 + 512], eq) and torch.equal(gsm_c[r0 // 32:r0 // 32 + 32], es), f"H.dY rows {r0}"
+    # the saved activation operand (K = 14336 columns) on sampled token bands
+    for r0 in _bands(M, 4):
         eq, es = O.quantize(O.rht_left(xd[r0:r0 + 256].cpu(), signs, perm), axis=0)
         assert torch.equal(x_qm[r0 // 2:r0 // 2 + 128].cpu(), eq) and torch.equal(x_sm[r0 // 32:r0 // 32 + 8].cpu(), es), f"H.x rows {r0}"
 

@@ -149,6 +149,54 @@ def test_linear_autograd(m, shape, use_2dblock_x, use_2dblock_w, use_sr, use_h, 
     _linear_autograd_case(m, shape, use_2dblock_x, use_2dblock_w, use_sr, use_h, clip_mode, dtype, use_uos, floors=not use_uos)
 
 
+def test_autograd_with_words_made_in_the_kernel(m):
+    """The default backward path: no source of explicit words installed, the quantizer of dY draws its words itself from
+    the device-resident Philox stream.  The words are rebuilt from (key, counter) and the gradients compared with the
+    oracle's flow on those words -- once for the linear function, once for the grouped one."""
+    from alto_amd.mxfp4 import _runtime as rt
+    signs, perm = hadamard_from_seed(1234)
+    SEED = 0x5EED5EED
+    # ---- linear
+    Mr, N, K = 256, 384, 512
+    x = randn_outliers((Mr, K), torch.bfloat16, seed=1)
+    w = randn_outliers((N, K), torch.bfloat16, seed=2)
+    go = randn_outliers((Mr, N), torch.bfloat16, seed=3) / (Mr * N)
+    m.enable_device_philox_state(True, seed=SEED)
+    try:
+        assert rt.philox_in_kernel()
+        xg, wg = x.to(DEV).requires_grad_(True), w.to(DEV).requires_grad_(True)
+        y = m.MXFP4LinearFunction.apply(xg, wg, False, True, True, False, "none", False, m.HadamardTransform(signs, perm), False)
+        y.backward(go.to(DEV))
+        st = rt.philox_device_state(torch.device(DEV)).cpu()
+        assert int(st[1]) == Mr * N // 4, "the counter moved past one word per element of dY"
+        r = rt.draw_rand_bits((Mr, N), torch.device(DEV), seed=SEED, offset=0).cpu()
+    finally:
+        m.enable_device_philox_state(False)
+    y_ref, saved = O.linear_forward_ref(x, w, False, True, hadamard=(signs, perm))
+    dx_ref, dw_ref = O.linear_backward_ref(go, saved, False, True, use_sr_grad=True, rand_bits=r, hadamard=(signs, perm))
+    assert O.rel_frobenius(xg.grad.cpu(), dx_ref) < TOL[torch.bfloat16] and O.rel_frobenius(wg.grad.cpu(), dw_ref) < TOL[torch.bfloat16]
+    # ---- grouped (reference contract: one expert id per 128 rows)
+    E, Ng, Kg, Mt = 4, 256, 256, 1024
+    a, wts = _grouped_inputs(Mt, Ng, Kg, E, seed=70)
+    idx = torch.randint(0, E, (Mt // 128,), generator=torch.Generator().manual_seed(71), dtype=torch.int32).repeat_interleave(128)
+    gog = randn_outliers((Mt, Ng), torch.bfloat16, seed=72) / (Mt * Ng)
+    m.enable_device_philox_state(True, seed=SEED + 1)
+    m.HadamardFactory.configure(seed=1234)
+    try:
+        ag, wgg = a.to(DEV).requires_grad_(True), wts.to(DEV).requires_grad_(True)
+        out = m.mxfp4_grouped_gemm(ag, wgg, idx.to(DEV), use_sr_grad=True, use_hadamard=True)
+        out.backward(gog.to(DEV))
+        r = rt.draw_rand_bits((Mt, Ng), torch.device(DEV), seed=SEED + 1, offset=0).cpu()
+    finally:
+        m.enable_device_philox_state(False)
+    wq, ws = O.quantize(wts, axis=-1, is_2d_block=True)
+    gq, gs = O.quantize(gog, use_sr=True, rand_bits=r)
+    assert O.rel_frobenius(ag.grad.cpu(), O.grouped_gemm_dx_ref(gq, gs, wq, ws, idx, k_pack_w=False)) < 4e-3
+    gqm, gsm = O.quantize(O.rht_left(gog, signs, perm), axis=0, use_sr=True, rand_bits=r)
+    aqm, asm = O.quantize(O.rht_left(a, signs, perm), axis=0)
+    assert O.rel_frobenius(wgg.grad.cpu(), O.grouped_gemm_dw_ref(gqm, gsm, aqm, asm, idx, E)) < 4e-3
+
+
 @pytest.mark.parametrize("use_2dblock_x,use_2dblock_w", [(False, True), (False, False), (True, True), (True, False)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 def test_linear_autograd_large_shape(m, use_2dblock_x, use_2dblock_w, dtype):
@@ -294,6 +342,24 @@ def test_grouped_unaligned_rows_forward(m):
     ref = O.grouped_gemm_ref(aq, as_, wq, ws, idx)
     assert O.rel_frobenius(out.cpu(), ref) < 1e-5
     assert bool((out[201:] == 0).all())
+
+
+def test_grouped_offsets_that_go_backwards_never_share_a_row(m):
+    """Malformed offsets (not monotonic): a group starts at the running maximum of the ends before it, so every row is
+    written by exactly one expert (or zero-filled) -- offsets [0, 1000, 500, 2000] give expert 0 rows [0, 1000), expert 1
+    nothing, expert 2 rows [1000, 2000).  Same rule on the tiled and on the direct kernel."""
+    from alto_amd.mxfp4 import grouped_gemm as G
+    for (M_buf, N, K, offs_l) in [(2304, 512, 512, [0, 1000, 500, 2000]), (224, 64, 128, [0, 100, 50, 200])]:
+        E = 3
+        a, w = _grouped_inputs(M_buf, N, K, E, seed=61)
+        aq, as_ = O.quantize(a)
+        wq, ws = O.quantize(w, axis=-1, is_2d_block=True)
+        offs = torch.tensor(offs_l, dtype=torch.int32)
+        out = G.grouped_forward(*dev(aq, as_, wq, ws), G.groups_from_offsets(offs.to(DEV)), False, True, torch.float32)
+        fixed = torch.tensor([offs_l[0], offs_l[1], offs_l[1], offs_l[3]], dtype=torch.int32)   # what the running maximum makes of them
+        ref = O.grouped_gemm_ref(aq, as_, wq, ws, O.indices_from_offsets(fixed[1:]))
+        assert O.rel_frobenius(out[:offs_l[3]].cpu(), ref[:offs_l[3]]) < 1e-5, (M_buf, N, K)
+        assert bool((out[offs_l[3]:] == 0).all())
 
 
 def test_grouped_small_problem_direct_kernels(m):

@@ -181,13 +181,14 @@ def test_config2_fused_gradient_quantizer_full_size(m):
     rq, rs, cq, cs = m.quantize_rowcol(x.to(DEV), False, use_sr=True, rand_bits=r.to(DEV), hadamard=h)
     assert rq.shape == (M, C // 2) and rs.shape == (M, C // 32)
     assert cq.shape == (M // 2, C) and cq.stride() == (1, M // 2) and cs.shape == (M // 32, C) and cs.stride() == (1, M // 32)
-    # oracle on a spread of 32-row blocks (quantisation is local to a block row, so slices compare exactly)
-    for b0 in [0, 37, 100, 255]:
-        sl = slice(32 * b0, 32 * (b0 + 4))
+    # the whole tensor, both copies, against the oracle (in slabs of 1024 rows: quantisation is local to a 32-row block)
+    rq_c, rs_c, cq_c, cs_c = rq.cpu(), rs.cpu(), cq.cpu(), cs.cpu()
+    for r0 in range(0, M, 1024):
+        sl = slice(r0, r0 + 1024)
         exp_r = O.quantize(x[sl], axis=-1, use_sr=True, rand_bits=r[sl])
-        _check_pair((rq[sl], rs[sl]), exp_r, f"cfg2 row blocks {b0}")
+        _check_pair((rq_c[sl], rs_c[sl]), exp_r, f"cfg2 row copy, rows {r0}")
         exp_c = O.quantize(O.rht_left(x[sl], signs, perm), axis=0, use_sr=True, rand_bits=r[sl])
-        _check_pair((cq[16 * b0:16 * (b0 + 4)], cs[b0:b0 + 4]), exp_c, f"cfg2 col blocks {b0}")
+        _check_pair((cq_c[r0 // 2:r0 // 2 + 512], cs_c[r0 // 32:r0 // 32 + 32]), exp_c, f"cfg2 column copy, rows {r0}")
     # whole-tensor property: stochastic rounding is unbiased, so the dequantized row copy averages to the input
     dq = m.convert_from_mxfp4(rq, rs, torch.float32)
     xd = x.to(DEV).float()

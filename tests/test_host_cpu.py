@@ -238,6 +238,42 @@ def test_weight_cache_is_keyed_by_object_identity():
         L.enable_weight_cache(False)
 
 
+def test_weight_cache_hits_for_a_parameter():
+    """The training case: the weight is an nn.Parameter, and the plain-tensor alias the kernels work on is a new object
+    in every forward.  The entry must belong to the Parameter (hit on the second forward, miss after an optimizer-style
+    update, gone with the Parameter)."""
+    import gc
+    from alto_amd.mxfp4 import linear as L
+    calls = []
+
+    def fake_rowcol(w, *a, **k):
+        calls.append(w)
+        return ("q", len(calls))
+
+    real = L.quantize_rowcol
+    L.quantize_rowcol = fake_rowcol
+    L.enable_weight_cache(True)
+    try:
+        p = torch.nn.Parameter(torch.zeros(64, 32))
+        outs = []
+        for _ in range(3):
+            alias = L.unwrap_weight_wrapper(p)
+            assert alias is not p and type(alias) is torch.Tensor
+            outs.append(L._quantize_weight_2d(alias, False, owner=p))
+        assert len(calls) == 1 and outs[0] is outs[1] is outs[2]
+        assert L.weight_cache_stats() == {"hits": 2, "misses": 1, "entries": 1}
+        with torch.no_grad():
+            p.add_(1.0)
+        assert L._quantize_weight_2d(L.unwrap_weight_wrapper(p), False, owner=p) is not outs[0] and len(calls) == 2
+        del p, alias
+        calls.clear()
+        gc.collect()
+        assert L.weight_cache_stats()["entries"] == 0
+    finally:
+        L.quantize_rowcol = real
+        L.enable_weight_cache(False)
+
+
 def test_product_never_imports_the_oracle_and_bench_refuses_more_than_one_gpu():
     """The oracle is the checker: nothing under the package may import it, and bench.py only inside its cpu_sample legs.
     bench.py measures one GPU and says so when asked for more."""
@@ -256,3 +292,18 @@ def test_product_never_imports_the_oracle_and_bench_refuses_more_than_one_gpu():
         assert last_def >= 0 and head[last_def:].lstrip().startswith("def cpu_sample"), "bench.py imports the oracle outside a cpu_sample leg"
     r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
     assert r.returncode != 0 and "one GPU" in r.stderr
+
+
+def test_wrapped_weights_and_config_survive_a_weights_only_round_trip(tmp_path):
+    """dispatch/tensor.py:499-503 and config.py:57 register the wrapper and the recipe as safe globals so that a state
+    dict holding wrapped weights loads with torch.load(weights_only=True)."""
+    import alto_amd.mxfp4 as m
+    cfg = m.TrainingOpConfig(use_hadamard=False, clip_mode="static")
+    w = torch.arange(64 * 32, dtype=torch.float32).reshape(64, 32)
+    wrapped = m.MXFP4TrainingWeightWrapperTensor(w.clone(), cfg)
+    path = tmp_path / "ckpt.pt"
+    torch.save({"weight": wrapped, "config": cfg}, path)
+    back = torch.load(path, weights_only=True)
+    assert isinstance(back["weight"], m.MXFP4TrainingWeightWrapperTensor)
+    assert back["config"] == cfg and back["weight"].config == cfg
+    assert torch.equal(back["weight"]._data, w)

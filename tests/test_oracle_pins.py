@@ -535,3 +535,83 @@ def test_hw_sr_dword_addressing_is_a_bijection_onto_the_stream():
             else:
                 exp = int(stream[4 * (R + (band * C + j) * 4 + (p2 % 16) // 4) + p2 % 4])
             assert int(cd[b, p2, j]) == exp
+
+
+# --------------------------------------------------------------------------- grouped backward twins
+def _toy_grouped(seed=5):
+    g = torch.Generator().manual_seed(seed)
+    offs = torch.tensor([64, 64, 160], dtype=torch.int32)          # expert 1 is empty; boundaries on multiples of 32
+    idx = O.indices_from_offsets(offs)
+    x = torch.randn(160, 64, generator=g).bfloat16()
+    go = (torch.randn(160, 32, generator=g) * 1e-2).bfloat16()
+    w = (torch.randn(3, 32, 64, generator=g) * 0.1).bfloat16()     # [E, N, K]
+    return offs, idx, x, go, w
+
+
+def _decode_fraction(codes, scales, r, c, packed_along_last, scale_of):
+    """Exact value of element (r, c) of a quantised matrix, through the scalar model's decode (independent of the torch
+    oracle's dequantize): the nibble, its grid value, times 2^(scale byte - 127)."""
+    if packed_along_last:
+        byte = int(codes[r, c // 2]); nib = (byte >> (4 * (c & 1))) & 0xF
+    else:
+        byte = int(codes[r // 2, c]); nib = (byte >> (4 * (r & 1))) & 0xF
+    e = int(scale_of(r, c)) - 127
+    return Fraction(S.decode(nib)) * (Fraction(2) ** e)
+
+
+def test_grouped_dx_reference_equals_the_dense_twin_per_expert_and_an_exact_sum():
+    offs, idx, x, go, w = _toy_grouped()
+    go_q, go_s = O.quantize(go)                                          # blocks along N (the reduction of dX)
+    bounds = [(0, 64), (64, 64), (64, 160)]
+    for k_pack_w in (False, True):
+        wq, ws = O.quantize(w, axis=-2 if k_pack_w else -1, is_2d_block=True)   # packed along N, or along K
+        dx = O.grouped_gemm_dx_ref(go_q, go_s, wq, ws, idx, use_2dblock_w=True, trans_weights=True, k_pack_w=k_pack_w)
+        assert dx.shape == (160, 64)
+        for e, (lo, hi) in enumerate(bounds):
+            if hi > lo:
+                ref = O.gemm_ref(go_q[lo:hi], go_s[lo:hi], wq[e], ws[e], use_2dblock_b=True, k_pack_b=k_pack_w)
+                assert torch.equal(dx[lo:hi], ref), (k_pack_w, e)
+        # exact rational sums for a few entries, decoded nibble by nibble
+        for (r, k) in [(0, 0), (63, 17), (64, 5), (159, 63)]:
+            e = int(idx[r])
+            tot = Fraction(0)
+            for n in range(32):
+                a = _decode_fraction(go_q, go_s, r, n, True, lambda rr, cc: go_s[rr, cc // 32])
+                b = _decode_fraction(wq[e], ws[e], n, k, not k_pack_w, lambda rr, cc: ws[e][rr // 32, cc // 32])
+                tot += a * b
+            assert Fraction(float(dx[r, k])) == tot, (k_pack_w, r, k)
+    # [E, K, N] storage gives the same dX
+    wt = w.transpose(-1, -2).contiguous()
+    wq2, ws2 = O.quantize(wt, axis=-2, is_2d_block=True)                 # packed along K (dim -2 of [E, K, N])
+    wq1, ws1 = O.quantize(w, axis=-1, is_2d_block=True)
+    assert torch.equal(O.grouped_gemm_dx_ref(go_q, go_s, wq2, ws2, idx, trans_weights=False, k_pack_w=False),
+                       O.grouped_gemm_dx_ref(go_q, go_s, wq1, ws1, idx, trans_weights=True, k_pack_w=False))
+
+
+def test_grouped_dw_reference_equals_the_dense_twin_per_expert_and_an_exact_sum():
+    offs, idx, x, go, w = _toy_grouped()
+    go_qm, go_sm = O.quantize(go, axis=0)                                # blocks along the tokens (the reduction of dW)
+    x_qm, x_sm = O.quantize(x, axis=0)
+    dw = O.grouped_gemm_dw_ref(go_qm, go_sm, x_qm, x_sm, idx, 3)
+    assert dw.shape == (3, 32, 64)
+    assert torch.equal(dw[1], torch.zeros(32, 64, dtype=dw.dtype)), "an expert without tokens gets a zero gradient"
+    for e, (lo, hi) in enumerate([(0, 64), (64, 64), (64, 160)]):
+        if hi > lo:
+            ref = O.gemm_ref(go_qm[lo // 2:hi // 2], go_sm[lo // 32:hi // 32], x_qm[lo // 2:hi // 2], x_sm[lo // 32:hi // 32], trans_a=True)
+            assert torch.equal(dw[e], ref), e
+    for (e, n, k) in [(0, 0, 0), (2, 31, 63), (2, 7, 20)]:
+        lo, hi = [(0, 64), (64, 64), (64, 160)][e]
+        tot = Fraction(0)
+        for t in range(lo, hi):
+            a = _decode_fraction(go_qm, go_sm, t, n, False, lambda rr, cc: go_sm[rr // 32, cc])
+            b = _decode_fraction(x_qm, x_sm, t, k, False, lambda rr, cc: x_sm[rr // 32, cc])
+            tot += a * b
+        assert Fraction(float(dw[e, n, k])) == tot, (e, n, k)
+    # [E, K, N] storage: the transposed gradient
+    assert torch.equal(O.grouped_gemm_dw_ref(go_qm, go_sm, x_qm, x_sm, idx, 3, trans_weights=False), dw.transpose(-1, -2))
+    # 2D blocks: one quantisation, packed along the last dim
+    go_q2, go_s2 = O.quantize(go, axis=-1, is_2d_block=True)
+    x_q2, x_s2 = O.quantize(x, axis=-1, is_2d_block=True)
+    dw2 = O.grouped_gemm_dw_ref(go_q2, go_s2, x_q2, x_s2, idx, 3, use_2dblock_x=True)
+    ref = O.dequantize(go_q2, go_s2, torch.float32, is_2d_block=True).double()[64:160].T @ O.dequantize(x_q2, x_s2, torch.float32, is_2d_block=True).double()[64:160]
+    assert torch.equal(dw2[2], ref)

@@ -49,6 +49,40 @@ def test_grouped_gemm_noalloc_equals_workspace_entry_point():
         assert bool((got[int(offs[-1]):] == 0).all())
 
 
+def test_grouped_gemm_noalloc_replays_from_a_hip_graph():
+    """After alto_mxfp4_init() the call makes no runtime query, so it can be captured: three replays, with the program's
+    own eager work between them (new activations written into the captured input buffers), each against the eager call."""
+    import alto_amd.mxfp4 as m
+    from alto_amd.mxfp4 import _runtime as rt
+    lib = rt.lib()
+    assert lib.alto_mxfp4_init() == 0, lib.alto_mxfp4_last_error()
+    E, N, K, rows = 4, 256, 512, 1024
+    w = (randn_outliers((E, N, K), torch.bfloat16, seed=5) * 0.02).to(DEV)
+    wq, ws = m.convert_to_mxfp4(w, is_2d_block=True)
+    offs = torch.tensor([0, 300, 300, 811, 1000], dtype=torch.int32, device=DEV)
+    aq, as_ = m.convert_to_mxfp4(randn_outliers((rows, K), torch.bfloat16, seed=6).to(DEV))
+    out = torch.zeros((rows, N), dtype=torch.bfloat16, device=DEV)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        _call(lib, rt, "alto_mxfp4_grouped_gemm_noalloc", aq, as_, wq, ws, offs, E, out)   # warm-up on the capture stream
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            _call(lib, rt, "alto_mxfp4_grouped_gemm_noalloc", aq, as_, wq, ws, offs, E, out)
+    torch.cuda.current_stream().wait_stream(side)
+    for rep in range(3):
+        nq, ns = m.convert_to_mxfp4(randn_outliers((rows, K), torch.bfloat16, seed=10 + rep).to(DEV))
+        aq.copy_(nq); as_.copy_(ns)
+        out.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        ref = torch.full((rows, N), float("nan"), dtype=torch.bfloat16, device=DEV)
+        wsp = torch.empty(lib.alto_mxfp4_grouped_gemm_workspace_bytes(rows, E), dtype=torch.uint8, device=DEV)
+        _call(lib, rt, "alto_mxfp4_grouped_gemm", aq, as_, wq, ws, offs, E, ref, wsp)
+        torch.cuda.synchronize()
+        assert torch.equal(out.view(torch.int16), ref.view(torch.int16)), f"replay {rep}"
+
+
 def test_grouped_gemm_noalloc_rejects_what_does_not_fit():
     from alto_amd.mxfp4 import _runtime as rt
     lib = rt.lib()
