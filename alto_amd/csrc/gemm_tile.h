@@ -45,6 +45,9 @@ struct TileArgs {
   int64_t as_bytes, bs_bytes;  // extent of the scale buffers in bytes (< 2^31)
   int s_k0;                    // first scale byte of this reduction inside the operands' scale rows (0 unless a sub-range of K)
   int s_row;                   // length of a whole scale row in bytes (>= 16): loads never reach past it
+  int k_lead = 0;              // the first k_lead (< 8) K groups of the reduction read as zero codes: a reduction over a
+                               // sub-range of K starts at the 128-byte line that holds its first group, so that every
+                               // operand load is one whole line, and the groups before the range drop out this way
 };
 
 // Every field of TileArgs is the same for all lanes.  When the struct arrives through memory (a real function call) the
@@ -75,6 +78,7 @@ __device__ __forceinline__ TileArgs uniform_args(const TileArgs& t) {
   o.a_bytes = uniform_i64(t.a_bytes); o.b_bytes = uniform_i64(t.b_bytes);
   o.as_bytes = uniform_i64(t.as_bytes); o.bs_bytes = uniform_i64(t.bs_bytes);
   o.s_k0 = __builtin_amdgcn_readfirstlane(t.s_k0); o.s_row = __builtin_amdgcn_readfirstlane(t.s_row);
+  o.k_lead = __builtin_amdgcn_readfirstlane(t.k_lead);
   return o;
 }
 
@@ -98,7 +102,7 @@ __device__ __forceinline__ void gemm_tile_zero(TileAcc& acc) {
 //   Scales: thread t owns tile row t of A (t < 256) or tile row t - 256 of B (unit stride along K, any alignment).
 struct TileLoader {
   __amdgpu_buffer_rsrc_t rsrc_a, rsrc_b, rsrc_s;
-  int wave, gpiece, arow0, brow0, a_last, a_first, b_last, kbytes, G, s_k0, s_row;
+  int wave, gpiece, arow0, brow0, a_last, a_first, b_last, kbytes, G, s_k0, s_row, k_lead;
   uint32_t ld_a, ld_b, soff;
 
   __device__ __forceinline__ void init(const TileArgs& ta) {
@@ -119,6 +123,7 @@ struct TileLoader {
     G = ta.G;
     s_k0 = ta.s_k0;
     s_row = ta.s_row;
+    k_lead = ta.k_lead;
     const bool s_is_a = wave < GT_TM / 64;   // scalar: the descriptor choice below must be provably wave-uniform
     rsrc_s = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(s_is_a ? ta.A.scales : ta.B.scales), 0,
                                                (int)(s_is_a ? ta.as_bytes : ta.bs_bytes), 0x00020000);
@@ -142,7 +147,7 @@ struct TileLoader {
     lds_u8* const lds = (lds_u8*)smem;
     const int koff = __builtin_amdgcn_readfirstlane(s * 128);   // scalar offset operand: must live in an SGPR
     // a piece beyond K gets bit 31 set in its offset: out of range for the descriptor, so zeros land in LDS
-    const uint32_t oob = (koff + gpiece * 16 < kbytes) ? 0u : 0x80000000u;
+    const uint32_t oob = (koff + gpiece * 16 < kbytes && s * 8 + gpiece >= k_lead) ? 0u : 0x80000000u;
 #pragma unroll
     for (int i = i0; i < i1; ++i) {
       int row;
@@ -164,31 +169,41 @@ struct TileLoader {
     }
   }
 
-  // 16 scale bytes of K block kb for this thread's row; groups at or beyond G read as 127 (scale 1.0) so that the zero
-  // codes of a K tail never meet a NaN scale byte.
+  // 16 scale bytes of K block kb for this thread's row, in two parts so that nothing touches the loaded registers until
+  // they are used (the wave would otherwise sit out the load's latency right here, two blocks before the bytes are needed):
+  // sload sends the load, sfix -- called when the bytes go to LDS -- makes groups at or beyond G read as 127 (scale 1.0),
+  // so that the zero codes of a K tail never meet a NaN scale byte.
   template <bool KTAIL>
-  __device__ __forceinline__ void sload(int kb, uint32_t (&sreg)[4]) const {
-    const int rem = G - kb * 16;   // wave-uniform
+  __device__ __forceinline__ void sload(int kb, v4i_t& raw) const {
     const int kb16 = __builtin_amdgcn_readfirstlane(kb * 16);
     if constexpr (!KTAIL) {   // G % 4 == 0 and the whole K range: every dword is all inside or all beyond K, one 16-byte load
-      v4i_t w4 = __builtin_amdgcn_raw_buffer_load_b128(rsrc_s, (int)soff, kb16, 0);
-#pragma unroll
-      for (int d = 0; d < 4; ++d) sreg[d] = rem - 4 * d >= 4 ? (uint32_t)w4[d] : 0x7F7F7F7Fu;
+      raw = __builtin_amdgcn_raw_buffer_load_b128(rsrc_s, (int)soff, kb16, 0);
       return;
     }
     // General case (any G, any sub-range of K): still one 16-byte load per row.  A block that would reach past the end
-    // of the scale row is loaded from the last 16 bytes of the row instead and shifted down by the difference, so no
-    // byte from beyond the row (possibly beyond the buffer) is ever used; bytes at or beyond G become 127.  All shift
-    // amounts and masks are wave-uniform and applied with mask arithmetic: no branch splits the MFMA loop.
+    // of the scale row is loaded from the last 16 bytes of the row instead (and shifted down by the difference in sfix),
+    // so no byte from beyond the row (possibly beyond the buffer) is ever used.
     const int want = s_k0 + kb16;                     // where the block starts in the scale row
     const int last = s_row - 16;
     const int off = __builtin_amdgcn_readfirstlane(want < last ? want : last);
+    raw = __builtin_amdgcn_raw_buffer_load_b128(rsrc_s, (int)soff, off, 0);
+  }
+  template <bool KTAIL>
+  __device__ __forceinline__ void sfix(int kb, const v4i_t& L, uint32_t (&sreg)[4]) const {
+    const int rem = G - kb * 16;   // wave-uniform
+    if constexpr (!KTAIL) {
+#pragma unroll
+      for (int d = 0; d < 4; ++d) sreg[d] = rem - 4 * d >= 4 ? (uint32_t)L[d] : 0x7F7F7F7Fu;
+      return;
+    }
+    // bytes at or beyond G become 127; all shift amounts and masks are wave-uniform and applied with mask arithmetic
+    const int want = s_k0 + kb * 16;
+    const int last = s_row - 16;
+    const int off = want < last ? want : last;
     int sh = want - off;                                 // bytes to shift down: 0 unless clamped
     sh = sh > 16 ? 16 : sh;
     const int q = sh >> 2, rb = sh & 3;
     int valid = rem < 0 ? 0 : (rem > 16 ? 16 : rem);     // bytes of this block that lie inside K
-    v4i_t L = __builtin_amdgcn_raw_buffer_load_b128(rsrc_s, (int)soff, off, 0);
-    asm volatile("" : "+v"(L));
     uint32_t mq[5];
 #pragma unroll
     for (int c = 0; c < 5; ++c) mq[c] = (uint32_t)(-(int)(q == c));   // all ones for the dword shift in effect
@@ -219,7 +234,7 @@ struct TileLoader {
 template <bool KTAIL>
 __device__ __forceinline__ void gemm_tile_mainloop(const TileArgs& ta, TileAcc& acc, uint8_t* smem) {
   TileLoader ld;
-  uint32_t sreg[4];
+  v4i_t sraw;   // scale bytes of a later block, as loaded
   __syncthreads();   // the LDS ring may still be read by a previous call
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;   // the wave index lives in a scalar register
@@ -243,6 +258,8 @@ __device__ __forceinline__ void gemm_tile_mainloop(const TileArgs& ta, TileAcc& 
   // LDS row layout (4 dwords): [h=0: K 0..255 | h=0: K 256..511 | h=1: K 0..255 | h=1: K 256..511], where the half-wave h
   // of the MFMA uses group 8 ms + 2 j + h at K step j of macro stage ms: byte j of dword 2 h + ms.
   auto swrite = [&](int kb) {
+    uint32_t sreg[4];
+    ld.template sfix<KTAIL>(kb, sraw, sreg);
     uint32_t* row = sscale + (kb & 1) * GT_SCALE_BUF_DW + tid * GT_SCALE_PITCH;
     row[0] = __builtin_amdgcn_perm(sreg[1], sreg[0], 0x06040200u);   // groups 0, 2, 4, 6
     row[1] = __builtin_amdgcn_perm(sreg[3], sreg[2], 0x06040200u);   // groups 8, 10, 12, 14
@@ -333,11 +350,14 @@ __device__ __forceinline__ void gemm_tile_mainloop(const TileArgs& ta, TileAcc& 
     read_frags(MS, 3, fa1, fb1);
     interleave();
     __builtin_amdgcn_sched_barrier(0);
-    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    // (the wait as a builtin: the compiler's own wait insertion then knows that nothing is outstanding behind it and does
+    // not guard later uses of registers loaded before this point)
+    __builtin_amdgcn_s_waitcnt(0);
+    asm volatile("s_barrier" ::: "memory");
     __builtin_amdgcn_s_setprio(3);
     if constexpr (MS == 0) {
       swrite(kb + 1);          // block kb+1 -> the other scale buffer (last read at the end of block kb-1)
-      ld.template sload<KTAIL>(kb + 2, sreg);
+      ld.template sload<KTAIL>(kb + 2, sraw);
       __builtin_amdgcn_sched_barrier(0);
     }
     ld.gload(smem, s + 2, MS, 0, 4);
@@ -353,10 +373,10 @@ __device__ __forceinline__ void gemm_tile_mainloop(const TileArgs& ta, TileAcc& 
   // and the first block's scales in registers.  Stages beyond K load zeros and blocks beyond K load unit scales, so
   // nothing below is conditional.
   ld.init(ta);
-  ld.template sload<KTAIL>(0, sreg);
+  ld.template sload<KTAIL>(0, sraw);
   ld.gload(smem, 0, 0, 0, 8);
   swrite(0);
-  ld.template sload<KTAIL>(1, sreg);
+  ld.template sload<KTAIL>(1, sraw);
   ld.gload(smem, 1, 1, 0, 4);   // the other half goes out in the first step of the loop
   asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)\n\ts_barrier" ::: "memory");   // all but stage 1's four loads
   read_frags(0, 0, fa0, fb0);

@@ -411,11 +411,15 @@ __global__ __launch_bounds__(GT_THREADS) void grouped_dw_tiled_kernel(OperandVie
     t0 &= ~(int64_t)31;
     t1 &= ~(int64_t)31;
     if (t1 <= t0) continue;
-    OperandView Pv = P, Qv = Q;   // codes start at the run; the scale rows keep their base and the run's offset rides in s_k0
-    Pv.codes += t0 / 2;
-    Qv.codes += t0 / 2;
-    TileArgs ta{Pv, Qv, (int64_t)tm * GT_TM, (int64_t)tn * GT_TN, 0, NP, NQ, (int)((t1 - t0) / 32), out_scale,
-                p_bytes - t0 / 2, q_bytes - t0 / 2, ps_bytes, qs_bytes, (int)(t0 / 32), (int)(M_total / 32)};
+    // The codes start at the 128-byte line (256 tokens) that holds the run's first token, so that every operand load is one
+    // whole line; the groups of that line that lie before the run read as zeros (k_lead).  The scale rows keep their
+    // base and the offset of the line rides in s_k0.
+    const int64_t ta0 = t0 & ~(int64_t)255;
+    OperandView Pv = P, Qv = Q;
+    Pv.codes += ta0 / 2;
+    Qv.codes += ta0 / 2;
+    TileArgs ta{Pv, Qv, (int64_t)tm * GT_TM, (int64_t)tn * GT_TN, 0, NP, NQ, (int)((t1 - ta0) / 32), out_scale,
+                p_bytes - ta0 / 2, q_bytes - ta0 / 2, ps_bytes, qs_bytes, (int)(ta0 / 32), (int)(M_total / 32), (int)((t0 - ta0) / 32)};
     gemm_tile_mainloop<true>(ta, acc, smem);
   }
   if (bad) {
