@@ -642,7 +642,6 @@ def main():
                 if key == "mfma_probe_random":
                     clock_observed = r.get("clock_mhz")
                 continue
-            primary_mem_release = None  # noqa: F841
             try:
                 try:
                     r = measure(w, dev, gen, max(5, args.steps // 2), max(2, args.warmup // 2), args.settle_ms)
@@ -689,7 +688,9 @@ def main():
                    "settle_ms": args.settle_ms},
         "ms_median": round(res["ms_median"], 5), "ms_min": round(res["ms_min"], 5), "ms_max": round(res["ms_max"], 5),
         "roofline": {"bound": res["bound"], "achieved": round(res["achieved"], 3), "peak": res["peak"], "unit": res["unit"],
-                     "frac": round(res["frac"], 4), "traffic": load_traffic(args.workload), "kernel": res["kernel"], "kernel_ms": round(res["ms"], 5)},
+                     "frac": round(res["frac"], 4), "traffic": load_traffic(args.workload), "kernel": res["kernel"], "kernel_ms": round(res["ms"], 5),
+                     # achieved / frac come from the event bracket around all K launches (ms_per_step), not from the per-step median
+                     "timing": "HIP events around the K timed launches on the launch stream"},
         "cpu_baseline": cpu,
         # the same steps on a device that had been idle (its clock still rising): beside `value`, never instead of it
         "from_idle": from_idle,
