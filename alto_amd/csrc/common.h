@@ -14,7 +14,7 @@ void set_error(const char* fmt, ...);
 int check_launch(const char* what);
 int quantize_dynamic_launch(const void* x, int dtype, int64_t batch, int64_t M, int64_t C, int64_t ld_x, int64_t bs_x, uint8_t* codes,
                             uint8_t* scales, int64_t ld_codes, int is_2d, int sr, const uint32_t* rand_bits, int64_t ld_rand,
-                            int64_t bs_rand, hipStream_t st);
+                            int64_t bs_rand, int use_uos, hipStream_t st);
 
 #define ALTO_REQUIRE(cond, ...)            \
   do {                                     \

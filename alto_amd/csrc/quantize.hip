@@ -630,8 +630,8 @@ int quantize_impl(const void* x, int dtype, int64_t batch, int64_t M, int64_t C,
   ALTO_REQUIRE(clip_mode == ALTO_CLIP_NONE || clip_mode == ALTO_CLIP_STATIC || clip_mode == ALTO_CLIP_DYNAMIC, "quantize: bad clip_mode %d", clip_mode);
   if (batch == 0 || M == 0 || C == 0) return ALTO_MXFP4_OK;
   if (clip_mode == ALTO_CLIP_DYNAMIC) {   // std-based scale: separate plain kernel, quantisation along the contiguous dim
-    ALTO_REQUIRE(do_row && !do_col && !hadamard && !use_uos,
-                 "quantize: clip_mode=dynamic gives the row output only (no column output, Hadamard or UOS); transpose on the host");
+    ALTO_REQUIRE(do_row && !do_col && !hadamard,
+                 "quantize: clip_mode=dynamic gives the row output only (no column output, no Hadamard); transpose on the host");
     if (sr_mode >= 2) {
       set_error("quantize: clip_mode=dynamic takes its random words from a tensor (fill one with alto_mxfp4_random_bits)");
       return ALTO_MXFP4_ENOTIMPL;
@@ -639,7 +639,7 @@ int quantize_impl(const void* x, int dtype, int64_t batch, int64_t M, int64_t C,
     ALTO_REQUIRE(ld_row_codes % 16 == 0, "quantize: clip_mode=dynamic needs 16-byte aligned code rows");
     ALTO_REQUIRE((M + 31) / 32 <= 65535, "quantize: M (%lld) exceeds 65535 row blocks", (long long)M);
     return quantize_dynamic_launch(x, dtype, batch, M, C, ld_x, bs_x, row_codes, row_scales, ld_row_codes, is_2d, sr_mode == 1,
-                                   rand_bits, ld_rand, bs_rand, reinterpret_cast<hipStream_t>(stream));
+                                   rand_bits, ld_rand, bs_rand, use_uos, reinterpret_cast<hipStream_t>(stream));
   }
 
   QuantParams p;

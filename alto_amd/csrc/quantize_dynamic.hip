@@ -19,6 +19,7 @@ struct DynParams {
   const uint32_t* rand; int64_t ld_r, bs_r;
   uint8_t* codes; uint8_t* scales; int64_t ld_c;
   int M, C;
+  int uos;   // scale from ceil(log2(max_abs / 7.25)) + 127 instead of the exponent rule (mxfp_quantization.py:75-78)
 };
 
 template <typename T>
@@ -65,7 +66,8 @@ __global__ __launch_bounds__(64) void quant_dynamic_kernel(DynParams p) {
   uint32_t e;
   if constexpr (BF) e = (((f2u(amax) >> 16) + 0x20u) >> 7) & 0x1FFu;
   else e = ((f2u(amax) + 0x200000u) >> 23) & 0x1FFu;
-  const uint32_t s = (e < 1u ? 1u : e) & 0xFFu;
+  uint32_t s = (e < 1u ? 1u : e) & 0xFFu;
+  if (p.uos) s = e8m0_uos(amax);
   if (!valid) return;
   if (!B2D) p.scales[(b * p.M + row) * (p.C / 32) + cb] = (uint8_t)s;
   else if (r == 0) p.scales[(b * (p.M / 32) + blockIdx.y) * (p.C / 32) + cb] = (uint8_t)s;
@@ -99,8 +101,8 @@ void launch(const DynParams& p, dim3 grid, hipStream_t st, bool is_2d, bool sr) 
 // Row output only; arguments already validated by alto_mxfp4_quantize_pitched.
 int quantize_dynamic_launch(const void* x, int dtype, int64_t batch, int64_t M, int64_t C, int64_t ld_x, int64_t bs_x, uint8_t* codes,
                             uint8_t* scales, int64_t ld_codes, int is_2d, int sr, const uint32_t* rand_bits, int64_t ld_rand,
-                            int64_t bs_rand, hipStream_t st) {
-  DynParams p{x, ld_x, bs_x, rand_bits, ld_rand, bs_rand, codes, scales, ld_codes, (int)M, (int)C};
+                            int64_t bs_rand, int use_uos, hipStream_t st) {
+  DynParams p{x, ld_x, bs_x, rand_bits, ld_rand, bs_rand, codes, scales, ld_codes, (int)M, (int)C, use_uos ? 1 : 0};
   dim3 grid((unsigned)((C / 32 + 1) / 2), (unsigned)((M + 31) / 32), (unsigned)batch);
   if (dtype == ALTO_DT_BF16) launch<__bf16>(p, grid, st, is_2d != 0, sr != 0);
   else launch<float>(p, grid, st, is_2d != 0, sr != 0);

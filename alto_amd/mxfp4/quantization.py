@@ -257,8 +257,6 @@ def _convert_dynamic(x: torch.Tensor, ax: int, is_2d_block: bool, use_sr: bool, 
     """``clip_mode="dynamic"`` (std-based scale, mxfp_quantization.py:54-59,65-70): an optional knob served by a plain
     kernel that quantises along the contiguous dim; other axes are brought there with a copy, a Hadamard transform runs
     as its own launch first."""
-    if use_uos:
-        raise NotImplementedError("clip_mode='dynamic' together with use_uos is not implemented")
     if hadamard is not None:
         x = hadamard_left(x, hadamard)
     xt = x.transpose(ax, -1)
@@ -268,7 +266,7 @@ def _convert_dynamic(x: torch.Tensor, ax: int, is_2d_block: bool, use_sr: bool, 
     r3 = None
     if use_sr:
         r3 = rand_bits.transpose(ax, -1).contiguous().reshape(x3.shape)
-    codes, scales, _, _ = _quantize_call(x3, True, False, is_2d_block, use_sr, r3, None, rt.CLIP["dynamic"], False)
+    codes, scales, _, _ = _quantize_call(x3, True, False, is_2d_block, use_sr, r3, None, rt.CLIP["dynamic"], use_uos)
     codes = codes.reshape(*shp[:-1], shp[-1] // 2)
     scales = scales.reshape(*shp[:-2], shp[-2] // 32, shp[-1] // 32) if is_2d_block else scales.reshape(*shp[:-1], shp[-1] // 32)
     return codes.transpose(ax, -1), scales.transpose(ax, -1)

@@ -53,6 +53,12 @@ def main():
         dq = ref_utils.convert_from_mxfp4_pytorch(q, s, output_dtype=torch.float32, clip_mode="dynamic", **kw)
         out[f"dyn_{name}_dq"] = dq.contiguous().numpy().copy()
 
+    # dynamic clip together with the UOS scale rule (the reference's kernel allows the pair, its own test skips it): fp32 only
+    for name, kw in (("row", dict(axis=-1)), ("col", dict(axis=-2)), ("2d", dict(axis=-1, is_2d_block=True))):
+        q, s = ref_utils.convert_to_mxfp4_pytorch(x, clip_mode="dynamic", use_uos=True, **kw)
+        out[f"dynuos_{name}_codes"] = q.contiguous().numpy().copy()
+        out[f"dynuos_{name}_scales"] = s.contiguous().numpy().copy()
+
     # ---- the twin's other modes (clip none / static, the UOS scale rule), bf16 and fp32: they pin the scale rule, the
     # round-to-nearest encode and the packing by bytes the reference wrote, beside the closed-form pins of the oracle.
     # The twin rounds to nearest only (no stochastic rounding), so these are RNE vectors.

@@ -133,6 +133,27 @@ def test_dynamic_clip_equals_the_reference_twin(name, kw):
     assert torch.equal(dq.contiguous(), torch.from_numpy(d[f"dyn_{name}_dq"]))
 
 
+@pytest.mark.parametrize("name,kw", [("row", dict(axis=-1)), ("col", dict(axis=-2)), ("2d", dict(axis=-1, is_2d_block=True))])
+def test_dynamic_clip_with_uos_equals_the_reference_twin(name, kw):
+    """clip_mode="dynamic" together with use_uos (mxfp_quantization.py:54-78 allows the pair): the twin's fp32 bytes."""
+    d = _ref_vectors()
+    x = torch.from_numpy(d["dyn_x"])
+    q, s = O.quantize(x, clip_mode="dynamic", use_uos=True, **kw)
+    assert torch.equal(s.contiguous(), torch.from_numpy(d[f"dynuos_{name}_scales"]))
+    assert torch.equal(q.contiguous(), torch.from_numpy(d[f"dynuos_{name}_codes"]))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name,kw", [("row", dict(axis=-1)), ("col", dict(axis=-2)), ("2d", dict(axis=-1, is_2d_block=True))])
+def test_hip_dynamic_clip_with_uos_equals_the_reference_twin(name, kw):
+    import alto_amd.mxfp4 as m
+    d = _ref_vectors()
+    x = torch.from_numpy(d["dyn_x"]).cuda()
+    q, s = m.convert_to_mxfp4(x, clip_mode="dynamic", use_uos=True, **kw)
+    assert_bytes_equal(s.contiguous(), torch.from_numpy(d[f"dynuos_{name}_scales"]), f"dynamic+uos {name} scales")
+    assert_bytes_equal(q.contiguous(), torch.from_numpy(d[f"dynuos_{name}_codes"]), f"dynamic+uos {name} codes")
+
+
 @pytest.mark.parametrize("name", ["a", "b", "c"])
 def test_attention_model_equals_the_reference_cpu_model(name):
     """The oracle's MXFP4 attention recurrence gives the reference CPU model's outputs (test_mxfp_pnq.py:87-149) bit for

@@ -223,14 +223,15 @@ def test_edge_cases(m):
 @pytest.mark.parametrize("is_2d", [False, True])
 @pytest.mark.parametrize("use_sr", [False, True])
 @pytest.mark.parametrize("axis", [-1, 0])
-def test_dynamic_clip(m, dtype, is_2d, use_sr, axis):
+@pytest.mark.parametrize("use_uos", [False, True])
+def test_dynamic_clip(m, dtype, is_2d, use_sr, axis, use_uos):
     """clip_mode="dynamic" (std-based scale, mxfp_quantization.py:54-59,65-70): bit-equal to the CPU model, whose order of
     the fp32 sums is the kernel's (the reference leaves it to Triton's reduction: parity with that order is unpinned)."""
     x = randn_outliers((96, 160), dtype, seed=31)
     r = rand_bits((96, 160), seed=32) if use_sr else None
-    got = m.convert_to_mxfp4(x.to(DEV), axis=axis, is_2d_block=is_2d, use_sr=use_sr, clip_mode="dynamic",
+    got = m.convert_to_mxfp4(x.to(DEV), axis=axis, is_2d_block=is_2d, use_sr=use_sr, clip_mode="dynamic", use_uos=use_uos,
                              rand_bits=None if r is None else r.to(DEV))
-    exp = O.quantize(x, axis=axis, is_2d_block=is_2d, use_sr=use_sr, rand_bits=r, clip_mode="dynamic")
+    exp = O.quantize(x, axis=axis, is_2d_block=is_2d, use_sr=use_sr, rand_bits=r, clip_mode="dynamic", use_uos=use_uos)
     _check_pair(got, exp, "dynamic clip")
     # the clip does something: scales differ from the absmax rule somewhere
     plain = O.quantize(x, axis=axis, is_2d_block=is_2d, use_sr=use_sr, rand_bits=r)
