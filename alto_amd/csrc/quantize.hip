@@ -491,21 +491,12 @@ __global__ __launch_bounds__(256) void quant_kernel(const QuantParams p) {
   }
 }
 
-// Standalone transform: thread t owns one column, loads the 32 rows of a block in permuted order, runs the same
-// butterfly as the fused quantizer and writes each position back to the row it came from.
-template <typename T>
-__global__ __launch_bounds__(256) void hadamard_kernel(const T* __restrict__ x, int64_t ld_x, T* __restrict__ y, int64_t ld_y, int C,
-                                                       const QuantParams p) {
-  const int cc = blockIdx.x * 256 + threadIdx.x;
-  if (cc >= C) return;
-  const int64_t row0 = (int64_t)blockIdx.y * 32;
-  float z[32];
+// The 32-point butterfly both standalone kernels share: z holds the block in permuted order (z[k] = element perm^-1[k]).
+// `in_flip` / `out_flip` are sign masks over k: the inverse transform (W^T) applies diag(Q) to the input, the forward
+// transform to the output, and the other mask is zero.
+__device__ __forceinline__ void hadamard32(float (&z)[32], uint32_t in_flip, uint32_t out_flip) {
 #pragma unroll
-  for (int k = 0; k < 32; ++k) {
-    const T v = x[(row0 + packed_byte(p.pinv4, k)) * ld_x + cc];
-    if constexpr (sizeof(T) == 2) z[k] = u2f((uint32_t)__builtin_bit_cast(unsigned short, v) << 16);
-    else z[k] = v;
-  }
+  for (int k = 0; k < 32; ++k) z[k] = u2f(f2u(z[k]) ^ (((in_flip >> k) & 1u) << 31));
 #pragma unroll
   for (int h = 1; h < 32; h <<= 1) {
 #pragma unroll
@@ -518,12 +509,73 @@ __global__ __launch_bounds__(256) void hadamard_kernel(const T* __restrict__ x, 
     }
   }
 #pragma unroll
-  for (int k = 0; k < 32; ++k) {
-    float q = div_sqrt32_signed(z[k], ((p.sign_mask >> k) & 1u) << 31);
-    T o;
-    if constexpr (sizeof(T) == 2) o = __builtin_bit_cast(T, (unsigned short)f32_to_bf16_bits(q));
-    else o = q;
-    y[(row0 + packed_byte(p.pinv4, k)) * ld_y + cc] = o;
+  for (int k = 0; k < 32; ++k) z[k] = div_sqrt32_signed(z[k], ((out_flip >> k) & 1u) << 31);
+}
+
+template <typename T>
+__device__ __forceinline__ float load_as_f32(const T* q) {
+  if constexpr (sizeof(T) == 2) return u2f((uint32_t)__builtin_bit_cast(unsigned short, *q) << 16);
+  else return *q;
+}
+
+template <typename T>
+__device__ __forceinline__ void store_from_f32(T* q, float v) {
+  if constexpr (sizeof(T) == 2) *q = __builtin_bit_cast(T, (unsigned short)f32_to_bf16_bits(v));
+  else *q = v;
+}
+
+// Standalone transform along the rows' index (W or W^T from the left): thread t owns one column, loads the 32 rows of
+// a block in permuted order, runs the same butterfly as the fused quantizer and writes each position back to the row
+// it came from.
+template <typename T>
+__global__ __launch_bounds__(256) void hadamard_kernel(const T* __restrict__ x, int64_t ld_x, T* __restrict__ y, int64_t ld_y, int C,
+                                                       const QuantParams p, uint32_t in_flip, uint32_t out_flip) {
+  const int cc = blockIdx.x * 256 + threadIdx.x;
+  if (cc >= C) return;
+  const int64_t row0 = (int64_t)blockIdx.y * 32;
+  float z[32];
+#pragma unroll
+  for (int k = 0; k < 32; ++k) z[k] = load_as_f32(&x[(row0 + packed_byte(p.pinv4, k)) * ld_x + cc]);
+  hadamard32(z, in_flip, out_flip);
+#pragma unroll
+  for (int k = 0; k < 32; ++k) store_from_f32(&y[(row0 + packed_byte(p.pinv4, k)) * ld_y + cc], z[k]);
+}
+
+// Standalone transform along the columns' index (W or W^T from the right): a workgroup takes 256 chunks of 32
+// neighbouring elements of a row.  Half a wave moves one chunk between memory and LDS (whole 128- or 64-byte
+// segments); then thread t picks chunk t out of LDS in permuted order (pitch 33 dwords: no bank conflicts either
+// way), runs the butterfly and puts the results back for the same half-wave pattern to store.
+template <typename T>
+__global__ __launch_bounds__(256) void hadamard_rows_kernel(const T* __restrict__ x, int64_t ld_x, T* __restrict__ y, int64_t ld_y,
+                                                            int chunks_per_row, int64_t n_chunks, const QuantParams p,
+                                                            uint32_t in_flip, uint32_t out_flip) {
+  __shared__ float tile[256 * 33];
+  const int tid = threadIdx.x, j = tid & 31, grp = tid >> 5;
+  const int64_t base = (int64_t)blockIdx.x * 256;
+  const int64_t g0 = base + grp * 32;   // the first of the 32 chunks this half-wave moves
+  int64_t row = g0 / chunks_per_row;
+  int ch = (int)(g0 - row * chunks_per_row);
+  {
+    int64_t r = row;
+    int c = ch;
+    for (int i = 0; i < 32; ++i) {
+      if (g0 + i < n_chunks) tile[(grp * 32 + i) * 33 + j] = load_as_f32(&x[r * ld_x + c * 32 + j]);
+      if (++c == chunks_per_row) { c = 0; ++r; }
+    }
+  }
+  __syncthreads();
+  if (base + tid < n_chunks) {
+    float z[32];
+#pragma unroll
+    for (int k = 0; k < 32; ++k) z[k] = tile[tid * 33 + packed_byte(p.pinv4, k)];
+    hadamard32(z, in_flip, out_flip);
+#pragma unroll
+    for (int k = 0; k < 32; ++k) tile[tid * 33 + packed_byte(p.pinv4, k)] = z[k];
+  }
+  __syncthreads();
+  for (int i = 0; i < 32; ++i) {
+    if (g0 + i < n_chunks) store_from_f32(&y[row * ld_y + ch * 32 + j], tile[(grp * 32 + i) * 33 + j]);
+    if (++ch == chunks_per_row) { ch = 0; ++row; }
   }
 }
 
@@ -731,23 +783,45 @@ extern "C" int alto_mxfp4_philox_advance(uint64_t* philox_state, uint64_t words,
   return check_launch("philox_advance");
 }
 
-extern "C" int alto_mxfp4_hadamard(const void* x, int dtype, int64_t M, int64_t C, int64_t ld_x, void* y, int64_t ld_y,
-                                   const int8_t* signs, const uint8_t* perm, void* stream) {
+extern "C" int alto_mxfp4_hadamard_apply(const void* x, int dtype, int64_t M, int64_t C, int64_t ld_x, void* y, int64_t ld_y,
+                                         const int8_t* signs, const uint8_t* perm, int inverse, int left_mul, void* stream) {
   using namespace alto;
   ALTO_REQUIRE(x && y, "hadamard: NULL pointer");
   ALTO_REQUIRE(dtype == ALTO_DT_BF16 || dtype == ALTO_DT_F32, "hadamard: bad dtype %d", dtype);
-  ALTO_REQUIRE(M >= 0 && C >= 0 && M % 32 == 0, "hadamard: M (%lld) must be a multiple of 32", (long long)M);
+  ALTO_REQUIRE(M >= 0 && C >= 0, "hadamard: negative size");
+  ALTO_REQUIRE(!left_mul || M % 32 == 0, "hadamard: M (%lld) must be a multiple of 32", (long long)M);
+  ALTO_REQUIRE(left_mul || C % 32 == 0, "hadamard: C (%lld) must be a multiple of 32 for a multiplication from the right", (long long)C);
   ALTO_REQUIRE(ld_x >= C && ld_y >= C, "hadamard: row stride smaller than C");
-  ALTO_REQUIRE(M / 32 <= 65535 && C < (1ll << 31), "hadamard: size out of range");
+  ALTO_REQUIRE(C < (1ll << 31), "hadamard: size out of range");
   QuantParams p{};
   int rc = fill_hadamard(p, signs, perm, "hadamard");
   if (rc != ALTO_MXFP4_OK) return rc;
   if (M == 0 || C == 0) return ALTO_MXFP4_OK;
-  dim3 grid((unsigned)((C + 255) / 256), (unsigned)(M / 32));
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-  if (dtype == ALTO_DT_BF16)
-    hipLaunchKernelGGL(hadamard_kernel<__bf16>, grid, dim3(256), 0, st, (const __bf16*)x, ld_x, (__bf16*)y, ld_y, (int)C, p);
-  else
-    hipLaunchKernelGGL(hadamard_kernel<float>, grid, dim3(256), 0, st, (const float*)x, ld_x, (float*)y, ld_y, (int)C, p);
+  if (left_mul) {
+    // y = W x (or W^T x): out[i] = sum_j W[i][j] x[j]
+    ALTO_REQUIRE(M / 32 <= 65535, "hadamard: size out of range");
+    const uint32_t in_flip = inverse ? p.sign_mask : 0u, out_flip = inverse ? 0u : p.sign_mask;
+    dim3 grid((unsigned)((C + 255) / 256), (unsigned)(M / 32));
+    if (dtype == ALTO_DT_BF16)
+      hipLaunchKernelGGL(hadamard_kernel<__bf16>, grid, dim3(256), 0, st, (const __bf16*)x, ld_x, (__bf16*)y, ld_y, (int)C, p, in_flip, out_flip);
+    else
+      hipLaunchKernelGGL(hadamard_kernel<float>, grid, dim3(256), 0, st, (const float*)x, ld_x, (float*)y, ld_y, (int)C, p, in_flip, out_flip);
+  } else {
+    // y = x W: out[j] = sum_i x[i] W[i][j] = (W^T x^T)[j], so the row vector sees the transpose of what a column sees
+    const uint32_t in_flip = inverse ? 0u : p.sign_mask, out_flip = inverse ? p.sign_mask : 0u;
+    const int64_t n_chunks = M * (C / 32);
+    ALTO_REQUIRE((n_chunks + 255) / 256 < (1ll << 31), "hadamard: size out of range");
+    dim3 grid((unsigned)((n_chunks + 255) / 256));
+    if (dtype == ALTO_DT_BF16)
+      hipLaunchKernelGGL(hadamard_rows_kernel<__bf16>, grid, dim3(256), 0, st, (const __bf16*)x, ld_x, (__bf16*)y, ld_y, (int)(C / 32), n_chunks, p, in_flip, out_flip);
+    else
+      hipLaunchKernelGGL(hadamard_rows_kernel<float>, grid, dim3(256), 0, st, (const float*)x, ld_x, (float*)y, ld_y, (int)(C / 32), n_chunks, p, in_flip, out_flip);
+  }
   return check_launch("hadamard");
+}
+
+extern "C" int alto_mxfp4_hadamard(const void* x, int dtype, int64_t M, int64_t C, int64_t ld_x, void* y, int64_t ld_y,
+                                   const int8_t* signs, const uint8_t* perm, void* stream) {
+  return alto_mxfp4_hadamard_apply(x, dtype, M, C, ld_x, y, ld_y, signs, perm, 0, 1, stream);
 }

@@ -39,11 +39,10 @@ class HadamardTransform:
         return w0[p][:, p]
 
     def __call__(self, value: torch.Tensor, inverse: bool = False, left_mul: bool = False) -> torch.Tensor:
-        """``(W @ value.view(M/32, 32, C)) / sqrt(32)`` in the input dtype (left_mul only, as the MXFP4 path uses it)."""
-        if inverse or not left_mul:
-            raise NotImplementedError("only left_mul=True, inverse=False is used by the MXFP4 path and implemented")
-        from .quantization import hadamard_left  # local import: quantization imports this module
-        return hadamard_left(value, self)
+        """``W @ value`` (``left_mul``) or ``value @ W`` over blocks of 32, divided by ``sqrt(32)``, in the input dtype;
+        ``inverse`` uses ``W.T`` (transform.py:115-142).  The MXFP4 path itself only uses ``left_mul=True``."""
+        from .quantization import hadamard_apply  # local import: quantization imports this module
+        return hadamard_apply(value, self, inverse=inverse, left_mul=left_mul)
 
 
 class HadamardFactory:

@@ -325,20 +325,36 @@ def quantize_rowcol(
     return rc[0], rs[0], cc[0].transpose(0, 1), cs[0].transpose(0, 1)
 
 
+def hadamard_apply(x: torch.Tensor, h: HadamardTransform, inverse: bool = False, left_mul: bool = False) -> torch.Tensor:
+    """``h(x, inverse, left_mul)`` of the reference (transform.py:115-142) in the dtype of ``x``.
+
+    ``left_mul``: ``W @ x`` over the last two dims in blocks of 32 rows; otherwise ``x @ W`` in blocks of 32 along the
+    last dim.  ``inverse`` multiplies with ``W.T`` instead.  Leading dims are batch dims.
+    """
+    assert x.dtype in (torch.float32, torch.bfloat16)
+    rt.require_gpu(x)
+    if left_mul:
+        torch._check(x.dim() >= 2 and x.shape[-2] % 32 == 0, lambda: f"left_mul needs a row count that is a multiple of 32, got {tuple(x.shape)}")
+    else:
+        torch._check(x.dim() >= 1 and x.shape[-1] % 32 == 0, lambda: f"the last dim must be a multiple of 32, got {tuple(x.shape)}")
+    C = x.shape[-1]
+    x2 = x.reshape(-1, C)   # whole blocks of 32 rows stay whole: every matrix has a multiple of 32 rows
+    if x2.stride(-1) != 1 and x2.numel():
+        x2 = x2.contiguous()
+    y = torch.empty(x2.shape, dtype=x.dtype, device=x.device)
+    M = x2.shape[0]
+    if M and C:
+        rc = rt.lib().alto_mxfp4_hadamard_apply(x2.data_ptr(), rt.dtype_code(x.dtype), M, C, x2.stride(0) if M > 1 else C, y.data_ptr(), C,
+                                                h.signs.data_ptr(), None if h.perm is None else h.perm.data_ptr(),
+                                                int(bool(inverse)), int(bool(left_mul)), rt.stream_ptr(x.device))
+        check(rc, "alto_mxfp4_hadamard_apply")
+    return y.reshape(x.shape)
+
+
 def hadamard_left(x: torch.Tensor, h: HadamardTransform) -> torch.Tensor:
     """``h(x, left_mul=True)``: the transform along dim 0 in blocks of 32 rows, output in the dtype of ``x``."""
-    assert x.dim() == 2 and x.dtype in (torch.float32, torch.bfloat16)
-    rt.require_gpu(x)
-    torch._check(x.shape[0] % 32 == 0)
-    xc = x if x.stride(-1) == 1 else x.contiguous()
-    y = torch.empty(x.shape, dtype=x.dtype, device=x.device)
-    M, C = x.shape
-    if M == 0 or C == 0:
-        return y
-    rc = rt.lib().alto_mxfp4_hadamard(xc.data_ptr(), rt.dtype_code(x.dtype), M, C, xc.stride(0), y.data_ptr(), y.stride(0),
-                                      h.signs.data_ptr(), None if h.perm is None else h.perm.data_ptr(), rt.stream_ptr(x.device))
-    check(rc, "alto_mxfp4_hadamard")
-    return y
+    assert x.dim() == 2
+    return hadamard_apply(x, h, inverse=False, left_mul=True)
 
 
 def convert_from_mxfp4(

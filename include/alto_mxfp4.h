@@ -169,6 +169,17 @@ int alto_mxfp4_hadamard(const void* x, int dtype, int64_t M, int64_t C, int64_t 
                         const int8_t* signs, const uint8_t* perm, void* stream);
 
 /*
+ * The other three forms of HadamardTransform.__call__(value, inverse, left_mul) (transform.py:115-142), same
+ * arithmetic (fixed butterfly order, one division by float32(sqrt(32)), one rounding to `dtype`):
+ *   left_mul = 1: y[32b + i][c] = sum_j V[i][j] x[32b + j][c]      (M % 32 == 0)
+ *   left_mul = 0: y[r][32b + j] = sum_i x[r][32b + i] V[i][j]      (C % 32 == 0)
+ * with V = W, or V = W^T when `inverse` is set (W is orthogonal up to the factor 32, so W^T / sqrt(32) undoes
+ * W / sqrt(32)).  alto_mxfp4_hadamard is the case inverse = 0, left_mul = 1.
+ */
+int alto_mxfp4_hadamard_apply(const void* x, int dtype, int64_t M, int64_t C, int64_t ld_x, void* y, int64_t ld_y,
+                              const int8_t* signs, const uint8_t* perm, int inverse, int left_mul, void* stream);
+
+/*
  * Dequantizer.  Replaces _convert_from_mxfp4_kernel
  * (alto/kernels/fp4/mxfp4/mxfp_quantization.py:342-407, 487-545).
  * codes [R][C/2] dense, scales [R][C/32] (1D) or [R/32][C/32] (2D) dense;

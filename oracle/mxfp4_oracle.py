@@ -66,7 +66,7 @@ __all__ = [
     "BLOCK", "SQRT32_F32", "E2M1_GRID",
     "e8m0_from_absmax", "block_scales", "encode_e2m1_rne", "encode_e2m1_sr", "decode_e2m1",
     "pack_nibbles", "unpack_nibbles", "quantize", "dequantize",
-    "hadamard_matrix", "rht_left", "rht_left_dense",
+    "hadamard_matrix", "rht_left", "rht_left_dense", "rht", "rht_dense",
     "gemm_ref", "linear_forward_ref", "linear_backward_ref",
     "indices_from_offsets", "grouped_gemm_ref", "grouped_gemm_dx_ref", "grouped_gemm_dw_ref",
     "rel_frobenius", "dge_bwd_ref", "weight_grid_values", "E2M1_BREAK_POINTS",
@@ -392,6 +392,55 @@ def rht_left(x: torch.Tensor, signs: torch.Tensor, perm: Optional[torch.Tensor])
     y = z[:, p, :] * signs.float()[p].reshape(1, n, 1)
     y = y / torch.tensor(SQRT32_F32, dtype=torch.float32)
     return y.reshape(M, C).to(x.dtype)
+
+
+def rht(x: torch.Tensor, signs: torch.Tensor, perm: Optional[torch.Tensor], inverse: bool = False, left_mul: bool = False) -> torch.Tensor:
+    """All four forms of ``HadamardTransform.__call__`` (transform.py:115-142), FIXED summation order.
+
+    ``left_mul``: ``V @ x`` over the last two dims in blocks of 32 rows, else ``x @ V`` in blocks of 32 along the last
+    dim (matrix.py:152-161 unflattens the larger operand), ``V = W`` or ``W.T`` (``inverse``, transform.py:130-131).
+    With ``W[i, j] = Q[p[i]] H[p[i], p[j]]`` every form is: scatter the 32 inputs to ``z[p[j]]``, butterfly as in
+    :func:`rht_left`, gather ``z[p[i]]``; ``Q`` multiplies the gathered outputs where the output index is W's row index
+    (``W @ x`` and ``x @ W.T``) and the scattered inputs where the input index is (``W.T @ x`` and ``x @ W``).
+    """
+    if not left_mul:
+        return rht(x.transpose(-1, -2) if x.dim() >= 2 else x.reshape(-1, 1), signs, perm, not inverse, True).transpose(-1, -2).reshape(x.shape)
+    shape = x.shape
+    M, C = shape[-2], shape[-1]
+    assert M % BLOCK == 0
+    n = BLOCK
+    p = torch.arange(n) if perm is None else perm.long()
+    q = signs.float()[p].reshape(1, n, 1)
+    xb = x.float().reshape(-1, n, C)
+    z = torch.empty_like(xb)
+    z[:, p, :] = xb * q if inverse else xb
+    h = 1
+    while h < n:
+        zz = z.reshape(z.shape[0], n // (2 * h), 2, h, C)
+        a = zz[:, :, 0].clone()
+        b = zz[:, :, 1].clone()
+        zz[:, :, 0] = a + b
+        zz[:, :, 1] = a - b
+        h *= 2
+    y = z[:, p, :]
+    if not inverse:
+        y = y * q
+    y = y / torch.tensor(SQRT32_F32, dtype=torch.float32)
+    return y.reshape(shape).to(x.dtype)
+
+
+def rht_dense(x: torch.Tensor, signs: torch.Tensor, perm: Optional[torch.Tensor], inverse: bool = False, left_mul: bool = False,
+              dtype=torch.float32) -> torch.Tensor:
+    """The reference's own formulation (transform.py:125-142 with matrix.py:152-161): dense matmuls, the backend's order."""
+    W = hadamard_matrix(signs, perm).to(dtype)
+    if inverse:
+        W = W.T
+    v = x.to(dtype)
+    if left_mul:
+        y = (W @ v.unflatten(-2, (v.shape[-2] // BLOCK, BLOCK))).flatten(-3, -2)
+    else:
+        y = (v.unflatten(-1, (v.shape[-1] // BLOCK, BLOCK)) @ W).flatten(-2, -1)
+    return y / torch.tensor(SQRT32_F32, dtype=torch.float32).to(dtype)
 
 
 def rht_left_dense(x: torch.Tensor, signs: torch.Tensor, perm: Optional[torch.Tensor], dtype=torch.float32) -> torch.Tensor:

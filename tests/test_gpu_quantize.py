@@ -127,6 +127,49 @@ def test_hadamard_standalone_bit_exact(m, dtype, shape):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("inverse", [False, True])
+@pytest.mark.parametrize("left_mul", [False, True])
+@pytest.mark.parametrize("shape", [(32, 32), (64, 96), (3, 64, 2880), (1, 32), (5, 7, 64), (2, 2, 96, 40), (700, 2048)])
+def test_hadamard_every_form_bit_exact(m, dtype, inverse, left_mul, shape):
+    """HadamardTransform.__call__(value, inverse, left_mul) (transform.py:115-142), batch dims included."""
+    if left_mul and (len(shape) < 2 or shape[-2] % 32):
+        pytest.skip("left_mul needs whole blocks of 32 rows")
+    if not left_mul and shape[-1] % 32:
+        pytest.skip("right multiplication needs whole blocks of 32 columns")
+    signs, perm = hadamard_from_seed(77)
+    x = laplace(shape, 1e-2, dtype, seed=5)
+    for sg, pm in ((signs, perm), (signs, None)):
+        h = m.HadamardTransform(sg, pm)
+        y = h(x.to(DEV), inverse=inverse, left_mul=left_mul)
+        assert y.dtype == dtype and y.shape == x.shape
+        assert_bytes_equal(y.cpu(), O.rht(x, sg, pm, inverse, left_mul), f"hadamard inverse={inverse} left_mul={left_mul}")
+    yd = O.rht_dense(x, signs, perm, inverse, left_mul, torch.float64)
+    eps = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -24
+    sum_err = 2.0 ** -21 * float(x.abs().max()) * 32 ** 0.5
+    yp = m.HadamardTransform(signs, perm)(x.to(DEV), inverse=inverse, left_mul=left_mul)
+    assert bool(((yp.cpu().double() - yd).abs() <= eps * yd.abs() + sum_err).all())
+
+
+def test_hadamard_strided_input_and_bad_shapes(m):
+    signs, perm = hadamard_from_seed(78)
+    h = m.HadamardTransform(signs, perm)
+    base = laplace((64, 256), 1e-2, torch.float32, seed=6)
+    view = base[:, 32:160]                       # row stride 256, 128 columns
+    for inverse in (False, True):
+        for left_mul in (False, True):
+            got = h(base.to(DEV)[:, 32:160], inverse=inverse, left_mul=left_mul)
+            assert_bytes_equal(got.cpu(), O.rht(view, signs, perm, inverse, left_mul), "strided view")
+    tr = base.t()                                # last dim not contiguous
+    assert_bytes_equal(h(base.to(DEV).t()).cpu(), O.rht(tr, signs, perm, False, False), "transposed view")
+    with pytest.raises(RuntimeError):
+        h(torch.zeros(33, 64, device=DEV), left_mul=True)
+    with pytest.raises(RuntimeError):
+        h(torch.zeros(32, 48, device=DEV))
+    e = h(torch.zeros(0, 64, device=DEV))
+    assert e.shape == (0, 64)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("use_sr", [False, True])
 @pytest.mark.parametrize("use_h", [False, True])
 @pytest.mark.parametrize("clip_mode", ["none", "static"])

@@ -94,8 +94,8 @@ def test_hadamard_factory_matches_reference_draw_order():
     assert torch.equal(t.weight, O.hadamard_matrix(signs, perm))
     t2 = HadamardFactory.create_transform()          # the class-level generator advances between calls
     assert not (torch.equal(t2.signs, t.signs) and torch.equal(t2.perm, t.perm))
-    with pytest.raises(NotImplementedError):
-        t(torch.zeros(32, 8), left_mul=False)
+    with pytest.raises(RuntimeError, match="MI355X only"):   # no CPU path behind the transform
+        t(torch.zeros(32, 32), left_mul=False)
 
 
 def test_training_op_config():

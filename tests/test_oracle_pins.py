@@ -303,6 +303,42 @@ def test_rht_butterfly_vs_dense_fp64():
     assert torch.equal(O.rht_left(xi, signs, perm), O.rht_left_dense(xi, signs, perm, torch.float32).bfloat16())
 
 
+@pytest.mark.parametrize("inverse", [False, True])
+@pytest.mark.parametrize("left_mul", [False, True])
+def test_rht_all_four_forms_vs_the_dense_formulation(inverse, left_mul):
+    """The butterfly forms against transform.py:125-142 restated with dense matmuls (W[perm][:, perm], .T for the
+    inverse, the 32-blocks unflattened as matrix.py:152-161 does).  A misplaced sign vector, a swapped perm / inverse
+    perm or a transposed operand changes whole outputs, far beyond the tolerance."""
+    g = torch.Generator().manual_seed(15)
+    signs = torch.randint(0, 2, (32,), generator=g) * 2 - 1
+    perm = torch.randperm(32, generator=g)
+    x = torch.randn(3, 64, 96, generator=g)
+    y = O.rht(x, signs, perm, inverse, left_mul)
+    yd = O.rht_dense(x, signs, perm, inverse, left_mul, torch.float64)
+    assert float((y.double() - yd).abs().max()) < 2e-6
+    assert float((O.rht(x, signs, perm, not inverse, left_mul).double() - yd).abs().max()) > 0.1   # the check has teeth
+    # sums that are exact in fp32 come out identical whatever the order; bf16 output rounds once
+    xi = torch.randint(-8, 9, (64, 96), generator=g).bfloat16()
+    assert torch.equal(O.rht(xi, signs, perm, inverse, left_mul), O.rht_dense(xi, signs, perm, inverse, left_mul, torch.float32).bfloat16())
+    if left_mul and not inverse:
+        assert torch.equal(O.rht(x[0], signs, perm, False, True), O.rht_left(x[0], signs, perm))
+
+
+def test_rht_inverse_undoes_forward():
+    """W is 32 times an orthogonal matrix: (W.T / s)(W / s) x = x * 32 / s^2 with s = float32(sqrt 32), for either side."""
+    g = torch.Generator().manual_seed(16)
+    signs = torch.randint(0, 2, (32,), generator=g) * 2 - 1
+    perm = torch.randperm(32, generator=g)
+    x = torch.randn(64, 64, generator=g, dtype=torch.float64)
+    k = 32.0 / float(O.SQRT32_F32) ** 2
+    for left_mul in (False, True):
+        back = O.rht_dense(O.rht_dense(x, signs, perm, False, left_mul, torch.float64), signs, perm, True, left_mul, torch.float64)
+        assert torch.allclose(back, x * k, atol=1e-12)
+        xf = x.float()
+        back32 = O.rht(O.rht(xf, signs, perm, False, left_mul), signs, perm, True, left_mul)
+        assert float((back32.double() - x).abs().max()) < 1e-5
+
+
 def test_rht_preserves_wgrad_product():
     g = torch.Generator().manual_seed(6)
     signs = torch.randint(0, 2, (32,), generator=g) * 2 - 1
