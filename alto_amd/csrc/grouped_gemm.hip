@@ -320,12 +320,15 @@ __global__ __launch_bounds__(GT_THREADS) void grouped_tiled_kernel(OperandView A
 constexpr int GT_DW_MAX_GROUPS = 32768;
 constexpr int GT_DW_LDS_BYTES = GT_LDS_BYTES + 2 * (GT_DW_MAX_GROUPS / 64) * 8;   // + 8 KB of masks
 
+// The body of the kernel as a function of its own because of the `__restrict__` on the output: inlining then marks every
+// memory operation in here, the global->LDS loads of the K loop included, as not aliasing the output, and only with that
+// mark does the compiler's wait insertion keep those loads in flight across the LDS reads that follow them (unmarked, it
+// puts an `s_waitcnt vmcnt(0)` before the next fragment read, twice per stage, and the loop runs at the load latency).
 template <typename OutT>
-__global__ __launch_bounds__(GT_THREADS) void grouped_dw_tiled_kernel(OperandView P, OperandView Q, int64_t NP, int64_t NQ,
-                                                                      const int32_t* offs, const int32_t* group_expert, int num_groups,
-                                                                      int64_t M_total, OutT* dw, int64_t s_e, int64_t ld, float out_scale,
-                                                                      int tiles_p, int tiles_q, int xq_log2) {
-  extern __shared__ __align__(16) uint8_t smem[];
+__device__ __forceinline__ void grouped_dw_tile(const OperandView& P, const OperandView& Q, int64_t NP, int64_t NQ,
+                                                const int32_t* offs, const int32_t* group_expert, int num_groups,
+                                                int64_t M_total, OutT* __restrict__ dw, int64_t s_e, int64_t ld, float out_scale,
+                                                int tiles_p, int tiles_q, int xq_log2, uint8_t* smem) {
   const int e = blockIdx.y;
   int tm, tn;
   {
@@ -432,6 +435,15 @@ __global__ __launch_bounds__(GT_THREADS) void grouped_dw_tiled_kernel(OperandVie
   }
   TileArgs ta{P, Q, (int64_t)tm * GT_TM, (int64_t)tn * GT_TN, 0, NP, NQ, 0, out_scale, 0, 0, 0, 0, 0, 0};
   gemm_tile_store<OutT>(ta, acc, dw + e * s_e, ld, smem);
+}
+
+template <typename OutT>
+__global__ __launch_bounds__(GT_THREADS) void grouped_dw_tiled_kernel(OperandView P, OperandView Q, int64_t NP, int64_t NQ,
+                                                                      const int32_t* offs, const int32_t* group_expert, int num_groups,
+                                                                      int64_t M_total, OutT* dw, int64_t s_e, int64_t ld, float out_scale,
+                                                                      int tiles_p, int tiles_q, int xq_log2) {
+  extern __shared__ __align__(16) uint8_t smem[];
+  grouped_dw_tile<OutT>(P, Q, NP, NQ, offs, group_expert, num_groups, M_total, dw, s_e, ld, out_scale, tiles_p, tiles_q, xq_log2, smem);
 }
 
 // upper bound on the number of passes: every band is one, every group start inside a band adds one, plus the unrouted head and tail
