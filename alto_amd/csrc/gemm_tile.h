@@ -230,8 +230,9 @@ struct TileLoader {
 // (K a multiple of 512) and s_k0 == 0: then every 16-byte scale block of a row lies inside the row.  KTAIL = true
 // handles any G and any start inside the scale rows (a reduction over a sub-range of K).  Requirements
 // checked by the host: unit-stride scale rows, operand extents below 2^31 bytes.  Every thread of the workgroup must
-// call it; it may be called again (same or other operands) to keep accumulating.
-template <bool KTAIL>
+// call it; it may be called again (same or other operands) to keep accumulating.  ODD_STAGES: a last 512-K block whose
+// second 256-K stage lies wholly beyond K runs its first stage only (needs KTAIL).
+template <bool KTAIL, bool ODD_STAGES = false>
 __device__ __forceinline__ void gemm_tile_mainloop(const TileArgs& ta, TileAcc& acc, uint8_t* smem) {
   TileLoader ld;
   v4i_t sraw;   // scale bytes of a later block, as loaded
@@ -383,7 +384,10 @@ __device__ __forceinline__ void gemm_tile_mainloop(const TileArgs& ta, TileAcc& 
   read_scales(reinterpret_cast<const uint8_t*>(sscale), sa, sb);
 
   // ---- main loop: one iteration = one 512-K block = 2 macro stages
-  for (int kb = 0; kb < KB; ++kb) {
+  const int NS = (ta.G + 7) / 8;         // macro stages that hold any K at all
+  const int KBF = ODD_STAGES ? NS / 2 : KB;
+  int kb = 0;
+  for (; kb < KBF; ++kb) {
     stage(std::integral_constant<int, 0>{}, 2 * kb, kb);
     stage(std::integral_constant<int, 1>{}, 2 * kb + 1, kb);
 #pragma unroll
@@ -391,6 +395,7 @@ __device__ __forceinline__ void gemm_tile_mainloop(const TileArgs& ta, TileAcc& 
 #pragma unroll
     for (int u = 0; u < 2; ++u) { sb[u][0] = sb_next[u][0]; sb[u][1] = sb_next[u][1]; }
   }
+  if (ODD_STAGES && (NS & 1)) stage(std::integral_constant<int, 0>{}, 2 * kb, kb);   // the last block's second stage lies wholly beyond K
   // loads of the (zero-filled) stages past the end may still be landing in the ring the epilogue reuses
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
@@ -477,11 +482,13 @@ __device__ __forceinline__ void gemm_tile_store(const TileArgs& ta, TileAcc& acc
   }
 }
 
-template <typename OutT, bool KTAIL>
+// ODD: the K range ends in the first 256-K stage of its last 512-K block (an odd number of stages): that block's second
+// stage is not run.  A launch-time choice because the extra exit makes the even case slower when compiled in.
+template <typename OutT, bool KTAIL, bool ODD = false>
 __device__ __forceinline__ void gemm_tile_256x256(const TileArgs& ta, OutT* __restrict__ c, int64_t ldc, uint8_t* smem) {
   TileAcc acc;
   gemm_tile_zero(acc);
-  gemm_tile_mainloop<KTAIL>(ta, acc, smem);
+  gemm_tile_mainloop<KTAIL, ODD>(ta, acc, smem);
   gemm_tile_store<OutT>(ta, acc, c, ldc, smem);
 }
 

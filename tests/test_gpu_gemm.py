@@ -49,7 +49,7 @@ def test_gemm_matches_dequant_matmul(m, shape, use_2dblock_a, use_2dblock_b, tra
 
 
 @pytest.mark.parametrize("shape", [(64, 96, 160), (100, 72, 96), (33, 40, 32), (256, 256, 2880), (200, 136, 544), (128, 128, 992),
-                                   (300, 264, 512), (136, 256, 1312)])
+                                   (300, 264, 512), (136, 256, 1312), (256, 128, 768), (128, 256, 1792), (264, 136, 1376)])
 def test_gemm_ragged_shapes_and_kpack_false(m, shape):
     M, N, K = shape
     a = randn_outliers((M, K), torch.bfloat16, seed=3)
@@ -327,6 +327,33 @@ def test_grouped_gemm_ragged_offsets_and_padding(m):
     dw_ref = O.grouped_gemm_dw_ref(gqm, gsm, aqm, asm, idx, E, trans_weights=False)
     assert O.rel_frobenius(wg.grad.cpu(), dw_ref) < 4e-3
     assert bool((wg.grad[1] == 0).all()), "an expert without tokens gets a zero gradient"
+
+
+def test_grouped_tiled_odd_stage_counts(m):
+    """Reductions that end in the first 256-wide stage of their last 512-wide block, in all three tiled kernels: forward over
+    K = 1280 (5 stages), dX over N = 768 (3 stages), dW over token runs of 2, 2 and 3 stages (the last two start inside a line)."""
+    E, N, K = 4, 768, 1280
+    sizes = [320, 0, 224, 544]
+    ends = torch.tensor(sizes).cumsum(0).to(torch.int32)
+    M = int(ends[-1])
+    a, w = _grouped_inputs(M, N, K, E, seed=150)
+    w_kn = w.transpose(1, 2).contiguous()
+    go = randn_outliers((M, N), torch.bfloat16, seed=152) / (M * N)
+    ag = a.to(DEV).requires_grad_(True)
+    wg = w_kn.to(DEV).requires_grad_(True)
+    out = m._quantize_then_mxfp_scaled_grouped_mm(ag, wg, ends.to(DEV), False, True, False, False, False, "none", False)
+    out.backward(go.to(DEV))
+    idx = O.indices_from_offsets(ends)
+    aq, as_ = O.quantize(a)
+    wq, ws = O.quantize(w, axis=-1, is_2d_block=True)
+    assert O.rel_frobenius(out.detach().cpu(), O.grouped_gemm_ref(aq, as_, wq, ws, idx)) < 4e-3
+    gq, gs = O.quantize(go)
+    assert O.rel_frobenius(ag.grad.cpu(), O.grouped_gemm_dx_ref(gq, gs, wq, ws, idx, k_pack_w=False)) < 4e-3
+    gqm, gsm = O.quantize(go, axis=0)
+    aqm, asm = O.quantize(a, axis=0)
+    dw_ref = O.grouped_gemm_dw_ref(gqm, gsm, aqm, asm, idx, E, trans_weights=False)
+    assert O.rel_frobenius(wg.grad.cpu(), dw_ref) < 4e-3
+    assert bool((wg.grad[1] == 0).all())
 
 
 def test_grouped_unaligned_rows_forward(m):
