@@ -69,12 +69,22 @@ def triton_attention_mxfp4(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, al
                            bias: Optional[torch.Tensor] = None, sm_scale: Optional[float] = None, dropout_p: float = 0.0,
                            cu_seqlens_q=0, cu_seqlens_k=0, max_seqlens_q: Optional[int] = None, max_seqlens_k: Optional[int] = None,
                            causal: bool = True, return_scores: bool = False, use_exp2: bool = True, layout: str = "bhsd"):
-    """(q, k, v) [B,H,S,D] -> (out bf16, softmax_lse fp32, exp_scores placeholder), as :1206-1239.
+    """(q, k, v) [B,H,S,D] (or [B,S,H,D] with ``layout="bshd"``) -> (out bf16 in the layout of q, softmax_lse fp32 [B,H,S],
+    exp_scores placeholder), as :1206-1239.
 
     ``use_exp2`` is accepted either way: both settings evaluate exp(x) as exp2(x * log2 e) on the GPU's exp unit.
     """
+    if layout == "bshd":
+        # [B, S, H, D] tensors: the same attention on the permuted views, result back in [B, S, H, D].  (The reference's
+        # wrapper has no consistent behaviour to reproduce here: it takes 2D blocks over (heads, head dim) of the tensor as
+        # given and then reads those scales with strides permuted as if they were per (32 rows, 32 of head dim),
+        # triton_flash_attention_mxfp4.py:68-77,1023-1025,1105-1107.)
+        out, lse, scores = triton_attention_mxfp4(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2), alibi_slopes, bias, sm_scale,
+                                                  dropout_p, cu_seqlens_q, cu_seqlens_k, max_seqlens_q, max_seqlens_k, causal, return_scores,
+                                                  use_exp2, "bhsd")
+        return out.transpose(1, 2), lse, scores
     if layout != "bhsd":
-        raise NotImplementedError(f"layout {layout!r}: only 'bhsd' is implemented (the layout ALTO's dispatch layer passes)")
+        raise NotImplementedError(f"layout {layout!r}: 'bhsd' and 'bshd' are implemented ('thd' packs variable-length sequences)")
     if alibi_slopes is not None or bias is not None:
         raise NotImplementedError("alibi slopes and bias are not implemented")
     if dropout_p != 0.0:

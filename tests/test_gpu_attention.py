@@ -132,10 +132,19 @@ def test_module_form_and_prequantised_entry(m):
         attn(q.to(DEV), k.to(DEV), v.to(DEV), attention_masks=object())
 
 
+def test_layout_bshd_is_the_same_attention_on_permuted_views(m):
+    q, k, v = (t.to(DEV) for t in _qkv(2, 4, 2, 128, 192, 64, 64, seed=9))      # [B, H, S, D]
+    o, lse, _ = m.triton_attention_mxfp4(q, k, v, causal=True)
+    qs, ks, vs = (t.transpose(1, 2).contiguous() for t in (q, k, v))            # [B, S, H, D]
+    o2, lse2, _ = m.triton_attention_mxfp4(qs, ks, vs, causal=True, layout="bshd")
+    assert o2.shape == qs.shape[:3] + (v.shape[-1],)
+    assert torch.equal(o2.transpose(1, 2), o) and torch.equal(lse2, lse)
+
+
 def test_rejected_arguments(m):
     q, k, v = (t.to(DEV) for t in _qkv(1, 2, 2, 64, 64, 64, 64, seed=1))
     with pytest.raises(NotImplementedError):
-        m.triton_attention_mxfp4(q, k, v, layout="bshd")
+        m.triton_attention_mxfp4(q, k, v, layout="thd")
     with pytest.raises(NotImplementedError):
         m.triton_attention_mxfp4(q, k, v, dropout_p=0.1)
     with pytest.raises(NotImplementedError):
