@@ -242,6 +242,14 @@ int alto_mxfp4_grouped_gemm(const uint8_t* a, int64_t lda, const uint8_t* a_scal
                             void* workspace, int64_t workspace_bytes, void* stream);
 
 /*
+ * Per-device set-up that the entry points otherwise do on first use: resolves, for the CURRENT device, the address of the
+ * library's built-in pass-list array.  Call it once per device (with that device current) before capturing a HIP graph
+ * that contains alto_mxfp4_grouped_gemm_noalloc.  Idempotent, thread-safe, allocates nothing.  No counterpart in the
+ * reference.
+ */
+int alto_mxfp4_init(void);
+
+/*
  * alto_mxfp4_grouped_gemm without the workspace argument, for callers that cannot allocate device memory (code under HIP
  * graph capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  The pass list
  * lives in a 1 MiB array that is part of the library's device code (one copy per GPU, held until the process ends), so
@@ -252,14 +260,6 @@ int alto_mxfp4_grouped_gemm(const uint8_t* a, int64_t lda, const uint8_t* a_scal
  * belongs to.  Its address is looked up on the first use on a device (a runtime query that may load the code object):
  * call alto_mxfp4_init() on every device beforehand when the first call would otherwise fall inside a stream capture.
  */
-/*
- * Per-device set-up that the entry points otherwise do on first use: resolves, for the CURRENT device, the address of the
- * library's built-in pass-list array.  Call it once per device (with that device current) before capturing a HIP graph
- * that contains alto_mxfp4_grouped_gemm_noalloc.  Idempotent, thread-safe, allocates nothing.  No counterpart in the
- * reference.
- */
-int alto_mxfp4_init(void);
-
 int alto_mxfp4_grouped_gemm_noalloc(const uint8_t* a, int64_t lda, const uint8_t* a_scales, int64_t a_ss_r, int64_t a_ss_k, int a_is_2d,
                                     const uint8_t* w, int64_t w_stride_e, int64_t ldw,
                                     const uint8_t* w_scales, int64_t ws_stride_e, int64_t ws_r, int64_t ws_k, int w_is_2d,
@@ -279,7 +279,9 @@ int64_t alto_mxfp4_grouped_gemm_workspace_bytes(int64_t M_total, int num_groups)
  * token ranges of two experts must be a multiple of 32 (the reference requires 128, cg_backward.py:443-447): an MX
  * block along the token dim cannot be split between experts.  The kernel checks this on the device (no host sync):
  * dW[e] of an expert with a misaligned boundary is written with NaN, never with a silently wrong gradient.
- * dW of experts with no tokens is written with zeros.  Element (e, n, k) lands at
+ * dW of experts with no tokens is written with zeros.  `offs` must be non-decreasing: every [offs[g], offs[g+1]) is
+ * taken as given (empty when it runs backwards), so ranges that overlap would credit a token to two experts.
+ * Element (e, n, k) lands at
  * dw[e * dw_stride_e + n * dw_stride_n + k * dw_stride_k].
  */
 int alto_mxfp4_grouped_gemm_dw(const uint8_t* go, int64_t ld_go, const uint8_t* go_scales, int64_t gs_r, int64_t gs_k, int go_is_2d,
