@@ -188,8 +188,15 @@ struct TileLoader {
     const int off = __builtin_amdgcn_readfirstlane(want < last ? want : last);
     raw = __builtin_amdgcn_raw_buffer_load_b128(rsrc_s, (int)soff, off, 0);
   }
-  template <bool KTAIL>
+  // FAST: the caller knows that the block lies inside its scale row and inside K (every block but the last of a
+  // reduction): the bytes are used as loaded
+  template <bool KTAIL, bool FAST = false>
   __device__ __forceinline__ void sfix(int kb, const v4i_t& L, uint32_t (&sreg)[4]) const {
+    if constexpr (KTAIL && FAST) {
+#pragma unroll
+      for (int d = 0; d < 4; ++d) sreg[d] = (uint32_t)L[d];
+      return;
+    }
     const int rem = G - kb * 16;   // wave-uniform
     if constexpr (!KTAIL) {
 #pragma unroll
@@ -258,9 +265,9 @@ __device__ __forceinline__ void gemm_tile_mainloop(const TileArgs& ta, TileAcc& 
 
   // LDS row layout (4 dwords): [h=0: K 0..255 | h=0: K 256..511 | h=1: K 0..255 | h=1: K 256..511], where the half-wave h
   // of the MFMA uses group 8 ms + 2 j + h at K step j of macro stage ms: byte j of dword 2 h + ms.
-  auto swrite = [&](int kb) {
+  auto swrite = [&](int kb, auto fastc) {
     uint32_t sreg[4];
-    ld.template sfix<KTAIL>(kb, sraw, sreg);
+    ld.template sfix<KTAIL, decltype(fastc)::value>(kb, sraw, sreg);
     uint32_t* row = sscale + (kb & 1) * GT_SCALE_BUF_DW + tid * GT_SCALE_PITCH;
     row[0] = __builtin_amdgcn_perm(sreg[1], sreg[0], 0x06040200u);   // groups 0, 2, 4, 6
     row[1] = __builtin_amdgcn_perm(sreg[3], sreg[2], 0x06040200u);   // groups 8, 10, 12, 14
@@ -333,7 +340,7 @@ __device__ __forceinline__ void gemm_tile_mainloop(const TileArgs& ta, TileAcc& 
   // loads of stage s+2 go out into it: half of them during the last step, half during the first step of the next
   // stage, one load per two MFMAs.  (A wave issues in order, and the address unit takes a 1 KB load about every 16
   // clocks per compute unit: a burst of eight loads per wave would hold the MFMAs behind it for a thousand clocks.)
-  auto stage = [&](auto msc, int s, int kb) {
+  auto stage = [&](auto msc, int s, int kb, auto fastc) {
     constexpr int MS = decltype(msc)::value;
     __builtin_amdgcn_s_setprio(2);
     ld.gload(smem, s + 1, MS ^ 1, 4, 8);
@@ -357,7 +364,7 @@ __device__ __forceinline__ void gemm_tile_mainloop(const TileArgs& ta, TileAcc& 
     asm volatile("s_barrier" ::: "memory");
     __builtin_amdgcn_s_setprio(3);
     if constexpr (MS == 0) {
-      swrite(kb + 1);          // block kb+1 -> the other scale buffer (last read at the end of block kb-1)
+      swrite(kb + 1, fastc);   // block kb+1 -> the other scale buffer (last read at the end of block kb-1)
       ld.template sload<KTAIL>(kb + 2, sraw);
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -376,7 +383,7 @@ __device__ __forceinline__ void gemm_tile_mainloop(const TileArgs& ta, TileAcc& 
   ld.init(ta);
   ld.template sload<KTAIL>(0, sraw);
   ld.gload(smem, 0, 0, 0, 8);
-  swrite(0);
+  swrite(0, std::false_type{});
   ld.template sload<KTAIL>(1, sraw);
   ld.gload(smem, 1, 1, 0, 4);   // the other half goes out in the first step of the loop
   asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)\n\ts_barrier" ::: "memory");   // all but stage 1's four loads
@@ -387,15 +394,27 @@ __device__ __forceinline__ void gemm_tile_mainloop(const TileArgs& ta, TileAcc& 
   const int NS = (ta.G + 7) / 8;         // macro stages that hold any K at all
   const int KBF = ODD_STAGES ? NS / 2 : KB;
   int kb = 0;
-  for (; kb < KBF; ++kb) {
-    stage(std::integral_constant<int, 0>{}, 2 * kb, kb);
-    stage(std::integral_constant<int, 1>{}, 2 * kb + 1, kb);
+  auto block = [&](int kb, auto fastc) {
+    stage(std::integral_constant<int, 0>{}, 2 * kb, kb, fastc);
+    stage(std::integral_constant<int, 1>{}, 2 * kb + 1, kb, std::false_type{});
 #pragma unroll
     for (int t = 0; t < 4; ++t) { sa[t][0] = sa_next[t][0]; sa[t][1] = sa_next[t][1]; }
 #pragma unroll
     for (int u = 0; u < 2; ++u) { sb[u][0] = sb_next[u][0]; sb[u][1] = sb_next[u][1]; }
+  };
+  if constexpr (KTAIL) {
+    // Iteration kb passes scale block kb + 1 on to LDS.  Only the last block that holds any K (KB - 1, passed on by
+    // iteration KB - 2) can reach past its row or past K and needs its bytes fixed; earlier ones are used as loaded,
+    // later ones are never read.  Three loops in a row rather than a test inside one: the tile needs nearly every
+    // register, and a branch inside the loop body makes the compiler spill.
+    const int kfull = KB - 2;
+    for (; kb < kfull && kb < KBF; ++kb) block(kb, std::true_type{});
+    for (; kb < kfull + 1 && kb < KBF; ++kb) block(kb, std::false_type{});
+    for (; kb < KBF; ++kb) block(kb, std::true_type{});
+  } else {
+    for (; kb < KBF; ++kb) block(kb, std::false_type{});
   }
-  if (ODD_STAGES && (NS & 1)) stage(std::integral_constant<int, 0>{}, 2 * kb, kb);   // the last block's second stage lies wholly beyond K
+  if (ODD_STAGES && (NS & 1)) stage(std::integral_constant<int, 0>{}, 2 * kb, kb, std::false_type{});   // the last block's second stage lies wholly beyond K
   // loads of the (zero-filled) stages past the end may still be landing in the ring the epilogue reuses
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
