@@ -237,9 +237,16 @@ struct TileLoader {
 // (K a multiple of 512) and s_k0 == 0: then every 16-byte scale block of a row lies inside the row.  KTAIL = true
 // handles any G and any start inside the scale rows (a reduction over a sub-range of K).  Requirements
 // checked by the host: unit-stride scale rows, operand extents below 2^31 bytes.  Every thread of the workgroup must
-// call it; it may be called again (same or other operands) to keep accumulating.  ODD_STAGES: a last 512-K block whose
-// second 256-K stage lies wholly beyond K runs its first stage only (needs KTAIL).
-template <bool KTAIL, bool ODD_STAGES = false>
+// call it; it may be called again (same or other operands) to keep accumulating.
+// How the reduction ends (KTAIL only; K is padded to whole 512-K blocks otherwise):
+//   LMS = -1  every 512-K block that holds any K runs both of its 256-K stages in full (any G, nothing known at compile time)
+//   LMS = -2  as -1, but a last block whose second stage lies wholly beyond K runs its first stage only (tested at run
+//             time; for callers whose G differs from call to call)
+//   LMS = 0/1 the caller knows G when it picks the kernel: the last stage that holds any K is stage LMS of its block and
+//             has NST (1 .. 4) K steps of 64; it runs exactly those, without the wait and the barrier of a full stage
+//             (nothing is loaded behind it), and no stage beyond it runs at all.  No run-time test: the tile needs nearly
+//             every register, and control flow around its MFMAs makes the compiler spill.
+template <bool KTAIL, int LMS = -1, int NST = 4>
 __device__ __forceinline__ void gemm_tile_mainloop(const TileArgs& ta, TileAcc& acc, uint8_t* smem) {
   TileLoader ld;
   v4i_t sraw;   // scale bytes of a later block, as loaded
@@ -392,7 +399,7 @@ __device__ __forceinline__ void gemm_tile_mainloop(const TileArgs& ta, TileAcc& 
 
   // ---- main loop: one iteration = one 512-K block = 2 macro stages
   const int NS = (ta.G + 7) / 8;         // macro stages that hold any K at all
-  const int KBF = ODD_STAGES ? NS / 2 : KB;
+  const int KBF = !KTAIL || LMS == -1 ? KB : (LMS == -2 ? NS / 2 : (NS > 0 ? (NS - 1) / 2 : 0));   // whole blocks in the loops
   int kb = 0;
   auto block = [&](int kb, auto fastc) {
     stage(std::integral_constant<int, 0>{}, 2 * kb, kb, fastc);
@@ -414,7 +421,23 @@ __device__ __forceinline__ void gemm_tile_mainloop(const TileArgs& ta, TileAcc& 
   } else {
     for (; kb < KBF; ++kb) block(kb, std::false_type{});
   }
-  if (ODD_STAGES && (NS & 1)) stage(std::integral_constant<int, 0>{}, 2 * kb, kb, std::false_type{});   // the last block's second stage lies wholly beyond K
+  if constexpr (KTAIL && LMS == -2) {
+    if (NS & 1) stage(std::integral_constant<int, 0>{}, 2 * kb, kb, std::false_type{});   // the last block's second stage lies wholly beyond K
+  }
+  if constexpr (KTAIL && LMS >= 0) {
+    static_assert(LMS <= 1 && NST >= 1 && NST <= 4, "last stage: 0 or 1, with 1 to 4 K steps");
+    if constexpr (LMS == 1) stage(std::integral_constant<int, 0>{}, 2 * kb, kb, std::true_type{});   // (passes on a scale block beyond K)
+    // The last stage: its step-0 pieces are in fa0 / fb0 and its loads have landed (the stage before has waited and met
+    // the other waves); its scale bytes are in sa / sb.
+    using LM = std::integral_constant<int, LMS>;
+    if constexpr (NST > 1) read_frags(LMS, 1, fa1, fb1);
+    mfma8(LM{}, std::integral_constant<int, 0>{}, fa0, fb0);
+    if constexpr (NST > 2) read_frags(LMS, 2, fa0, fb0);
+    if constexpr (NST > 1) mfma8(LM{}, std::integral_constant<int, 1>{}, fa1, fb1);
+    if constexpr (NST > 3) read_frags(LMS, 3, fa1, fb1);
+    if constexpr (NST > 2) mfma8(LM{}, std::integral_constant<int, 2>{}, fa0, fb0);
+    if constexpr (NST > 3) mfma8(LM{}, std::integral_constant<int, 3>{}, fa1, fb1);
+  }
   // loads of the (zero-filled) stages past the end may still be landing in the ring the epilogue reuses
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
@@ -501,14 +524,21 @@ __device__ __forceinline__ void gemm_tile_store(const TileArgs& ta, TileAcc& acc
   }
 }
 
-// ODD: the K range ends in the first 256-K stage of its last 512-K block (an odd number of stages): that block's second
-// stage is not run.  A launch-time choice because the extra exit makes the even case slower when compiled in.
-template <typename OutT, bool KTAIL, bool ODD = false>
+// LMS / NST: how the reduction ends, as in gemm_tile_mainloop.
+template <typename OutT, bool KTAIL, int LMS = -1, int NST = 4>
 __device__ __forceinline__ void gemm_tile_256x256(const TileArgs& ta, OutT* __restrict__ c, int64_t ldc, uint8_t* smem) {
   TileAcc acc;
   gemm_tile_zero(acc);
-  gemm_tile_mainloop<KTAIL, ODD>(ta, acc, smem);
+  gemm_tile_mainloop<KTAIL, LMS, NST>(ta, acc, smem);
   gemm_tile_store<OutT>(ta, acc, c, ldc, smem);
+}
+
+// The (LMS, NST) pair of a reduction over G groups of 32 whose length is known at launch (see gemm_tile_mainloop):
+// stage of the last block that holds the end of K, and its number of 64-wide K steps.  G must not be a multiple of 16.
+inline void gemm_tile_last_stage(int64_t G, int& lms, int& nst) {
+  const int64_t ns = (G + 7) / 8;
+  lms = (int)((ns - 1) & 1);
+  nst = (int)((G - 8 * (ns - 1) + 1) / 2);
 }
 
 }  // namespace alto

@@ -26,7 +26,7 @@ __device__ __forceinline__ bool tile_coords(int wg, int tiles_m, int tiles_n, in
   return true;
 }
 
-template <typename OutT, bool KTAIL, bool ODD>
+template <typename OutT, bool KTAIL, int LMS, int NST>
 __global__ __launch_bounds__(GT_THREADS) void gemm_tiled_kernel(OperandView A, OperandView B, int64_t M, int64_t N, int G,
                                                          OutT* c, int64_t ldc, float out_scale, int tiles_m, int tiles_n) {
   extern __shared__ __align__(16) uint8_t smem[];
@@ -35,14 +35,14 @@ __global__ __launch_bounds__(GT_THREADS) void gemm_tiled_kernel(OperandView A, O
   TileArgs ta{A, B, (int64_t)tm * GT_TM, (int64_t)tn * GT_TN, 0, M, N, G, out_scale,
               (M - 1) * A.ld + G * 16, (N - 1) * B.ld + G * 16,
               ((A.is_2d ? M / 32 : M) - 1) * A.ss_r + G, ((B.is_2d ? N / 32 : N) - 1) * B.ss_r + G, 0, G};
-  gemm_tile_256x256<OutT, KTAIL, ODD>(ta, c, ldc, smem);
+  gemm_tile_256x256<OutT, KTAIL, LMS, NST>(ta, c, ldc, smem);
 }
 
-template <typename OutT, bool KTAIL, bool ODD = false>
+template <typename OutT, bool KTAIL, int LMS = -1, int NST = 4>
 int launch_tiled(const OperandView& A, const OperandView& B, int64_t M, int64_t N, int64_t K, void* c, int64_t ldc, float out_scale, hipStream_t st) {
   // the opt-in for > 64 KB of dynamic LDS is per function, set once per process (two host threads may make their first
   // call together: forward on the caller's thread, backward on the autograd thread)
-  auto kern = gemm_tiled_kernel<OutT, KTAIL, ODD>;
+  auto kern = gemm_tiled_kernel<OutT, KTAIL, LMS, NST>;
   static std::once_flag once;
   static hipError_t attr_rc = hipSuccess;
   std::call_once(once, [&] { attr_rc = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, GT_LDS_BYTES); });
@@ -72,16 +72,28 @@ bool gemm_tiled_supported(const OperandView& A, const OperandView& B, int64_t M,
 void gemm_tiled_launch(const OperandView& A, const OperandView& B, int64_t M, int64_t N, int64_t K, void* c, int c_dtype, int64_t ldc,
                        float out_scale, hipStream_t st) {
   const bool tail = (K / 32) % 16 != 0;   // K not a multiple of 512: the last scale block of a row is partial
-  const bool odd = ((K / 32 + 7) / 8) % 2 != 0;   // an odd number of 256-K stages (implies tail)
-  if (c_dtype == ALTO_DT_BF16) {
-    if (odd) launch_tiled<__bf16, true, true>(A, B, M, N, K, c, ldc, out_scale, st);
-    else if (tail) launch_tiled<__bf16, true>(A, B, M, N, K, c, ldc, out_scale, st);
-    else launch_tiled<__bf16, false>(A, B, M, N, K, c, ldc, out_scale, st);
+#define ALTO_TILED_LAUNCH(T, ...) launch_tiled<T, __VA_ARGS__>(A, B, M, N, K, c, ldc, out_scale, st)
+  if (!tail) {
+    if (c_dtype == ALTO_DT_BF16) ALTO_TILED_LAUNCH(__bf16, false);
+    else ALTO_TILED_LAUNCH(float, false);
+  } else if (c_dtype != ALTO_DT_BF16) {
+    ALTO_TILED_LAUNCH(float, true);   // (fp32 output: the general ending)
   } else {
-    if (odd) launch_tiled<float, true, true>(A, B, M, N, K, c, ldc, out_scale, st);
-    else if (tail) launch_tiled<float, true>(A, B, M, N, K, c, ldc, out_scale, st);
-    else launch_tiled<float, false>(A, B, M, N, K, c, ldc, out_scale, st);
+    // K is known here: the kernel that ends the reduction exactly where K ends
+    int lms, nst;
+    gemm_tile_last_stage(K / 32, lms, nst);
+    switch (lms * 4 + nst - 1) {
+      case 0: ALTO_TILED_LAUNCH(__bf16, true, 0, 1); break;
+      case 1: ALTO_TILED_LAUNCH(__bf16, true, 0, 2); break;
+      case 2: ALTO_TILED_LAUNCH(__bf16, true, 0, 3); break;
+      case 3: ALTO_TILED_LAUNCH(__bf16, true, 0, 4); break;
+      case 4: ALTO_TILED_LAUNCH(__bf16, true, 1, 1); break;
+      case 5: ALTO_TILED_LAUNCH(__bf16, true, 1, 2); break;
+      case 6: ALTO_TILED_LAUNCH(__bf16, true, 1, 3); break;
+      default: ALTO_TILED_LAUNCH(__bf16, true, 1, 4); break;
+    }
   }
+#undef ALTO_TILED_LAUNCH
 }
 
 }  // namespace alto

@@ -289,7 +289,7 @@ __global__ __launch_bounds__(PLAN_THREADS) void grouped_plan_kernel(PassWalk wk,
   if (t == PLAN_THREADS - 1) ws[0] = scan[t] < max_pass ? scan[t] : max_pass;
 }
 
-template <typename OutT, bool KTAIL, bool ODD>
+template <typename OutT, bool KTAIL, int LMS, int NST>
 __global__ __launch_bounds__(GT_THREADS) void grouped_tiled_kernel(OperandView A, const uint8_t* w, int64_t w_stride_e, int64_t ldw,
                                                                    const uint8_t* w_scales, int64_t ws_stride_e, int64_t ws_r, int w_is_2d,
                                                                    const int32_t* plan, int64_t M_total, int64_t N, int G, OutT* out, int64_t ldo, int tiles_n) {
@@ -310,7 +310,7 @@ __global__ __launch_bounds__(GT_THREADS) void grouped_tiled_kernel(OperandView A
   TileArgs ta{A, B, row0, n0, m_lo, m_hi, N, G, 1.0f,
               (M_total - 1) * A.ld + G * 16, (N - 1) * ldw + G * 16,
               ((A.is_2d ? M_total / 32 : M_total) - 1) * A.ss_r + G, ((w_is_2d ? N / 32 : N) - 1) * ws_r + G, 0, G};
-  gemm_tile_256x256<OutT, KTAIL, ODD>(ta, out, ldo, smem);
+  gemm_tile_256x256<OutT, KTAIL, LMS, NST>(ta, out, ldo, smem);
 }
 
 // dW[e] tile: rows [256 tm, +256) of the first operand (P) x rows [256 tn, +256) of the second (Q), reduced over the
@@ -423,7 +423,7 @@ __device__ __forceinline__ void grouped_dw_tile(const OperandView& P, const Oper
     Qv.codes += ta0 / 2;
     TileArgs ta{Pv, Qv, (int64_t)tm * GT_TM, (int64_t)tn * GT_TN, 0, NP, NQ, (int)((t1 - ta0) / 32), out_scale,
                 p_bytes - ta0 / 2, q_bytes - ta0 / 2, ps_bytes, qs_bytes, (int)(ta0 / 32), (int)(M_total / 32), (int)((t0 - ta0) / 32)};
-    gemm_tile_mainloop<true, true>(ta, acc, smem);
+    gemm_tile_mainloop<true, -2>(ta, acc, smem);
   }
   if (bad) {
 #pragma unroll
@@ -450,13 +450,13 @@ __global__ __launch_bounds__(GT_THREADS) void grouped_dw_tiled_kernel(OperandVie
 inline int64_t grouped_max_passes(int64_t M_total, int64_t num_groups) { return (M_total + GT_TM - 1) / GT_TM + num_groups + 2; }
 inline int64_t grouped_workspace_bytes(int64_t M_total, int64_t num_groups) { return 16 + 16 * grouped_max_passes(M_total, num_groups); }
 
-template <typename OutT, bool KTAIL, bool ODD = false>
+template <typename OutT, bool KTAIL, int LMS = -1, int NST = 4>
 int launch_grouped_tiled(const OperandView& A, const uint8_t* w, int64_t w_stride_e, int64_t ldw, const uint8_t* w_scales, int64_t ws_stride_e,
                          int64_t ws_r, int w_is_2d, const int32_t* offs, const int32_t* group_expert, int num_groups, int num_experts,
                          int64_t M_total, int64_t N, int64_t K, void* out, int64_t ldo, int32_t* plan, hipStream_t st) {
   // the opt-in for > 64 KB of dynamic LDS is per function, set once per process (thread-safe: forward and backward may
   // make their first calls from two host threads)
-  auto kern = grouped_tiled_kernel<OutT, KTAIL, ODD>;
+  auto kern = grouped_tiled_kernel<OutT, KTAIL, LMS, NST>;
   static std::once_flag once;
   static hipError_t attr_rc = hipSuccess;
   std::call_once(once, [&] { attr_rc = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, GT_LDS_BYTES); });
@@ -537,13 +537,27 @@ int grouped_gemm_impl(const uint8_t* a, int64_t lda, const uint8_t* a_scales, in
                  (long long)plan_bytes, (long long)M_total, num_groups, (long long)need);
     const bool tail = (K / 32) % 16 != 0;
     int32_t* pl = reinterpret_cast<int32_t*>(plan);
-    const bool odd = ((K / 32 + 7) / 8) % 2 != 0;   // an odd number of 256-K stages (implies tail)
-    int rc;
+    int rc = -1;
 #define ALTO_GROUPED_LAUNCH(T, ...) launch_grouped_tiled<T, __VA_ARGS__>(A, w, w_stride_e, ldw, w_scales, ws_stride_e, ws_r, w_is_2d, offs, group_expert, num_groups, num_experts, M_total, N, K, out, ldo, pl, st)
-    if (out_dtype == ALTO_DT_BF16)
-      rc = odd ? ALTO_GROUPED_LAUNCH(__bf16, true, true) : tail ? ALTO_GROUPED_LAUNCH(__bf16, true) : ALTO_GROUPED_LAUNCH(__bf16, false);
-    else
-      rc = odd ? ALTO_GROUPED_LAUNCH(float, true, true) : tail ? ALTO_GROUPED_LAUNCH(float, true) : ALTO_GROUPED_LAUNCH(float, false);
+    if (!tail) {
+      rc = out_dtype == ALTO_DT_BF16 ? ALTO_GROUPED_LAUNCH(__bf16, false) : ALTO_GROUPED_LAUNCH(float, false);
+    } else if (out_dtype != ALTO_DT_BF16) {
+      rc = ALTO_GROUPED_LAUNCH(float, true);   // (fp32 output: the general ending)
+    } else {
+      // K is known here: the kernel that ends the reduction exactly where K ends
+      int lms, nst;
+      gemm_tile_last_stage(K / 32, lms, nst);
+      switch (lms * 4 + nst - 1) {
+        case 0: rc = ALTO_GROUPED_LAUNCH(__bf16, true, 0, 1); break;
+        case 1: rc = ALTO_GROUPED_LAUNCH(__bf16, true, 0, 2); break;
+        case 2: rc = ALTO_GROUPED_LAUNCH(__bf16, true, 0, 3); break;
+        case 3: rc = ALTO_GROUPED_LAUNCH(__bf16, true, 0, 4); break;
+        case 4: rc = ALTO_GROUPED_LAUNCH(__bf16, true, 1, 1); break;
+        case 5: rc = ALTO_GROUPED_LAUNCH(__bf16, true, 1, 2); break;
+        case 6: rc = ALTO_GROUPED_LAUNCH(__bf16, true, 1, 3); break;
+        default: rc = ALTO_GROUPED_LAUNCH(__bf16, true, 1, 4); break;
+      }
+    }
 #undef ALTO_GROUPED_LAUNCH
     if (rc != 0) {
       set_error("grouped_gemm: could not reserve %d bytes of LDS", GT_LDS_BYTES);

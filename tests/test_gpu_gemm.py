@@ -69,6 +69,23 @@ def test_gemm_ragged_shapes_and_kpack_false(m, shape):
     assert O.rel_frobenius(c.cpu(), ref) < 1e-5
 
 
+@pytest.mark.parametrize("K", [544, 640, 704, 768, 800, 864, 928, 992, 1312, 2880])
+def test_gemm_bf16_output_every_ending_of_the_reduction(m, K):
+    """bf16 output picks the tile kernel that ends the reduction where K ends: the last 256-wide stage may be the first or
+    the second of its 512-wide block and hold 1 to 4 steps of 64 -- eight endings, all of them here (K / 32 = 17 ... 90)."""
+    M, N = 256, 264
+    a = randn_outliers((M, K), torch.bfloat16, seed=13)
+    b = randn_outliers((N, K), torch.bfloat16, seed=14)
+    aq, as_ = O.quantize(a)
+    bq, bs = O.quantize(b)
+    ref = O.gemm_ref(aq, as_, bq, bs, trans_b=True)
+    c16 = m.blockwise_mxfp4_gemm(*dev(aq, as_, bq, bs), trans_b=True, output_dtype=torch.bfloat16)
+    c32 = m.blockwise_mxfp4_gemm(*dev(aq, as_, bq, bs), trans_b=True, output_dtype=torch.float32)
+    assert O.rel_frobenius(c32.cpu(), ref) < 1e-5
+    # same accumulation, one rounding apart
+    assert torch.equal(c16.cpu(), c32.bfloat16().cpu())
+
+
 def test_gemm_one_hot_exactness(m):
     """Nibble order and scale pairing, checked with values whose products are exact: C must equal the integer answer."""
     M, N, K = 64, 64, 128
@@ -329,10 +346,12 @@ def test_grouped_gemm_ragged_offsets_and_padding(m):
     assert bool((wg.grad[1] == 0).all()), "an expert without tokens gets a zero gradient"
 
 
-def test_grouped_tiled_odd_stage_counts(m):
-    """Reductions that end in the first 256-wide stage of their last 512-wide block, in all three tiled kernels: forward over
-    K = 1280 (5 stages), dX over N = 768 (3 stages), dW over token runs of 2, 2 and 3 stages (the last two start inside a line)."""
-    E, N, K = 4, 768, 1280
+@pytest.mark.parametrize("N,K", [(768, 1280), (800, 608), (928, 704), (992, 544), (864, 2880)])
+def test_grouped_tiled_odd_stage_counts(m, N, K):
+    """Reductions that do not end on a 512-wide block, in all three tiled kernels: forward over K, dX over N (the pairs
+    cover last stages in either half of a block with 1 to 4 steps of 64), dW over token runs of 2, 2 and 3 stages (the last
+    two start inside a line)."""
+    E = 4
     sizes = [320, 0, 224, 544]
     ends = torch.tensor(sizes).cumsum(0).to(torch.int32)
     M = int(ends[-1])
