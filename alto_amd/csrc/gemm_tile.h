@@ -244,8 +244,9 @@ struct TileLoader {
 //             time; for callers whose G differs from call to call)
 //   LMS = 0/1 the caller knows G when it picks the kernel: the last stage that holds any K is stage LMS of its block and
 //             has NST (1 .. 4) K steps of 64; it runs exactly those, without the wait and the barrier of a full stage
-//             (nothing is loaded behind it), and no stage beyond it runs at all.  No run-time test: the tile needs nearly
-//             every register, and control flow around its MFMAs makes the compiler spill.
+//             (nothing is loaded behind it), the stage before it loads nothing beyond K, and no stage beyond it runs at
+//             all.  No run-time test: the tile needs nearly every register, and control flow around its MFMAs makes the
+//             compiler spill.  Without a K tail the reduction always ends this way (LMS = 1, NST = 4).
 template <bool KTAIL, int LMS = -1, int NST = 4>
 __device__ __forceinline__ void gemm_tile_mainloop(const TileArgs& ta, TileAcc& acc, uint8_t* smem) {
   TileLoader ld;
@@ -347,8 +348,10 @@ __device__ __forceinline__ void gemm_tile_mainloop(const TileArgs& ta, TileAcc& 
   // loads of stage s+2 go out into it: half of them during the last step, half during the first step of the next
   // stage, one load per two MFMAs.  (A wave issues in order, and the address unit takes a 1 KB load about every 16
   // clocks per compute unit: a burst of eight loads per wave would hold the MFMAs behind it for a thousand clocks.)
-  auto stage = [&](auto msc, int s, int kb, auto fastc) {
+  // PEN (the stage before the last one, when the end of K is known at compile time): nothing beyond K is loaded.
+  auto stage = [&](auto msc, int s, int kb, auto fastc, auto penc) {
     constexpr int MS = decltype(msc)::value;
+    constexpr bool PEN = decltype(penc)::value;
     __builtin_amdgcn_s_setprio(2);
     ld.gload(smem, s + 1, MS ^ 1, 4, 8);
     mfma8(msc, std::integral_constant<int, 0>{}, fa0, fb0);
@@ -370,17 +373,18 @@ __device__ __forceinline__ void gemm_tile_mainloop(const TileArgs& ta, TileAcc& 
     __builtin_amdgcn_s_waitcnt(0);
     asm volatile("s_barrier" ::: "memory");
     __builtin_amdgcn_s_setprio(3);
-    if constexpr (MS == 0) {
+    if constexpr (MS == 0 && !PEN) {
       swrite(kb + 1, fastc);   // block kb+1 -> the other scale buffer (last read at the end of block kb-1)
       ld.template sload<KTAIL>(kb + 2, sraw);
       __builtin_amdgcn_sched_barrier(0);
     }
-    ld.gload(smem, s + 2, MS, 0, 4);
+    if constexpr (!PEN) ld.gload(smem, s + 2, MS, 0, 4);
     if constexpr (MS == 1)   // the next block's scales (in LDS since this stage's barrier) ride along with the last step
       read_scales(reinterpret_cast<const uint8_t*>(sscale + ((kb + 1) & 1) * GT_SCALE_BUF_DW), sa_next, sb_next);
     mfma8(msc, std::integral_constant<int, 3>{}, fa1, fb1);
     read_frags(MS ^ 1, 0, fa0, fb0);
-    interleave_loads();
+    if constexpr (PEN) interleave();
+    else interleave_loads();
     __builtin_amdgcn_sched_barrier(0);
   };
 
@@ -399,11 +403,17 @@ __device__ __forceinline__ void gemm_tile_mainloop(const TileArgs& ta, TileAcc& 
 
   // ---- main loop: one iteration = one 512-K block = 2 macro stages
   const int NS = (ta.G + 7) / 8;         // macro stages that hold any K at all
-  const int KBF = !KTAIL || LMS == -1 ? KB : (LMS == -2 ? NS / 2 : (NS > 0 ? (NS - 1) / 2 : 0));   // whole blocks in the loops
+  // ENDS: where K ends is known at compile time (always without a K tail: the second stage of the last block, in full)
+  constexpr bool ENDS = KTAIL ? LMS >= 0 : LMS != -3;   // (-3: a caller without a K tail that wants the plain loop over whole blocks)
+  constexpr int ELMS = KTAIL ? LMS : 1, ENST = KTAIL ? NST : 4;
+  static_assert(!ENDS || (ELMS >= 0 && ELMS <= 1 && ENST >= 1 && ENST <= 4), "last stage: 0 or 1, with 1 to 4 K steps");
+  const int KBF = ENDS ? (NS > 0 ? (NS - 1) / 2 : 0) : (KTAIL && LMS == -2 ? NS / 2 : KB);   // whole blocks in the loops
+  using F = std::false_type;
+  using T = std::true_type;
   int kb = 0;
-  auto block = [&](int kb, auto fastc) {
-    stage(std::integral_constant<int, 0>{}, 2 * kb, kb, fastc);
-    stage(std::integral_constant<int, 1>{}, 2 * kb + 1, kb, std::false_type{});
+  auto block = [&](int kb, auto fastc, auto penc) {
+    stage(std::integral_constant<int, 0>{}, 2 * kb, kb, fastc, F{});
+    stage(std::integral_constant<int, 1>{}, 2 * kb + 1, kb, F{}, penc);
 #pragma unroll
     for (int t = 0; t < 4; ++t) { sa[t][0] = sa_next[t][0]; sa[t][1] = sa_next[t][1]; }
 #pragma unroll
@@ -414,29 +424,32 @@ __device__ __forceinline__ void gemm_tile_mainloop(const TileArgs& ta, TileAcc& 
     // iteration KB - 2) can reach past its row or past K and needs its bytes fixed; earlier ones are used as loaded,
     // later ones are never read.  Three loops in a row rather than a test inside one: the tile needs nearly every
     // register, and a branch inside the loop body makes the compiler spill.
+    // With the end of K known, iteration KB - 2 is the last of the loops (KBF = KB - 1); when the last stage is the
+    // first of its block, the second stage of that iteration is the one before it.
     const int kfull = KB - 2;
-    for (; kb < kfull && kb < KBF; ++kb) block(kb, std::true_type{});
-    for (; kb < kfull + 1 && kb < KBF; ++kb) block(kb, std::false_type{});
-    for (; kb < KBF; ++kb) block(kb, std::true_type{});
+    for (; kb < kfull && kb < KBF; ++kb) block(kb, T{}, F{});
+    for (; kb < kfull + 1 && kb < KBF; ++kb) block(kb, F{}, std::bool_constant<ENDS && ELMS == 0>{});
+    if constexpr (!ENDS)
+      for (; kb < KBF; ++kb) block(kb, T{}, F{});
   } else {
-    for (; kb < KBF; ++kb) block(kb, std::false_type{});
+    for (; kb < KBF; ++kb) block(kb, F{}, F{});
   }
   if constexpr (KTAIL && LMS == -2) {
-    if (NS & 1) stage(std::integral_constant<int, 0>{}, 2 * kb, kb, std::false_type{});   // the last block's second stage lies wholly beyond K
+    if (NS & 1) stage(std::integral_constant<int, 0>{}, 2 * kb, kb, F{}, F{});   // the last block's second stage lies wholly beyond K
   }
-  if constexpr (KTAIL && LMS >= 0) {
-    static_assert(LMS <= 1 && NST >= 1 && NST <= 4, "last stage: 0 or 1, with 1 to 4 K steps");
-    if constexpr (LMS == 1) stage(std::integral_constant<int, 0>{}, 2 * kb, kb, std::true_type{});   // (passes on a scale block beyond K)
-    // The last stage: its step-0 pieces are in fa0 / fb0 and its loads have landed (the stage before has waited and met
-    // the other waves); its scale bytes are in sa / sb.
-    using LM = std::integral_constant<int, LMS>;
-    if constexpr (NST > 1) read_frags(LMS, 1, fa1, fb1);
+  if constexpr (ENDS) {
+    if constexpr (ELMS == 1) stage(std::integral_constant<int, 0>{}, 2 * kb, kb, T{}, T{});   // the stage before the last
+    // The last stage, only the steps it has: its step-0 pieces are in fa0 / fb0 and its loads have landed (the stage before
+    // has waited and met the other waves), its scale bytes are in sa / sb; nothing is loaded behind it, so it neither
+    // waits nor meets anybody.
+    using LM = std::integral_constant<int, ELMS>;
+    if constexpr (ENST > 1) read_frags(ELMS, 1, fa1, fb1);
     mfma8(LM{}, std::integral_constant<int, 0>{}, fa0, fb0);
-    if constexpr (NST > 2) read_frags(LMS, 2, fa0, fb0);
-    if constexpr (NST > 1) mfma8(LM{}, std::integral_constant<int, 1>{}, fa1, fb1);
-    if constexpr (NST > 3) read_frags(LMS, 3, fa1, fb1);
-    if constexpr (NST > 2) mfma8(LM{}, std::integral_constant<int, 2>{}, fa0, fb0);
-    if constexpr (NST > 3) mfma8(LM{}, std::integral_constant<int, 3>{}, fa1, fb1);
+    if constexpr (ENST > 2) read_frags(ELMS, 2, fa0, fb0);
+    if constexpr (ENST > 1) mfma8(LM{}, std::integral_constant<int, 1>{}, fa1, fb1);
+    if constexpr (ENST > 3) read_frags(ELMS, 3, fa1, fb1);
+    if constexpr (ENST > 2) mfma8(LM{}, std::integral_constant<int, 2>{}, fa0, fb0);
+    if constexpr (ENST > 3) mfma8(LM{}, std::integral_constant<int, 3>{}, fa1, fb1);
   }
   // loads of the (zero-filled) stages past the end may still be landing in the ring the epilogue reuses
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -529,7 +542,8 @@ template <typename OutT, bool KTAIL, int LMS = -1, int NST = 4>
 __device__ __forceinline__ void gemm_tile_256x256(const TileArgs& ta, OutT* __restrict__ c, int64_t ldc, uint8_t* smem) {
   TileAcc acc;
   gemm_tile_zero(acc);
-  gemm_tile_mainloop<KTAIL, LMS, NST>(ta, acc, smem);
+  // (with fp32 output and no K tail the specialised ending pushes the register allocation into spilling: plain loop there)
+  gemm_tile_mainloop<KTAIL, (!KTAIL && sizeof(OutT) == 4) ? -3 : LMS, NST>(ta, acc, smem);
   gemm_tile_store<OutT>(ta, acc, c, ldc, smem);
 }
 
