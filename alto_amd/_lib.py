@@ -51,6 +51,10 @@ SIGNATURES = {
     "alto_mxfp4_grouped_gemm": (c_int, [c_vp, c_i64, c_vp, c_i64, c_i64, c_int,
                                         c_vp, c_i64, c_i64, c_vp, c_i64, c_i64, c_i64, c_int,
                                         c_vp, c_vp, c_int, c_int, c_i64, c_i64, c_i64, c_vp, c_int, c_i64, c_vp, c_i64, c_vp]),
+    "alto_mxfp4_grouped_gemm_planned": (c_int, [c_vp, c_i64, c_vp, c_i64, c_i64, c_int,
+                                        c_vp, c_i64, c_i64, c_vp, c_i64, c_i64, c_i64, c_int,
+                                        c_vp, c_vp, c_int, c_int, c_i64, c_i64, c_i64, c_vp, c_int, c_i64, c_vp, c_i64, c_vp]),
+    "alto_mxfp4_grouped_gemm_plan": (c_int, [c_vp, c_vp, c_int, c_int, c_i64, c_vp, c_i64, c_vp]),
     "alto_mxfp4_grouped_gemm_noalloc": (c_int, [c_vp, c_i64, c_vp, c_i64, c_i64, c_int,
                                                 c_vp, c_i64, c_i64, c_vp, c_i64, c_i64, c_i64, c_int,
                                                 c_vp, c_vp, c_int, c_int, c_i64, c_i64, c_i64, c_vp, c_int, c_i64, c_vp]),

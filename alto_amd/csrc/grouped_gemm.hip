@@ -453,7 +453,7 @@ inline int64_t grouped_workspace_bytes(int64_t M_total, int64_t num_groups) { re
 template <typename OutT, bool KTAIL, int LMS = -1, int NST = 4>
 int launch_grouped_tiled(const OperandView& A, const uint8_t* w, int64_t w_stride_e, int64_t ldw, const uint8_t* w_scales, int64_t ws_stride_e,
                          int64_t ws_r, int w_is_2d, const int32_t* offs, const int32_t* group_expert, int num_groups, int num_experts,
-                         int64_t M_total, int64_t N, int64_t K, void* out, int64_t ldo, int32_t* plan, hipStream_t st) {
+                         int64_t M_total, int64_t N, int64_t K, void* out, int64_t ldo, int32_t* plan, bool build_plan, hipStream_t st) {
   // the opt-in for > 64 KB of dynamic LDS is per function, set once per process (thread-safe: forward and backward may
   // make their first calls from two host threads)
   auto kern = grouped_tiled_kernel<OutT, KTAIL, LMS, NST>;
@@ -464,7 +464,7 @@ int launch_grouped_tiled(const OperandView& A, const uint8_t* w, int64_t w_strid
   const int tiles_m = (int)((M_total + GT_TM - 1) / GT_TM), tiles_n = (int)((N + GT_TN - 1) / GT_TN);
   const int max_pass = (int)grouped_max_passes(M_total, num_groups);
   PassWalk wk{offs, group_expert, num_groups, num_experts, M_total};
-  hipLaunchKernelGGL(grouped_plan_kernel, dim3(1), dim3(PLAN_THREADS), 0, st, wk, tiles_m, plan, max_pass);
+  if (build_plan) hipLaunchKernelGGL(grouped_plan_kernel, dim3(1), dim3(PLAN_THREADS), 0, st, wk, tiles_m, plan, max_pass);
   hipLaunchKernelGGL(kern, dim3((unsigned)grouped_grid_size(max_pass, tiles_n)), dim3(GT_THREADS), GT_LDS_BYTES, st, A, w, w_stride_e, ldw, w_scales, ws_stride_e, ws_r,
                      w_is_2d, plan, M_total, N, (int)(K / 32), (OutT*)out, ldo, tiles_n);
   return 0;
@@ -508,7 +508,7 @@ int grouped_gemm_impl(const uint8_t* a, int64_t lda, const uint8_t* a_scales, in
                       const uint8_t* w_scales, int64_t ws_stride_e, int64_t ws_r, int64_t ws_k, int w_is_2d,
                       const int32_t* offs, const int32_t* group_expert, int num_groups, int num_experts,
                       int64_t M_total, int64_t N, int64_t K, void* out, int out_dtype, int64_t ldo,
-                      void* plan, int64_t plan_bytes, const char* plan_name, void* stream) {
+                      void* plan, int64_t plan_bytes, const char* plan_name, bool build_plan, void* stream) {
   ALTO_REQUIRE(a && a_scales && w && w_scales && offs && out, "grouped_gemm: NULL pointer");
   ALTO_REQUIRE(num_groups > 0 && num_groups <= 65536, "grouped_gemm: num_groups (%d) out of range", num_groups);
   ALTO_REQUIRE(group_expert != nullptr || num_groups == num_experts, "grouped_gemm: without group_expert, num_groups must equal num_experts");
@@ -538,7 +538,7 @@ int grouped_gemm_impl(const uint8_t* a, int64_t lda, const uint8_t* a_scales, in
     const bool tail = (K / 32) % 16 != 0;
     int32_t* pl = reinterpret_cast<int32_t*>(plan);
     int rc = -1;
-#define ALTO_GROUPED_LAUNCH(T, ...) launch_grouped_tiled<T, __VA_ARGS__>(A, w, w_stride_e, ldw, w_scales, ws_stride_e, ws_r, w_is_2d, offs, group_expert, num_groups, num_experts, M_total, N, K, out, ldo, pl, st)
+#define ALTO_GROUPED_LAUNCH(T, ...) launch_grouped_tiled<T, __VA_ARGS__>(A, w, w_stride_e, ldw, w_scales, ws_stride_e, ws_r, w_is_2d, offs, group_expert, num_groups, num_experts, M_total, N, K, out, ldo, pl, build_plan, st)
     if (!tail) {
       rc = out_dtype == ALTO_DT_BF16 ? ALTO_GROUPED_LAUNCH(__bf16, false) : ALTO_GROUPED_LAUNCH(float, false);
     } else if (out_dtype != ALTO_DT_BF16) {
@@ -593,7 +593,37 @@ extern "C" int alto_mxfp4_grouped_gemm(const uint8_t* a, int64_t lda, const uint
                                        int64_t M_total, int64_t N, int64_t K, void* out, int out_dtype, int64_t ldo,
                                        void* workspace, int64_t workspace_bytes, void* stream) {
   return alto::grouped_gemm_impl(a, lda, a_scales, a_ss_r, a_ss_k, a_is_2d, w, w_stride_e, ldw, w_scales, ws_stride_e, ws_r, ws_k, w_is_2d, offs, group_expert,
-                                 num_groups, num_experts, M_total, N, K, out, out_dtype, ldo, workspace, workspace_bytes, "the workspace", stream);
+                                 num_groups, num_experts, M_total, N, K, out, out_dtype, ldo, workspace, workspace_bytes, "the workspace", true, stream);
+}
+
+extern "C" int alto_mxfp4_grouped_gemm_planned(const uint8_t* a, int64_t lda, const uint8_t* a_scales, int64_t a_ss_r, int64_t a_ss_k, int a_is_2d,
+                                               const uint8_t* w, int64_t w_stride_e, int64_t ldw,
+                                               const uint8_t* w_scales, int64_t ws_stride_e, int64_t ws_r, int64_t ws_k, int w_is_2d,
+                                               const int32_t* offs, const int32_t* group_expert, int num_groups, int num_experts,
+                                               int64_t M_total, int64_t N, int64_t K, void* out, int out_dtype, int64_t ldo,
+                                               const void* workspace, int64_t workspace_bytes, void* stream) {
+  return alto::grouped_gemm_impl(a, lda, a_scales, a_ss_r, a_ss_k, a_is_2d, w, w_stride_e, ldw, w_scales, ws_stride_e, ws_r, ws_k, w_is_2d, offs, group_expert,
+                                 num_groups, num_experts, M_total, N, K, out, out_dtype, ldo, const_cast<void*>(workspace), workspace_bytes, "the workspace",
+                                 false, stream);
+}
+
+extern "C" int alto_mxfp4_grouped_gemm_plan(const int32_t* offs, const int32_t* group_expert, int num_groups, int num_experts, int64_t M_total,
+                                            void* workspace, int64_t workspace_bytes, void* stream) {
+  using namespace alto;
+  ALTO_REQUIRE(offs != nullptr, "grouped_gemm_plan: NULL offs");
+  ALTO_REQUIRE(num_groups > 0 && num_groups <= 65536, "grouped_gemm_plan: num_groups (%d) out of range", num_groups);
+  ALTO_REQUIRE(group_expert != nullptr || num_groups == num_experts, "grouped_gemm_plan: without group_expert, num_groups must equal num_experts");
+  ALTO_REQUIRE(num_experts > 0 && num_experts <= 4096, "grouped_gemm_plan: num_experts (%d) out of range", num_experts);
+  ALTO_REQUIRE(M_total >= 0 && M_total < (1ll << 31), "grouped_gemm_plan: M_total out of range");
+  const int64_t need = grouped_workspace_bytes(M_total, num_groups);
+  ALTO_REQUIRE(workspace != nullptr && workspace_bytes >= need && (reinterpret_cast<uintptr_t>(workspace) & 15) == 0,
+               "grouped_gemm_plan: workspace of %lld bytes is too small: M_total = %lld with %d groups needs %lld bytes (16-byte aligned)",
+               (long long)workspace_bytes, (long long)M_total, num_groups, (long long)need);
+  if (M_total == 0) return ALTO_MXFP4_OK;
+  PassWalk wk{offs, group_expert, num_groups, num_experts, M_total};
+  hipLaunchKernelGGL(grouped_plan_kernel, dim3(1), dim3(PLAN_THREADS), 0, reinterpret_cast<hipStream_t>(stream), wk, (int)((M_total + GT_TM - 1) / GT_TM),
+                     reinterpret_cast<int32_t*>(workspace), (int)grouped_max_passes(M_total, num_groups));
+  return check_launch("grouped_gemm_plan");
 }
 
 namespace alto {
@@ -646,7 +676,7 @@ extern "C" int alto_mxfp4_grouped_gemm_noalloc(const uint8_t* a, int64_t lda, co
   const int rc = scratch_of_current_device(&plan);
   if (rc != ALTO_MXFP4_OK) return rc;
   return grouped_gemm_impl(a, lda, a_scales, a_ss_r, a_ss_k, a_is_2d, w, w_stride_e, ldw, w_scales, ws_stride_e, ws_r, ws_k, w_is_2d, offs, group_expert,
-                           num_groups, num_experts, M_total, N, K, out, out_dtype, ldo, plan, ALTO_NOALLOC_SCRATCH_BYTES, "the built-in scratch array", stream);
+                           num_groups, num_experts, M_total, N, K, out, out_dtype, ldo, plan, ALTO_NOALLOC_SCRATCH_BYTES, "the built-in scratch array", true, stream);
 }
 
 extern "C" int alto_mxfp4_grouped_gemm_dw(const uint8_t* go, int64_t ld_go, const uint8_t* go_scales, int64_t gs_r, int64_t gs_k, int go_is_2d,

@@ -63,8 +63,11 @@ def _scale_strides(s: torch.Tensor):
     return s.stride(0), s.stride(1), s.stride(2)
 
 
-def grouped_forward(a_q, a_s, w_q, w_s, groups: Groups, use_2dblock_x, use_2dblock_w, output_dtype):
-    """out[r] = A[r] . W[e(r)]^T with w_q [E, N, K/2] (unit stride along K) and w_s [E, N or N/32, K/32]."""
+def grouped_forward(a_q, a_s, w_q, w_s, groups: Groups, use_2dblock_x, use_2dblock_w, output_dtype, plan=None, return_plan=False):
+    """out[r] = A[r] . W[e(r)]^T with w_q [E, N, K/2] (unit stride along K) and w_s [E, N or N/32, K/32].
+
+    ``plan``: the pass list an earlier call over the same ``groups`` and row count wrote (``return_plan=True`` hands it
+    out): the one-workgroup kernel that builds it is then not launched again (the input gradient reuses the forward's)."""
     E, N = w_q.shape[0], w_q.shape[1]
     K = a_q.shape[1] * 2
     assert w_q.shape[2] * 2 == K, f"Input K ({K}) must match weight K ({w_q.shape[2] * 2})"
@@ -74,17 +77,33 @@ def grouped_forward(a_q, a_s, w_q, w_s, groups: Groups, use_2dblock_x, use_2dblo
         w_q = w_q.contiguous()
     out = torch.empty((a_q.shape[0], N), dtype=output_dtype, device=a_q.device)
     if out.numel() == 0:
-        return out
+        return (out, plan) if return_plan else out
     # the pass list the kernels exchange (a few KB; torch's caching allocator hands it out without a device call)
     ws_bytes = rt.lib().alto_mxfp4_grouped_gemm_workspace_bytes(a_q.shape[0], groups.n)
-    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=a_q.device)
-    rc = rt.lib().alto_mxfp4_grouped_gemm(
+    if plan is not None:
+        assert plan.dtype == torch.uint8 and plan.numel() >= ws_bytes and plan.device == a_q.device
+        ws, fn, name = plan, rt.lib().alto_mxfp4_grouped_gemm_planned, "alto_mxfp4_grouped_gemm_planned"
+    else:
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=a_q.device)
+        fn, name = rt.lib().alto_mxfp4_grouped_gemm, "alto_mxfp4_grouped_gemm"
+    rc = fn(
         a_q.data_ptr(), a_q.stride(0), a_s.data_ptr(), a_s.stride(0), a_s.stride(1), int(use_2dblock_x),
         w_q.data_ptr(), w_q.stride(0), w_q.stride(1), w_s.data_ptr(), w_s.stride(0), w_s.stride(1), w_s.stride(2), int(use_2dblock_w),
         groups.offs.data_ptr(), rt.ptr(groups.expert), groups.n, E, a_q.shape[0], N, K, out.data_ptr(), rt.dtype_code(output_dtype), out.stride(0),
-        ws.data_ptr(), ws_bytes, rt.stream_ptr(a_q.device))
-    check(rc, "alto_mxfp4_grouped_gemm")
-    return out
+        ws.data_ptr(), ws.numel(), rt.stream_ptr(a_q.device))
+    check(rc, name)
+    return (out, ws) if return_plan else out
+
+
+def grouped_plan(groups: Groups, num_experts: int, m_total: int) -> torch.Tensor:
+    """The pass list of ``groups`` over ``m_total`` rows, for ``grouped_forward(..., plan=...)``."""
+    dev = groups.offs.device
+    ws_bytes = rt.lib().alto_mxfp4_grouped_gemm_workspace_bytes(m_total, groups.n)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    rc = rt.lib().alto_mxfp4_grouped_gemm_plan(groups.offs.data_ptr(), rt.ptr(groups.expert), groups.n, num_experts, m_total, ws.data_ptr(), ws_bytes,
+                                               rt.stream_ptr(dev))
+    check(rc, "alto_mxfp4_grouped_gemm_plan")
+    return ws
 
 
 def mxfp4_grouped_gemm_forward(inputs, expert_weights, expert_indices, input_scales, weight_scales, trans_weights=True,
@@ -206,8 +225,8 @@ class MXFP4GroupedGEMM(torch.autograd.Function):
             wq_nk, ws_nk, wq_kn, ws_kn = _quantize_experts(weights_owner, w, use_2dblock_w, use_uos)
         else:                                                                     # stored [E, K, N]: same pass, roles swapped
             wq_kn, ws_kn, wq_nk, ws_nk = _quantize_experts(weights_owner, w.transpose(1, 2), use_2dblock_w, use_uos)
-        out = grouped_forward(a_q, a_s, wq_nk, ws_nk, groups, use_2dblock_x, use_2dblock_w, original_dtype)
-        ctx.save_for_backward(a_qm, a_sm, wq_kn, ws_kn, groups.offs, groups.expert)
+        out, plan = grouped_forward(a_q, a_s, wq_nk, ws_nk, groups, use_2dblock_x, use_2dblock_w, original_dtype, return_plan=True)
+        ctx.save_for_backward(a_qm, a_sm, wq_kn, ws_kn, groups.offs, groups.expert, plan)   # (plan: the pass list, reused by dX)
         ctx.num_groups = groups.n
         ctx.trans_weights = trans_weights
         ctx.original_dtype = original_dtype
@@ -223,7 +242,7 @@ class MXFP4GroupedGEMM(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, grad_output):
-        a_qm, a_sm, wq_kn, ws_kn, g_offs, g_expert = ctx.saved_tensors
+        a_qm, a_sm, wq_kn, ws_kn, g_offs, g_expert, plan = ctx.saved_tensors
         groups = Groups(g_offs, g_expert, ctx.num_groups)
         go = grad_output if grad_output.is_contiguous() else grad_output.contiguous()
         sr = bool(ctx.use_sr_grad)
@@ -234,7 +253,7 @@ class MXFP4GroupedGEMM(torch.autograd.Function):
         else:
             go_q, go_s, go_qm, go_sm = quantize_rowcol(go, False, use_sr=sr, rand_bits=rand, hadamard=ctx.hadamard_transform,
                                                        clip_mode=ctx.clip_mode, use_uos=ctx.use_uos, pad_codes=True)
-        grad_inputs = grouped_forward(go_q, go_s, wq_kn, ws_kn, groups, ctx.use_2dblock_x, ctx.use_2dblock_w, ctx.original_dtype)
+        grad_inputs = grouped_forward(go_q, go_s, wq_kn, ws_kn, groups, ctx.use_2dblock_x, ctx.use_2dblock_w, ctx.original_dtype, plan=plan)
         grad_weights = grouped_dw(go_qm.transpose(0, 1), go_sm.transpose(0, 1), a_qm.transpose(0, 1), a_sm.transpose(0, 1),
                                   groups, ctx.num_experts, ctx.original_dtype, ctx.trans_weights,
                                   _wgrad_scale(ctx.clip_mode, ctx.use_dge), is_2d=ctx.use_2dblock_x)

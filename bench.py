@@ -340,6 +340,12 @@ class GroupedGemmDx(GroupedGemm):
         w = (torch.randn(self.E, self.N, self.K, device=dev, generator=gen) * 0.02).bfloat16()
         _, _, self.wq, self.ws = _quantize_call(_prep(w), True, True, True, False, None, None, 0, False, True)   # [E, K, N/2], [E, K/32, N/32]
         del w
+        # as in the autograd function, the input gradient reuses the pass list that the forward of the same groups wrote
+        self.plan = self.G.grouped_plan(self.groups, self.E, self.rows)
+
+    def step(self):
+        import torch
+        return self.G.grouped_forward(self.aq, self.as_, self.wq, self.ws, self.groups, False, True, torch.bfloat16, plan=self.plan)
 
     def cpu_sample(self):
         raise NotImplementedError("reported beside the forward workload, which carries the CPU leg")

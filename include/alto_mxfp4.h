@@ -242,6 +242,24 @@ int alto_mxfp4_grouped_gemm(const uint8_t* a, int64_t lda, const uint8_t* a_scal
                             void* workspace, int64_t workspace_bytes, void* stream);
 
 /*
+ * The two halves of alto_mxfp4_grouped_gemm for callers that run several grouped GEMMs over the same groups (the forward
+ * and the input gradient of one layer share them): alto_mxfp4_grouped_gemm_plan writes the pass list for (offs,
+ * group_expert, num_groups, num_experts, M_total) into `workspace` (the one-workgroup kernel only), and
+ * alto_mxfp4_grouped_gemm_planned is alto_mxfp4_grouped_gemm without that kernel: it trusts `workspace` to hold the list
+ * that a call of _plan -- or of alto_mxfp4_grouped_gemm itself -- wrote for exactly these five arguments, and only reads
+ * it (N, K and the operands may differ from call to call).  Same results as alto_mxfp4_grouped_gemm, bit for bit.  No
+ * counterpart in the reference, whose kernels scan the groups inside every program (cg_forward.py:120-140).
+ */
+int alto_mxfp4_grouped_gemm_plan(const int32_t* offs, const int32_t* group_expert, int num_groups, int num_experts, int64_t M_total,
+                                 void* workspace, int64_t workspace_bytes, void* stream);
+int alto_mxfp4_grouped_gemm_planned(const uint8_t* a, int64_t lda, const uint8_t* a_scales, int64_t a_ss_r, int64_t a_ss_k, int a_is_2d,
+                                    const uint8_t* w, int64_t w_stride_e, int64_t ldw,
+                                    const uint8_t* w_scales, int64_t ws_stride_e, int64_t ws_r, int64_t ws_k, int w_is_2d,
+                                    const int32_t* offs, const int32_t* group_expert, int num_groups, int num_experts,
+                                    int64_t M_total, int64_t N, int64_t K, void* out, int out_dtype, int64_t ldo,
+                                    const void* workspace, int64_t workspace_bytes, void* stream);
+
+/*
  * Per-device set-up that the entry points otherwise do on first use: resolves, for the CURRENT device, the address of the
  * library's built-in pass-list array.  Call it once per device (with that device current) before capturing a HIP graph
  * that contains alto_mxfp4_grouped_gemm_noalloc.  Idempotent, thread-safe, allocates nothing.  No counterpart in the

@@ -375,6 +375,35 @@ def test_grouped_tiled_odd_stage_counts(m, N, K):
     assert bool((wg.grad[1] == 0).all())
 
 
+@pytest.mark.parametrize("sorted_form", [True, False])
+def test_grouped_pass_list_built_once_and_reused(m, sorted_form):
+    """alto_mxfp4_grouped_gemm_plan + _planned against the one-call entry, bit for bit, for two different (N, K) over the
+    same groups -- the way the input gradient reuses the forward's list."""
+    from alto_amd.mxfp4 import grouped_gemm as G
+    E, M = 5, 1536
+    if sorted_form:
+        ends = torch.tensor([200, 200, 777, 1300, 1500]).to(torch.int32)
+        groups = G.groups_from_offsets(G.offsets_from_ends(ends.to(DEV)))
+    else:
+        idx = torch.randint(0, E, (M // 128,), generator=torch.Generator().manual_seed(3), dtype=torch.int32).repeat_interleave(128)
+        groups = G.groups_from_indices(idx.to(DEV))
+    plan = G.grouped_plan(groups, E, M)
+    keep = plan.clone()
+    for N, K in ((512, 768), (768, 512)):
+        a, w = _grouped_inputs(M, N, K, E, seed=90 + N)
+        aq, as_ = m.convert_to_mxfp4(a.to(DEV))
+        wq, ws = m.convert_to_mxfp4(w.to(DEV), is_2d_block=True)
+        one = G.grouped_forward(aq, as_, wq, ws, groups, False, True, torch.bfloat16)
+        two = G.grouped_forward(aq, as_, wq, ws, groups, False, True, torch.bfloat16, plan=plan)
+        assert torch.equal(one, two)
+        out3, plan3 = G.grouped_forward(aq, as_, wq, ws, groups, False, True, torch.bfloat16, return_plan=True)
+        assert torch.equal(out3, one)
+        n_pass = int(plan3[:4].view(torch.int32)[0])
+        assert torch.equal(plan3[:4], plan[:4]) and torch.equal(plan3[16:16 + 16 * n_pass], plan[16:16 + 16 * n_pass]), \
+            "the one-call entry writes the same list (the 12 bytes behind the count are padding)"
+    assert torch.equal(plan, keep), "the planned call only reads the list"
+
+
 def test_grouped_unaligned_rows_forward(m):
     """Forward with group boundaries at arbitrary rows (1D activation scales need no alignment)."""
     E, N, K = 4, 128, 256
