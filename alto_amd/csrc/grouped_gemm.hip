@@ -224,8 +224,26 @@ constexpr int PLAN_THREADS = 256;
 //    [t nb, (t + 1) nb) and emits, per band, one pass per run of groups of the same expert.
 // Either way a thread counts its passes, an exclusive scan of the counts gives its offset, and it writes them there,
 // so the list is in row order.
+// Inclusive scan over the workgroup's PLAN_THREADS values (thread order): inside a wave with lane shuffles, across the four
+// waves through four words of LDS -- two barriers instead of the two per doubling step of a scan through LDS.
+template <typename Op>
+__device__ __forceinline__ int plan_scan(int v, Op op, int* part) {
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    const int u = __shfl_up(v, d, 64);
+    if (lane >= d) v = op(v, u);
+  }
+  if (lane == 63) part[w] = v;
+  __syncthreads();
+  for (int k = 0; k < w; ++k) v = op(v, part[k]);
+  __syncthreads();   // `part` may be written again
+  return v;
+}
+
 __global__ __launch_bounds__(PLAN_THREADS) void grouped_plan_kernel(PassWalk wk, int tiles_m, int32_t* ws, int max_pass) {
-  __shared__ int scan[PLAN_THREADS];
+  __shared__ int part[PLAN_THREADS / 64];
+  __shared__ int carry[PLAN_THREADS];
   const int t = threadIdx.x;
   const bool sorted = wk.group_expert == nullptr;
   const int items = sorted ? wk.num_groups + 2 : tiles_m;
@@ -235,21 +253,16 @@ __global__ __launch_bounds__(PLAN_THREADS) void grouped_plan_kernel(PassWalk wk,
   // Sorted form: item i ends at E(i) = offs[i] (head: offs[0]; tail: M_total) and starts at the running maximum of the
   // ends before it, so the items tile [0, M_total) without overlap whatever the offsets are: a group whose end lies
   // below an earlier end is empty, one that starts below it is cut (the fallback kernel's row search does the same).
-  auto item_end = [&](int i) { return i == wk.num_groups + 1 ? Mt : wk.off_at(i); };
+  auto item_end_load = [&](int i) { return i == wk.num_groups + 1 ? Mt : wk.off_at(i); };
+  const int first_end = (sorted && i0 < i1) ? item_end_load(i0) : 0;   // (the usual case is one item per thread: one load in all)
+  auto item_end = [&](int i) { return i == i0 ? first_end : item_end_load(i); };
   int start = 0;   // running maximum of the ends before item i0
   if (sorted) {
     int lm = 0;
     for (int i = i0; i < i1; ++i) { const int v = item_end(i); lm = v > lm ? v : lm; }
-    scan[t] = lm;
+    carry[t] = plan_scan(lm, [](int a, int b) { return a > b ? a : b; }, part);   // inclusive max scan
     __syncthreads();
-    for (int d = 1; d < PLAN_THREADS; d <<= 1) {   // inclusive max scan
-      const int v = t >= d ? scan[t - d] : 0;
-      __syncthreads();
-      scan[t] = v > scan[t] ? v : scan[t];
-      __syncthreads();
-    }
-    start = t > 0 ? scan[t - 1] : 0;
-    __syncthreads();
+    start = t > 0 ? carry[t - 1] : 0;
   }
   auto item = [&](int i, int& run, int& lo, int& hi, int& e) {   // `run` carries the running maximum along the thread's items
     e = (i >= 1 && i <= wk.num_groups && (i - 1) < wk.num_experts) ? i - 1 : -1;
@@ -272,21 +285,14 @@ __global__ __launch_bounds__(PLAN_THREADS) void grouped_plan_kernel(PassWalk wk,
   };
   int cnt = 0;
   walk([&](int, int, int, int) { ++cnt; });
-  scan[t] = cnt;
-  __syncthreads();
-  for (int d = 1; d < PLAN_THREADS; d <<= 1) {   // inclusive scan
-    const int v = t >= d ? scan[t - d] : 0;
-    __syncthreads();
-    scan[t] += v;
-    __syncthreads();
-  }
-  int at = scan[t] - cnt;
+  const int upto = plan_scan(cnt, [](int a, int b) { return a + b; }, part);   // passes of threads 0 .. t
+  int at = upto - cnt;
   int4* list = reinterpret_cast<int4*>(ws + 4);
   walk([&](int row0, int lo, int hi, int e) {
     if (at < max_pass) list[at] = make_int4(row0, lo, hi, e);
     ++at;
   });
-  if (t == PLAN_THREADS - 1) ws[0] = scan[t] < max_pass ? scan[t] : max_pass;
+  if (t == PLAN_THREADS - 1) ws[0] = upto < max_pass ? upto : max_pass;
 }
 
 template <typename OutT, bool KTAIL, int LMS, int NST>
