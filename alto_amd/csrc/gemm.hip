@@ -51,3 +51,43 @@ extern "C" int alto_mxfp4_gemm(const uint8_t* a, int64_t lda, const uint8_t* a_s
     hipLaunchKernelGGL(gemm_simple_kernel<float>, grid, dim3(256), 0, st, A, B, M, N, (int)(K / 32), (float*)c, ldc, out_scale);
   return check_launch("gemm");
 }
+
+extern "C" int64_t alto_mxfp4_packed_scales_bytes(int64_t rows, int64_t K) {
+  if (rows < 0 || K < 0 || K % 32 != 0) return 0;
+  return ((K / 32 + 15) / 16) * rows * 16;
+}
+
+extern "C" int alto_mxfp4_pack_scales(const uint8_t* scales, int64_t ss_r, int64_t ss_k, int is_2d, int64_t rows, int64_t K, uint8_t* packed, void* stream) {
+  using namespace alto;
+  ALTO_REQUIRE(scales && packed, "pack_scales: NULL pointer");
+  ALTO_REQUIRE(rows >= 0 && K >= 0 && K % 32 == 0, "pack_scales: K (%lld) must be a multiple of 32", (long long)K);
+  ALTO_REQUIRE(!is_2d || rows % 32 == 0, "pack_scales: 2D scales need rows (%lld) %% 32 == 0", (long long)rows);
+  ALTO_REQUIRE((reinterpret_cast<uintptr_t>(packed) & 15) == 0, "pack_scales: packed must be 16-byte aligned");
+  ALTO_REQUIRE((K / 32 + 15) / 16 <= 65535, "pack_scales: K too large");
+  if (rows == 0 || K == 0) return ALTO_MXFP4_OK;
+  pack_scales_launch(scales, ss_r, ss_k, is_2d, rows, K / 32, packed, reinterpret_cast<hipStream_t>(stream));
+  return check_launch("pack_scales");
+}
+
+extern "C" int alto_mxfp4_gemm_ps(const uint8_t* a, int64_t lda, const uint8_t* a_packed, const uint8_t* b, int64_t ldb, const uint8_t* b_packed,
+                                  int64_t M, int64_t N, int64_t K, void* c, int64_t ldc, float out_scale, void* stream) {
+  using namespace alto;
+  ALTO_REQUIRE(a && b && a_packed && b_packed && c, "gemm_ps: NULL pointer");
+  ALTO_REQUIRE(M >= 0 && N >= 0 && K >= 0 && K % 32 == 0, "gemm_ps: K (%lld) must be a multiple of 32", (long long)K);
+  ALTO_REQUIRE(lda >= K / 2 && ldb >= K / 2 && lda % 16 == 0 && ldb % 16 == 0, "gemm_ps: lda/ldb must be >= K/2 and multiples of 16 bytes");
+  ALTO_REQUIRE(((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b) | reinterpret_cast<uintptr_t>(a_packed) | reinterpret_cast<uintptr_t>(b_packed)) & 15) == 0,
+               "gemm_ps: a, b and their packed scales must be 16-byte aligned");
+  ALTO_REQUIRE(ldc >= N, "gemm_ps: ldc < N");
+  if (M == 0 || N == 0) return ALTO_MXFP4_OK;
+  const int64_t KB = (K / 32 + 15) / 16;
+  OperandView A{a, lda, a_packed, 16, M * 16, 0};
+  OperandView B{b, ldb, b_packed, 16, N * 16, 0};
+  // the packed form exists for the 256x256 tile kernel only: same shape conditions as alto_mxfp4_gemm's choice of it
+  OperandView Ap{a, lda, a_packed, 1, 1, 0}, Bp{b, ldb, b_packed, 1, 1, 0};
+  if (!(gemm_tiled_supported(Ap, Bp, M, N, K, c, ALTO_DT_BF16, ldc) && KB * M * 16 < (1ll << 31) && KB * N * 16 < (1ll << 31))) {
+    set_error("gemm_ps: shape (%lld, %lld, %lld) is not served by the tile kernel; use alto_mxfp4_gemm with plain scales", (long long)M, (long long)N, (long long)K);
+    return ALTO_MXFP4_ENOTIMPL;
+  }
+  gemm_tiled_launch_ps(A, B, M, N, K, c, ldc, out_scale, reinterpret_cast<hipStream_t>(stream));
+  return check_launch("gemm_ps");
+}

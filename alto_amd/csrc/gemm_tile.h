@@ -247,8 +247,15 @@ struct TileLoader {
 //             (nothing is loaded behind it), the stage before it loads nothing beyond K, and no stage beyond it runs at
 //             all.  No run-time test: the tile needs nearly every register, and control flow around its MFMAs makes the
 //             compiler spill.  Without a K tail the reduction always ends this way (LMS = 1, NST = 4).
-template <bool KTAIL, int LMS = -1, int NST = 4>
+// PS: both operands bring their scale bytes in the packed form of alto_mxfp4_pack_scales -- [block of 512 K][row][16 bytes
+// in the order of the LDS row below, bytes beyond K = 127] -- with OperandView::scales the base of it and
+// OperandView::ss_k the bytes from one block to the next (rows x 16).  A block of a tile's 256 + 256 rows is then 8 runs of
+// 1 KB, which the eight waves move straight into LDS with one load each (no registers, no fix-up, no ds_write; 8 cache
+// lines per load instead of the 64 of per-row scale rows).  Needs the end of K at compile time (LMS >= 0, or no K tail).
+template <bool KTAIL, int LMS = -1, int NST = 4, bool PS = false>
 __device__ __forceinline__ void gemm_tile_mainloop(const TileArgs& ta, TileAcc& acc, uint8_t* smem) {
+  static_assert(!PS || !KTAIL || LMS >= 0, "packed scales: the end of K must be known at compile time");
+  constexpr int SP = PS ? 4 : GT_SCALE_PITCH;   // dwords per row of a scale buffer in LDS
   TileLoader ld;
   v4i_t sraw;   // scale bytes of a later block, as loaded
   __syncthreads();   // the LDS ring may still be read by a previous call
@@ -268,8 +275,8 @@ __device__ __forceinline__ void gemm_tile_mainloop(const TileArgs& ta, TileAcc& 
     b_off = GT_TM * 128 + (uint32_t)(64 * wn + r) * 128 + c0;
   }
   // scale read offsets (bytes): row * 20 + 8h within a block buffer
-  const uint32_t sa_off = (uint32_t)(128 * wm + r) * (GT_SCALE_PITCH * 4) + 8 * h;
-  const uint32_t sb_off = (uint32_t)(GT_TM + 64 * wn + r) * (GT_SCALE_PITCH * 4) + 8 * h;
+  const uint32_t sa_off = (uint32_t)(128 * wm + r) * (SP * 4) + 8 * h;
+  const uint32_t sb_off = (uint32_t)(GT_TM + 64 * wn + r) * (SP * 4) + 8 * h;
 
   // LDS row layout (4 dwords): [h=0: K 0..255 | h=0: K 256..511 | h=1: K 0..255 | h=1: K 256..511], where the half-wave h
   // of the MFMA uses group 8 ms + 2 j + h at K step j of macro stage ms: byte j of dword 2 h + ms.
@@ -303,16 +310,28 @@ __device__ __forceinline__ void gemm_tile_mainloop(const TileArgs& ta, TileAcc& 
   auto read_scales = [&](const uint8_t* sblock, int (&xa)[4][2], int (&xb)[2][2]) {
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
-      const uint32_t* p = reinterpret_cast<const uint32_t*>(sblock + sa_off + t * 32 * GT_SCALE_PITCH * 4);
+      const uint32_t* p = reinterpret_cast<const uint32_t*>(sblock + sa_off + t * 32 * SP * 4);
       xa[t][0] = (int)p[0];
       xa[t][1] = (int)p[1];
     }
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
-      const uint32_t* p = reinterpret_cast<const uint32_t*>(sblock + sb_off + u * 32 * GT_SCALE_PITCH * 4);
+      const uint32_t* p = reinterpret_cast<const uint32_t*>(sblock + sb_off + u * 32 * SP * 4);
       xb[u][0] = (int)p[0];
       xb[u][1] = (int)p[1];
     }
+  };
+  // packed scales: block kb of this wave's 64 rows (waves 0-3: A rows, 4-7: B rows), 1 KB, straight into scale buffer kb & 1
+  const bool ps_a = wave < GT_TM / 64;   // scalar
+  const __amdgpu_buffer_rsrc_t rsrc_ps = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(ps_a ? ta.A.scales : ta.B.scales), 0,
+                                                                           (int)(ps_a ? ta.as_bytes : ta.bs_bytes), 0x00020000);
+  const int ps_row0 = __builtin_amdgcn_readfirstlane((int)((ps_a ? ta.m0 + 64 * wave : ta.n0 + 64 * (wave - GT_TM / 64)) * 16));
+  const int ps_blk = __builtin_amdgcn_readfirstlane((int)(ps_a ? ta.A.ss_k : ta.B.ss_k));
+  auto sdma = [&](int kb) {
+    typedef __attribute__((address_space(3))) uint8_t lds_u8s;
+    const int so = __builtin_amdgcn_readfirstlane(kb * ps_blk + ps_row0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_ps, (__attribute__((address_space(3))) void*)((lds_u8s*)sscale + (kb & 1) * (GT_TM + GT_TN) * SP * 4 + wave * 1024), 16,
+                                             lane * 16, so, 0, 0);
   };
   // 8 MFMAs of K step J (0..3) of macro stage MS (0..1 inside its 512-K block): scale byte J of dword MS
   auto mfma8 = [&](auto msc, auto jc, const v8i_t (&fa)[4], const v8i_t (&fb)[2]) {
@@ -374,13 +393,17 @@ __device__ __forceinline__ void gemm_tile_mainloop(const TileArgs& ta, TileAcc& 
     asm volatile("s_barrier" ::: "memory");
     __builtin_amdgcn_s_setprio(3);
     if constexpr (MS == 0 && !PEN) {
-      swrite(kb + 1, fastc);   // block kb+1 -> the other scale buffer (last read at the end of block kb-1)
-      ld.template sload<KTAIL>(kb + 2, sraw);
+      if constexpr (PS) {
+        sdma(kb + 1);            // block kb+1 -> the other scale buffer; this block's second stage waits for it
+      } else {
+        swrite(kb + 1, fastc);   // block kb+1 -> the other scale buffer (last read at the end of block kb-1)
+        ld.template sload<KTAIL>(kb + 2, sraw);
+      }
       __builtin_amdgcn_sched_barrier(0);
     }
     if constexpr (!PEN) ld.gload(smem, s + 2, MS, 0, 4);
     if constexpr (MS == 1)   // the next block's scales (in LDS since this stage's barrier) ride along with the last step
-      read_scales(reinterpret_cast<const uint8_t*>(sscale + ((kb + 1) & 1) * GT_SCALE_BUF_DW), sa_next, sb_next);
+      read_scales(reinterpret_cast<const uint8_t*>(sscale + ((kb + 1) & 1) * (GT_TM + GT_TN) * SP), sa_next, sb_next);
     mfma8(msc, std::integral_constant<int, 3>{}, fa1, fb1);
     read_frags(MS ^ 1, 0, fa0, fb0);
     if constexpr (PEN) interleave();
@@ -392,10 +415,16 @@ __device__ __forceinline__ void gemm_tile_mainloop(const TileArgs& ta, TileAcc& 
   // and the first block's scales in registers.  Stages beyond K load zeros and blocks beyond K load unit scales, so
   // nothing below is conditional.
   ld.init(ta);
-  ld.template sload<KTAIL>(0, sraw);
-  ld.gload(smem, 0, 0, 0, 8);
-  swrite(0, std::false_type{});
-  ld.template sload<KTAIL>(1, sraw);
+  if constexpr (PS) {
+    sdma(0);
+    ld.gload(smem, 0, 0, 0, 8);
+    (void)sraw;
+  } else {
+    ld.template sload<KTAIL>(0, sraw);
+    ld.gload(smem, 0, 0, 0, 8);
+    swrite(0, std::false_type{});
+    ld.template sload<KTAIL>(1, sraw);
+  }
   ld.gload(smem, 1, 1, 0, 4);   // the other half goes out in the first step of the loop
   asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)\n\ts_barrier" ::: "memory");   // all but stage 1's four loads
   read_frags(0, 0, fa0, fb0);
@@ -419,7 +448,7 @@ __device__ __forceinline__ void gemm_tile_mainloop(const TileArgs& ta, TileAcc& 
 #pragma unroll
     for (int u = 0; u < 2; ++u) { sb[u][0] = sb_next[u][0]; sb[u][1] = sb_next[u][1]; }
   };
-  if constexpr (KTAIL) {
+  if constexpr (KTAIL && !PS) {
     // Iteration kb passes scale block kb + 1 on to LDS.  Only the last block that holds any K (KB - 1, passed on by
     // iteration KB - 2) can reach past its row or past K and needs its bytes fixed; earlier ones are used as loaded,
     // later ones are never read.  Three loops in a row rather than a test inside one: the tile needs nearly every
@@ -538,12 +567,12 @@ __device__ __forceinline__ void gemm_tile_store(const TileArgs& ta, TileAcc& acc
 }
 
 // LMS / NST: how the reduction ends, as in gemm_tile_mainloop.
-template <typename OutT, bool KTAIL, int LMS = -1, int NST = 4>
+template <typename OutT, bool KTAIL, int LMS = -1, int NST = 4, bool PS = false>
 __device__ __forceinline__ void gemm_tile_256x256(const TileArgs& ta, OutT* __restrict__ c, int64_t ldc, uint8_t* smem) {
   TileAcc acc;
   gemm_tile_zero(acc);
   // (with fp32 output and no K tail the specialised ending pushes the register allocation into spilling: plain loop there)
-  gemm_tile_mainloop<KTAIL, (!KTAIL && sizeof(OutT) == 4) ? -3 : LMS, NST>(ta, acc, smem);
+  gemm_tile_mainloop<KTAIL, (!KTAIL && sizeof(OutT) == 4) ? -3 : LMS, NST, PS>(ta, acc, smem);
   gemm_tile_store<OutT>(ta, acc, c, ldc, smem);
 }
 

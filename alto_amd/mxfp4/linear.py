@@ -113,6 +113,37 @@ def _canonical_operand(t: torch.Tensor, s: torch.Tensor, rows_first: bool, k_pac
     return transpose_codes(tv.transpose(0, 1)), sv
 
 
+def pack_scales(scales: torch.Tensor, rows: int, K: int, is_2d_block: bool = False) -> torch.Tensor:
+    """Scales of one GEMM operand ([rows or rows/32, K/32], any strides) -> the packed form the tile kernels read without a
+    detour through registers: uint8 ``[ceil(K/512), rows, 16]``, the 16 bytes of a row and 512-K block in the order the MFMA
+    loop uses them, bytes beyond K = 127.  An internal operand layout (no counterpart in the reference)."""
+    rt.require_gpu(scales)
+    assert scales.dim() == 2 and scales.dtype == torch.uint8
+    out = torch.empty((-(-(K // 32) // 16), rows, 16), dtype=torch.uint8, device=scales.device)
+    if out.numel():
+        rc = rt.lib().alto_mxfp4_pack_scales(scales.data_ptr(), scales.stride(0), scales.stride(1), int(is_2d_block), rows, K, out.data_ptr(),
+                                             rt.stream_ptr(scales.device))
+        check(rc, "alto_mxfp4_pack_scales")
+    return out
+
+
+def packed_gemm_supported(M: int, N: int, K: int) -> bool:
+    """Shapes the packed-scale kernel serves (the 256x256 tile kernel's conditions; anything else takes plain scales)."""
+    return M >= 128 and N >= 128 and K >= 512 and N % 8 == 0 and M * (K // 2) < 2 ** 31 and N * (K // 2) < 2 ** 31
+
+
+def gemm_packed(a_q: torch.Tensor, a_ps: torch.Tensor, b_q: torch.Tensor, b_ps: torch.Tensor, out_scale: float = 1.0) -> torch.Tensor:
+    """C [M, N] (bf16) = A [M, K] . B [N, K]^T with codes packed along K and scales in the form of :func:`pack_scales`."""
+    M, N, K = a_q.shape[0], b_q.shape[0], a_q.shape[1] * 2
+    assert b_q.shape[1] * 2 == K and a_q.stride(1) == 1 and b_q.stride(1) == 1
+    assert a_ps.shape == (-(-(K // 32) // 16), M, 16) and b_ps.shape == (-(-(K // 32) // 16), N, 16) and a_ps.is_contiguous() and b_ps.is_contiguous()
+    c = torch.empty((M, N), dtype=torch.bfloat16, device=a_q.device)
+    rc = rt.lib().alto_mxfp4_gemm_ps(a_q.data_ptr(), a_q.stride(0), a_ps.data_ptr(), b_q.data_ptr(), b_q.stride(0), b_ps.data_ptr(), M, N, K,
+                                     c.data_ptr(), c.stride(0), float(out_scale), rt.stream_ptr(a_q.device))
+    check(rc, "alto_mxfp4_gemm_ps")
+    return c
+
+
 def blockwise_mxfp4_gemm(
     a: torch.Tensor,
     a_s: torch.Tensor,

@@ -273,6 +273,23 @@ class VendorGemm(Gemm):
         return torch._scaled_mm(a, b.t(), self.as_.view(torch.float8_e8m0fnu), self.bs.view(torch.float8_e8m0fnu), out_dtype=torch.bfloat16)
 
 
+class GemmPacked(Gemm):
+    """The same GEMM on operands whose scales are in the packed, GEMM-ready layout (``pack_scales``; done in ``setup``)."""
+
+    def setup(self, dev, gen):
+        super().setup(dev, gen)
+        from alto_amd.mxfp4 import linear as L
+        self.L = L
+        self.aps = L.pack_scales(self.as_, self.M, self.K, self.a_2d)
+        self.bps = L.pack_scales(self.bs, self.N, self.K, self.b_2d)
+
+    def step(self):
+        return self.L.gemm_packed(self.aq, self.aps, self.bq, self.bps)
+
+    def cpu_sample(self):
+        raise NotImplementedError("reported beside the plain-scale workload, which carries the CPU leg")
+
+
 class GroupedGemm(Workload):
     """Config 5: 32 experts, hidden 2880 -> 5760, 65536 routed rows with Zipf(1.1) expert skew, ragged int32 offsets [33]."""
     name = "cfg5_grouped_gemm[65536x5760x2880,E=32]"
@@ -523,6 +540,8 @@ def load_traffic(key):
 def make_workloads():
     return {
         "cfg3_fprop": Gemm("cfg3_fprop_gemm[8192x14336x4096]", 8192, 14336, 4096, False, True, "act", "weight"),
+        "cfg3_fprop_packed": GemmPacked("cfg3_fprop_gemm_packed_scales[8192x14336x4096]", 8192, 14336, 4096, False, True, "act", "weight"),
+        "cfg4_wgrad_packed": GemmPacked("cfg4_wgrad_gemm_packed_scales[4096x14336x8192]", 4096, 14336, 8192, False, False, "grad", "act"),
         "cfg3_fprop_vendor": VendorGemm("cfg3_fprop_gemm[8192x14336x4096] via torch._scaled_mm (1D scales on both operands)", 8192, 14336, 4096, False, False,
                                         "act", "weight"),
         "cfg2_quant": FusedGradQuant(),

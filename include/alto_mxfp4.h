@@ -216,6 +216,27 @@ int alto_mxfp4_gemm(const uint8_t* a, int64_t lda, const uint8_t* a_scales, int6
                     int64_t M, int64_t N, int64_t K, void* c, int c_dtype, int64_t ldc, float out_scale, void* stream);
 
 /*
+ * Packed scales: an internal layout of the scale bytes of one GEMM operand that the 256x256 tile kernels move into LDS
+ * with one load per wave and 512-K block, without registers, fix-ups or LDS writes (2 to 5 % of a GEMM).  No counterpart
+ * in the reference.  For an operand of `rows` rows and K / 32 groups:
+ *   packed[(kb * rows + row) * 16 + 4 * (2 h + ms) + j] = scale of group 16 kb + 8 ms + 2 j + h of that row
+ *   (kb < ceil(K / 512); h, ms in {0, 1}; j < 4), and 127 where that group lies beyond K.
+ * alto_mxfp4_pack_scales builds it from plain scales (1D: element (row, g) at scales[row * ss_r + g * ss_k]; 2D: row / 32
+ * instead of row); alto_mxfp4_packed_scales_bytes is its size.  The quantizers write it directly when asked to
+ * (alto_mxfp4_quantize_packed below).
+ */
+int64_t alto_mxfp4_packed_scales_bytes(int64_t rows, int64_t K);
+int alto_mxfp4_pack_scales(const uint8_t* scales, int64_t ss_r, int64_t ss_k, int is_2d, int64_t rows, int64_t K, uint8_t* packed, void* stream);
+
+/*
+ * alto_mxfp4_gemm on operands with packed scales, bf16 output: c[M][N] = a[M][K] . b[N][K]^T * out_scale.  Same results as
+ * alto_mxfp4_gemm, bit for bit.  Serves the shapes of the tile kernel only (M, N >= 128, K >= 512, N % 8 == 0, ldc % 8 ==
+ * 0, 16-byte aligned c): ALTO_MXFP4_ENOTIMPL otherwise, and the caller keeps plain scales for those.
+ */
+int alto_mxfp4_gemm_ps(const uint8_t* a, int64_t lda, const uint8_t* a_packed, const uint8_t* b, int64_t ldb, const uint8_t* b_packed,
+                       int64_t M, int64_t N, int64_t K, void* c, int64_t ldc, float out_scale, void* stream);
+
+/*
  * Ragged grouped GEMM for MoE experts.  Rows [offs[g], offs[g+1]) of A form group g and use
  * expert e(g) = group_expert ? group_expert[g] : g:
  *   out[r][:] = A[r][:] . W[e]^T,   W[e] = w + e * w_stride_e  ([N][K/2] bytes, row stride ldw),
