@@ -51,6 +51,8 @@ SIGNATURES = {
     "alto_mxfp4_packed_scales_bytes": (c_i64, [c_i64, c_i64]),
     "alto_mxfp4_pack_scales": (c_int, [c_vp, c_i64, c_i64, c_int, c_i64, c_i64, c_vp, c_vp]),
     "alto_mxfp4_gemm_ps": (c_int, [c_vp, c_i64, c_vp, c_vp, c_i64, c_vp, c_i64, c_i64, c_i64, c_vp, c_i64, c_f32, c_vp]),
+    "alto_mxfp4_grouped_gemm_ps": (c_int, [c_vp, c_i64, c_vp, c_vp, c_i64, c_i64, c_vp, c_i64, c_vp, c_vp, c_int, c_int, c_i64, c_i64, c_i64, c_vp, c_i64,
+                                          c_vp, c_i64, c_int, c_vp]),
     "alto_mxfp4_grouped_gemm": (c_int, [c_vp, c_i64, c_vp, c_i64, c_i64, c_int,
                                         c_vp, c_i64, c_i64, c_vp, c_i64, c_i64, c_i64, c_int,
                                         c_vp, c_vp, c_int, c_int, c_i64, c_i64, c_i64, c_vp, c_int, c_i64, c_vp, c_i64, c_vp]),

@@ -295,7 +295,7 @@ __global__ __launch_bounds__(PLAN_THREADS) void grouped_plan_kernel(PassWalk wk,
   if (t == PLAN_THREADS - 1) ws[0] = upto < max_pass ? upto : max_pass;
 }
 
-template <typename OutT, bool KTAIL, int LMS, int NST>
+template <typename OutT, bool KTAIL, int LMS, int NST, bool PS>
 __global__ __launch_bounds__(GT_THREADS) void grouped_tiled_kernel(OperandView A, const uint8_t* w, int64_t w_stride_e, int64_t ldw,
                                                                    const uint8_t* w_scales, int64_t ws_stride_e, int64_t ws_r, int w_is_2d,
                                                                    const int32_t* plan, int64_t M_total, int64_t N, int G, OutT* out, int64_t ldo, int tiles_n) {
@@ -312,11 +312,13 @@ __global__ __launch_bounds__(GT_THREADS) void grouped_tiled_kernel(OperandView A
     zero_rows<OutT>(out, ldo, m_lo, m_hi, n0, n1);
     return;
   }
-  OperandView B{w + e * w_stride_e, ldw, w_scales + e * ws_stride_e, ws_r, 1, w_is_2d};
+  // (packed scales: A.scales / w_scales + e * ws_stride_e are the packed bases, ss_k the bytes from block to block)
+  OperandView B{w + e * w_stride_e, ldw, w_scales + e * ws_stride_e, ws_r, PS ? N * 16 : 1, w_is_2d};
+  const int KB = (G + 15) / 16;
   TileArgs ta{A, B, row0, n0, m_lo, m_hi, N, G, 1.0f,
               (M_total - 1) * A.ld + G * 16, (N - 1) * ldw + G * 16,
-              ((A.is_2d ? M_total / 32 : M_total) - 1) * A.ss_r + G, ((w_is_2d ? N / 32 : N) - 1) * ws_r + G, 0, G};
-  gemm_tile_256x256<OutT, KTAIL, LMS, NST>(ta, out, ldo, smem);
+              PS ? KB * A.ss_k : ((A.is_2d ? M_total / 32 : M_total) - 1) * A.ss_r + G, PS ? KB * N * 16 : ((w_is_2d ? N / 32 : N) - 1) * ws_r + G, 0, G};
+  gemm_tile_256x256<OutT, KTAIL, LMS, NST, PS>(ta, out, ldo, smem);
 }
 
 // dW[e] tile: rows [256 tm, +256) of the first operand (P) x rows [256 tn, +256) of the second (Q), reduced over the
@@ -456,13 +458,13 @@ __global__ __launch_bounds__(GT_THREADS) void grouped_dw_tiled_kernel(OperandVie
 inline int64_t grouped_max_passes(int64_t M_total, int64_t num_groups) { return (M_total + GT_TM - 1) / GT_TM + num_groups + 2; }
 inline int64_t grouped_workspace_bytes(int64_t M_total, int64_t num_groups) { return 16 + 16 * grouped_max_passes(M_total, num_groups); }
 
-template <typename OutT, bool KTAIL, int LMS = -1, int NST = 4>
+template <typename OutT, bool KTAIL, int LMS = -1, int NST = 4, bool PS = false>
 int launch_grouped_tiled(const OperandView& A, const uint8_t* w, int64_t w_stride_e, int64_t ldw, const uint8_t* w_scales, int64_t ws_stride_e,
                          int64_t ws_r, int w_is_2d, const int32_t* offs, const int32_t* group_expert, int num_groups, int num_experts,
                          int64_t M_total, int64_t N, int64_t K, void* out, int64_t ldo, int32_t* plan, bool build_plan, hipStream_t st) {
   // the opt-in for > 64 KB of dynamic LDS is per function, set once per process (thread-safe: forward and backward may
   // make their first calls from two host threads)
-  auto kern = grouped_tiled_kernel<OutT, KTAIL, LMS, NST>;
+  auto kern = grouped_tiled_kernel<OutT, KTAIL, LMS, NST, PS>;
   static std::once_flag once;
   static hipError_t attr_rc = hipSuccess;
   std::call_once(once, [&] { attr_rc = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, GT_LDS_BYTES); });
@@ -514,7 +516,7 @@ int grouped_gemm_impl(const uint8_t* a, int64_t lda, const uint8_t* a_scales, in
                       const uint8_t* w_scales, int64_t ws_stride_e, int64_t ws_r, int64_t ws_k, int w_is_2d,
                       const int32_t* offs, const int32_t* group_expert, int num_groups, int num_experts,
                       int64_t M_total, int64_t N, int64_t K, void* out, int out_dtype, int64_t ldo,
-                      void* plan, int64_t plan_bytes, const char* plan_name, bool build_plan, void* stream) {
+                      void* plan, int64_t plan_bytes, const char* plan_name, bool build_plan, void* stream, bool ps = false) {
   ALTO_REQUIRE(a && a_scales && w && w_scales && offs && out, "grouped_gemm: NULL pointer");
   ALTO_REQUIRE(num_groups > 0 && num_groups <= 65536, "grouped_gemm: num_groups (%d) out of range", num_groups);
   ALTO_REQUIRE(group_expert != nullptr || num_groups == num_experts, "grouped_gemm: without group_expert, num_groups must equal num_experts");
@@ -529,13 +531,17 @@ int grouped_gemm_impl(const uint8_t* a, int64_t lda, const uint8_t* a_scales, in
   ALTO_REQUIRE(out_dtype == ALTO_DT_BF16 || out_dtype == ALTO_DT_F32, "grouped_gemm: bad out_dtype %d", out_dtype);
   if (M_total == 0 || N == 0) return ALTO_MXFP4_OK;
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-  OperandView A{a, lda, a_scales, a_ss_r, a_ss_k, a_is_2d};
+  OperandView A{a, lda, a_scales, a_ss_r, ps ? M_total * 16 : a_ss_k, a_is_2d};
   // 256x256 tiles when the problem fills them and the layouts fit their loads (unit-stride scale rows, 32-bit buffer
   // offsets, 16-byte output chunks); otherwise the direct kernel below
   const bool tiled = M_total >= 128 && N >= 128 && K >= 512 && a_ss_k == 1 && ws_k == 1 && N % 8 == 0 && ldo % 8 == 0 &&
                      (reinterpret_cast<uintptr_t>(out) & 15) == 0 && M_total * lda < (1ll << 31) && N * ldw < (1ll << 31) &&
                      M_total * a_ss_r < (1ll << 31) && N * ws_r < (1ll << 31) &&
                      grouped_max_passes(M_total, num_groups) * ((N + GT_TN - 1) / GT_TN) < (1ll << 28);
+  if (ps && !(tiled && out_dtype == ALTO_DT_BF16)) {
+    set_error("grouped_gemm_ps: shape (%lld, %lld, %lld) is not served by the tile kernel; use plain scales", (long long)M_total, (long long)N, (long long)K);
+    return ALTO_MXFP4_ENOTIMPL;
+  }
   if (tiled) {
     const int64_t need = grouped_workspace_bytes(M_total, num_groups);
     ALTO_REQUIRE(plan != nullptr && plan_bytes >= need && (reinterpret_cast<uintptr_t>(plan) & 15) == 0,
@@ -545,7 +551,21 @@ int grouped_gemm_impl(const uint8_t* a, int64_t lda, const uint8_t* a_scales, in
     int32_t* pl = reinterpret_cast<int32_t*>(plan);
     int rc = -1;
 #define ALTO_GROUPED_LAUNCH(T, ...) launch_grouped_tiled<T, __VA_ARGS__>(A, w, w_stride_e, ldw, w_scales, ws_stride_e, ws_r, w_is_2d, offs, group_expert, num_groups, num_experts, M_total, N, K, out, ldo, pl, build_plan, st)
-    if (!tail) {
+    if (ps) {
+      int lms = -1, nst = 4;
+      if (tail) gemm_tile_last_stage(K / 32, lms, nst);
+      switch (tail ? lms * 4 + nst - 1 : -1) {
+        case -1: rc = ALTO_GROUPED_LAUNCH(__bf16, false, -1, 4, true); break;
+        case 0: rc = ALTO_GROUPED_LAUNCH(__bf16, true, 0, 1, true); break;
+        case 1: rc = ALTO_GROUPED_LAUNCH(__bf16, true, 0, 2, true); break;
+        case 2: rc = ALTO_GROUPED_LAUNCH(__bf16, true, 0, 3, true); break;
+        case 3: rc = ALTO_GROUPED_LAUNCH(__bf16, true, 0, 4, true); break;
+        case 4: rc = ALTO_GROUPED_LAUNCH(__bf16, true, 1, 1, true); break;
+        case 5: rc = ALTO_GROUPED_LAUNCH(__bf16, true, 1, 2, true); break;
+        case 6: rc = ALTO_GROUPED_LAUNCH(__bf16, true, 1, 3, true); break;
+        default: rc = ALTO_GROUPED_LAUNCH(__bf16, true, 1, 4, true); break;
+      }
+    } else if (!tail) {
       rc = out_dtype == ALTO_DT_BF16 ? ALTO_GROUPED_LAUNCH(__bf16, false) : ALTO_GROUPED_LAUNCH(float, false);
     } else if (out_dtype != ALTO_DT_BF16) {
       rc = ALTO_GROUPED_LAUNCH(float, true);   // (fp32 output: the general ending)
@@ -611,6 +631,19 @@ extern "C" int alto_mxfp4_grouped_gemm_planned(const uint8_t* a, int64_t lda, co
   return alto::grouped_gemm_impl(a, lda, a_scales, a_ss_r, a_ss_k, a_is_2d, w, w_stride_e, ldw, w_scales, ws_stride_e, ws_r, ws_k, w_is_2d, offs, group_expert,
                                  num_groups, num_experts, M_total, N, K, out, out_dtype, ldo, const_cast<void*>(workspace), workspace_bytes, "the workspace",
                                  false, stream);
+}
+
+extern "C" int alto_mxfp4_grouped_gemm_ps(const uint8_t* a, int64_t lda, const uint8_t* a_packed, const uint8_t* w, int64_t w_stride_e, int64_t ldw,
+                                          const uint8_t* w_packed, int64_t wp_stride_e, const int32_t* offs, const int32_t* group_expert,
+                                          int num_groups, int num_experts, int64_t M_total, int64_t N, int64_t K, void* out, int64_t ldo,
+                                          void* workspace, int64_t workspace_bytes, int plan_built, void* stream) {
+  using namespace alto;
+  ALTO_REQUIRE(((reinterpret_cast<uintptr_t>(a_packed) | reinterpret_cast<uintptr_t>(w_packed) | (uintptr_t)wp_stride_e) & 15) == 0,
+               "grouped_gemm_ps: packed scales (and the stride between experts) must be 16-byte aligned");
+  ALTO_REQUIRE(K >= 0 && ((K / 32 + 15) / 16) * (M_total > N ? M_total : N) * 16 < (1ll << 31), "grouped_gemm_ps: packed scales beyond 2 GiB");
+  // A: [blocks][M_total][16]; expert e's weights: [blocks][N][16] at w_packed + e * wp_stride_e
+  return grouped_gemm_impl(a, lda, a_packed, 16, 1, 0, w, w_stride_e, ldw, w_packed, wp_stride_e, 16, 1, 0, offs, group_expert, num_groups, num_experts,
+                           M_total, N, K, out, ALTO_DT_BF16, ldo, workspace, workspace_bytes, "the workspace", plan_built == 0, stream, true);
 }
 
 extern "C" int alto_mxfp4_grouped_gemm_plan(const int32_t* offs, const int32_t* group_expert, int num_groups, int num_experts, int64_t M_total,

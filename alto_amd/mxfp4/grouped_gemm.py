@@ -95,6 +95,30 @@ def grouped_forward(a_q, a_s, w_q, w_s, groups: Groups, use_2dblock_x, use_2dblo
     return (out, ws) if return_plan else out
 
 
+def pack_expert_scales(w_s: torch.Tensor, N: int, K: int, is_2d_block: bool) -> torch.Tensor:
+    """Weight scales [E, N or N/32, K/32] -> packed [E, ceil(K/512), N, 16] (see ``linear.pack_scales``)."""
+    from .linear import pack_scales
+    return torch.stack([pack_scales(w_s[e], N, K, is_2d_block) for e in range(w_s.shape[0])])
+
+
+def grouped_forward_packed(a_q, a_ps, w_q, w_ps, groups: Groups, plan=None, return_plan=False):
+    """:func:`grouped_forward` on packed scales (bf16 output): ``a_ps`` [ceil(K/512), M, 16], ``w_ps`` [E, ceil(K/512), N, 16]."""
+    E, N = w_q.shape[0], w_q.shape[1]
+    M, K = a_q.shape[0], a_q.shape[1] * 2
+    assert w_q.shape[2] * 2 == K and a_q.stride(1) == 1 and w_q.stride(2) == 1
+    KB = -(-(K // 32) // 16)
+    assert a_ps.shape == (KB, M, 16) and w_ps.shape == (E, KB, N, 16) and a_ps.is_contiguous() and w_ps.is_contiguous()
+    out = torch.empty((M, N), dtype=torch.bfloat16, device=a_q.device)
+    ws_bytes = rt.lib().alto_mxfp4_grouped_gemm_workspace_bytes(M, groups.n)
+    ws = plan if plan is not None else torch.empty(ws_bytes, dtype=torch.uint8, device=a_q.device)
+    rc = rt.lib().alto_mxfp4_grouped_gemm_ps(
+        a_q.data_ptr(), a_q.stride(0), a_ps.data_ptr(), w_q.data_ptr(), w_q.stride(0), w_q.stride(1), w_ps.data_ptr(), w_ps.stride(0),
+        groups.offs.data_ptr(), rt.ptr(groups.expert), groups.n, E, M, N, K, out.data_ptr(), out.stride(0),
+        ws.data_ptr(), ws.numel(), int(plan is not None), rt.stream_ptr(a_q.device))
+    check(rc, "alto_mxfp4_grouped_gemm_ps")
+    return (out, ws) if return_plan else out
+
+
 def grouped_plan(groups: Groups, num_experts: int, m_total: int) -> torch.Tensor:
     """The pass list of ``groups`` over ``m_total`` rows, for ``grouped_forward(..., plan=...)``."""
     dev = groups.offs.device

@@ -341,6 +341,23 @@ class GroupedGemm(Workload):
         return run, 2.0 * rows * self.N * self.K, f"{rows} rows of the largest expert, dequantize + fp32 matmul"
 
 
+class GroupedGemmPacked(GroupedGemm):
+    """Config 5 forward on operands whose scales are in the packed, GEMM-ready layout (packed in ``setup``)."""
+    name = "cfg5_grouped_gemm_packed_scales[65536x5760x2880,E=32]"
+
+    def setup(self, dev, gen):
+        super().setup(dev, gen)
+        from alto_amd.mxfp4.linear import pack_scales
+        self.aps = pack_scales(self.as_, self.rows, self.K, False)
+        self.wps = self.G.pack_expert_scales(self.ws, self.wq.shape[1], self.K, True)
+
+    def step(self):
+        return self.G.grouped_forward_packed(self.aq, self.aps, self.wq, self.wps, self.groups)
+
+    def cpu_sample(self):
+        raise NotImplementedError("reported beside the plain-scale workload, which carries the CPU leg")
+
+
 class GroupedGemmDx(GroupedGemm):
     """Config 5 backward, input gradient: dX [65536, 2880] = dY [65536, 5760] . W[e] (reduction over N = 5760; the weights
     are the N-packed copy of their 2D-block quantisation), same ragged offsets."""
@@ -366,6 +383,20 @@ class GroupedGemmDx(GroupedGemm):
 
     def cpu_sample(self):
         raise NotImplementedError("reported beside the forward workload, which carries the CPU leg")
+
+
+class GroupedGemmDxPacked(GroupedGemmDx):
+    """Config 5 input gradient on packed scales, pass list reused."""
+    name = "cfg5_grouped_dx_packed_scales[65536x2880x5760,E=32]"
+
+    def setup(self, dev, gen):
+        super().setup(dev, gen)
+        from alto_amd.mxfp4.linear import pack_scales
+        self.aps = pack_scales(self.as_, self.rows, self.aq.shape[1] * 2, False)
+        self.wps = self.G.pack_expert_scales(self.ws, self.wq.shape[1], self.aq.shape[1] * 2, True)
+
+    def step(self):
+        return self.G.grouped_forward_packed(self.aq, self.aps, self.wq, self.wps, self.groups, plan=self.plan)
 
 
 class GroupedGemmDw(GroupedGemm):
@@ -553,6 +584,8 @@ def make_workloads():
         "cfg4_wgrad": Gemm("cfg4_wgrad_gemm[4096x14336x8192]", 4096, 14336, 8192, False, False, "grad", "act"),
         "cfg5_grouped": GroupedGemm(),
         "cfg5_grouped_dx": GroupedGemmDx(),
+        "cfg5_grouped_packed": GroupedGemmPacked(),
+        "cfg5_grouped_dx_packed": GroupedGemmDxPacked(),
         "cfg5_grouped_dw": GroupedGemmDw(),
         "attn_fwd": AttentionFwd(),
         "linear_step": LinearStep(False),

@@ -281,6 +281,18 @@ int alto_mxfp4_grouped_gemm_planned(const uint8_t* a, int64_t lda, const uint8_t
                                     const void* workspace, int64_t workspace_bytes, void* stream);
 
 /*
+ * alto_mxfp4_grouped_gemm on operands with packed scales (alto_mxfp4_pack_scales), bf16 output: a_packed is the packed form
+ * of the [M_total][K/32] activation scales, w_packed + e * wp_stride_e that of expert e's weight scales ([N] rows).
+ * plan_built != 0: `workspace` already holds the pass list for these groups (alto_mxfp4_grouped_gemm_plan or an earlier
+ * call), as in alto_mxfp4_grouped_gemm_planned.  Same results as alto_mxfp4_grouped_gemm, bit for bit; serves the tile
+ * kernel's shapes only (ALTO_MXFP4_ENOTIMPL otherwise).  No counterpart in the reference.
+ */
+int alto_mxfp4_grouped_gemm_ps(const uint8_t* a, int64_t lda, const uint8_t* a_packed, const uint8_t* w, int64_t w_stride_e, int64_t ldw,
+                               const uint8_t* w_packed, int64_t wp_stride_e, const int32_t* offs, const int32_t* group_expert,
+                               int num_groups, int num_experts, int64_t M_total, int64_t N, int64_t K, void* out, int64_t ldo,
+                               void* workspace, int64_t workspace_bytes, int plan_built, void* stream);
+
+/*
  * Per-device set-up that the entry points otherwise do on first use: resolves, for the CURRENT device, the address of the
  * library's built-in pass-list array.  Call it once per device (with that device current) before capturing a HIP graph
  * that contains alto_mxfp4_grouped_gemm_noalloc.  Idempotent, thread-safe, allocates nothing.  No counterpart in the

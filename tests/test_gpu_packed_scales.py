@@ -71,3 +71,29 @@ def test_packed_gemm_rejects_what_the_tile_kernel_does_not_serve(m):
     aq, as_ = m.convert_to_mxfp4(a)
     with pytest.raises(RuntimeError, match="not served by the tile kernel"):
         gemm_packed(aq, pack_scales(as_, M, K), aq, pack_scales(as_, N, K))
+
+
+@pytest.mark.parametrize("N,K", [(768, 1280), (800, 608), (512, 2880), (264, 512)])
+@pytest.mark.parametrize("sorted_form", [True, False])
+def test_grouped_gemm_with_packed_scales_equals_the_plain_call(m, N, K, sorted_form):
+    from alto_amd.mxfp4 import grouped_gemm as G
+    from alto_amd.mxfp4.linear import pack_scales
+    if N % 32:
+        pytest.skip("2D weight blocks need N % 32 == 0")
+    E, M = 5, 1536
+    if sorted_form:
+        ends = torch.tensor([200, 200, 777, 1300, 1500]).to(torch.int32)
+        groups = G.groups_from_offsets(G.offsets_from_ends(ends.to(DEV)))
+    else:
+        idx = torch.randint(0, E, (M // 128,), generator=torch.Generator().manual_seed(3), dtype=torch.int32).repeat_interleave(128)
+        groups = G.groups_from_indices(idx.to(DEV))
+    a = randn_outliers((M, K), torch.bfloat16, seed=31).to(DEV)
+    w = (randn_outliers((E, N, K), torch.bfloat16, seed=32) * 0.05).to(DEV)
+    aq, as_ = m.convert_to_mxfp4(a)
+    wq, ws = m.convert_to_mxfp4(w, is_2d_block=True)
+    want = G.grouped_forward(aq, as_, wq, ws, groups, False, True, torch.bfloat16)
+    a_ps, w_ps = pack_scales(as_, M, K), G.pack_expert_scales(ws, N, K, True)
+    got, plan = G.grouped_forward_packed(aq, a_ps, wq, w_ps, groups, return_plan=True)
+    assert torch.equal(got, want)
+    again = G.grouped_forward_packed(aq, a_ps, wq, w_ps, groups, plan=plan)
+    assert torch.equal(again, want)
