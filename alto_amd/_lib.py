@@ -40,6 +40,10 @@ SIGNATURES = {
                                           ctypes.c_uint64, ctypes.c_uint64, c_vp,
                                           c_int, c_vp, c_vp, c_int, c_int, c_vp]),
     "alto_mxfp4_quantize_sr_hw_words": (c_i64, [c_int, c_i64, c_i64, c_i64]),
+    "alto_mxfp4_quantize_ex": (c_int, [c_vp, c_int, c_i64, c_i64, c_i64, c_i64, c_i64,
+                                       c_vp, c_vp, c_vp, c_vp, c_i64, c_i64, c_int, c_int,
+                                       c_vp, c_i64, c_i64, ctypes.c_uint64, ctypes.c_uint64, c_vp,
+                                       c_int, c_vp, c_vp, c_int, c_int, c_int, c_vp]),
     "alto_mxfp4_philox_advance": (c_int, [c_vp, ctypes.c_uint64, c_vp]),
     "alto_mxfp4_hadamard": (c_int, [c_vp, c_int, c_i64, c_i64, c_i64, c_vp, c_i64, c_vp, c_vp, c_vp]),
     "alto_mxfp4_hadamard_apply": (c_int, [c_vp, c_int, c_i64, c_i64, c_i64, c_vp, c_i64, c_vp, c_vp, c_int, c_int, c_vp]),

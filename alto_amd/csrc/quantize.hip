@@ -38,7 +38,12 @@ struct QuantParams {
   int clip_row;          // 1: multiply by 3/4 (in the input dtype) before encoding the row output
   int clip_col;
   int uos;
+  int pack_rs, pack_cs;  // 1: the 1D row / column scales go out in the packed form of alto_mxfp4_pack_scales (batch == 1)
 };
+
+// byte position of K group g16 (0..15) inside the 16 bytes of a row and 512-K block of packed scales: 4 (2 h + ms) + j with
+// g16 = 8 ms + 2 j + h
+__device__ __forceinline__ int packed_scale_pos(int g16) { return 4 * (2 * (g16 & 1) + (g16 >> 3)) + ((g16 >> 1) & 3); }
 
 // byte k of a packed table that lives in scalar registers (k is a compile-time constant where this is used)
 __device__ __forceinline__ int packed_byte(const uint32_t (&t)[8], int k) { return (int)((t[k >> 2] >> (8 * (k & 3))) & 0xFFu); }
@@ -252,9 +257,24 @@ __global__ __launch_bounds__(256) void quant_kernel(const QuantParams p) {
     // descriptors of the row outputs start at the tile's first row
     const __amdgpu_buffer_rsrc_t rsrc_rc = __builtin_amdgcn_make_buffer_rsrc(
         DO_ROW ? p.row_codes + (b * M + row0) * p.ld_rc : nullptr, 0, DO_ROW ? 0x7FFFFFFF : 0, 0x00020000);
+    // Row scales, plain: [M][C/32], the byte of (row, group g) at row * (C/32) + g.  Packed (one matrix): the 16 groups of
+    // a row's 512-element block share 16 bytes, ((g / 16) M + row) 16 + packed_scale_pos(g % 16).  One store serves both:
+    // the row pitch and the lane's column term are chosen here, outside the loop.
+    const bool prs = DO_ROW && !B2D && p.pack_rs;
+    const int ldrs = prs ? 16 : C / 32;
+    const int rs_col = prs ? ((c >> 9) * M) * 16 + packed_scale_pos((c >> 5) & 15) : (c >> 5);
     const __amdgpu_buffer_rsrc_t rsrc_rs = __builtin_amdgcn_make_buffer_rsrc(
-        (DO_ROW && !B2D) ? p.row_scales + (b * M + row0) * (int64_t)(C / 32) : nullptr, 0, (DO_ROW && !B2D) ? 0x7FFFFFFF : 0, 0x00020000);
-    const int ldrc = (int)p.ld_rc, ldrs = C / 32;
+        (DO_ROW && !B2D) ? p.row_scales + (prs ? (int64_t)row0 * 16 : (b * M + row0) * (int64_t)(C / 32)) : nullptr, 0,
+        (DO_ROW && !B2D) ? 0x7FFFFFFF : 0, 0x00020000);
+    const int ldrc = (int)p.ld_rc;
+    if (prs && ((C >> 5) & 15) != 0 && col0 + TILE_C >= C) {   // packed: the groups of the last block beyond C read as 127
+      const bool last = (tid & 3) == 0 && (c >> 5) == (C >> 5) - 1;
+      for (int gp = (C >> 5) & 15; gp < 16; ++gp) {
+        const int off = rsub * 16 + ((c >> 9) * M) * 16 + packed_scale_pos(gp);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) __builtin_amdgcn_raw_buffer_store_b8((uint8_t)127, rsrc_rs, (last && valid[i]) ? off : OOB, 8 * i * 16, 0);
+      }
+    }
     uint32_t blk = B2D ? blkmax[chunk >> 2] : 0;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -264,7 +284,9 @@ __global__ __launch_bounds__(256) void quant_kernel(const QuantParams p) {
       else s = BF ? e8m0_from_bf16_bits(a) : e8m0_from_f32_bits(a);
       // scales
       if (!B2D) {
-        if (DO_ROW) __builtin_amdgcn_raw_buffer_store_b8((uint8_t)s, rsrc_rs, (valid[i] && (tid & 3) == 0) ? rsub * ldrs + (c >> 5) : OOB, 8 * i * ldrs, 0);
+        if (DO_ROW) {
+          __builtin_amdgcn_raw_buffer_store_b8((uint8_t)s, rsrc_rs, (valid[i] && (tid & 3) == 0) ? rsub * ldrs + rs_col : OOB, 8 * i * ldrs, 0);
+        }
       } else if (i == 0 && rsub == 0 && (tid & 3) == 0 && valid[0]) {
         if (DO_ROW) p.row_scales[(b * (M / 32) + blockIdx.y) * (C / 32) + (c >> 5)] = (uint8_t)s;
         if (DO_COL) p.col_scales[(b * (C / 32) + (c >> 5)) * (M / 32) + blockIdx.y] = (uint8_t)s;
@@ -375,9 +397,19 @@ __global__ __launch_bounds__(256) void quant_kernel(const QuantParams p) {
       for (int k = 0; k < 32; k += 2) am = __builtin_fmaxf(__builtin_fmaxf(am, __builtin_fabsf(z[k])), __builtin_fabsf(z[k + 1]));
       if (GEN && p.uos) s = e8m0_uos(am);
       else s = BF ? e8m0_from_bf16_bits(f2u(am) >> 16) : e8m0_from_f32_bits(f2u(am));
+      // plain: [C][M/32], this band's byte of column cc at cc (M/32) + band.  Packed (one matrix): ((band / 16) C + cc) 16 +
+      // packed_scale_pos(band % 16); the last band also writes the 127s of the groups beyond M.
+      const bool pcs = p.pack_cs;
+      const int by = blockIdx.y, cs_pitch = pcs ? 16 : M / 32;
+      const uint8_t* cs_blk = p.col_scales + ((int64_t)(by >> 4) * C + col0) * 16;
       const __amdgpu_buffer_rsrc_t rsrc_cs = __builtin_amdgcn_make_buffer_rsrc(
-          p.col_scales + (b * C + col0) * (int64_t)(M / 32) + blockIdx.y, 0, 0x7FFFFFFF, 0x00020000);
-      __builtin_amdgcn_raw_buffer_store_b8((uint8_t)s, rsrc_cs, cvalid ? tid * (M / 32) : OOB, 0, 0);
+          const_cast<uint8_t*>(pcs ? cs_blk + packed_scale_pos(by & 15) : p.col_scales + (b * C + col0) * (int64_t)(M / 32) + by), 0, 0x7FFFFFFF, 0x00020000);
+      __builtin_amdgcn_raw_buffer_store_b8((uint8_t)s, rsrc_cs, cvalid ? tid * cs_pitch : OOB, 0, 0);
+      if (pcs && by == (M >> 5) - 1 && ((M >> 5) & 15) != 0) {
+        const __amdgpu_buffer_rsrc_t rsrc_pad = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(cs_blk), 0, 0x7FFFFFFF, 0x00020000);
+        for (int gp = (M >> 5) & 15; gp < 16; ++gp)
+          __builtin_amdgcn_raw_buffer_store_b8((uint8_t)127, rsrc_pad, cvalid ? tid * 16 + packed_scale_pos(gp) : OOB, 0, 0);
+      }
     }
     const float scale_f = u2f(s << 23);
     const float inv = u2f((254u - s) << 23);
@@ -651,7 +683,7 @@ int quantize_impl(const void* x, int dtype, int64_t batch, int64_t M, int64_t C,
                   uint8_t* row_codes, uint8_t* row_scales, uint8_t* col_codes, uint8_t* col_scales,
                   int64_t ld_row_codes, int64_t ld_col_codes, int is_2d, int sr_mode,
                   const uint32_t* rand_bits, int64_t ld_rand, int64_t bs_rand, uint64_t seed, uint64_t offset, const uint64_t* philox_state,
-                  int hadamard, const int8_t* signs, const uint8_t* perm, int clip_mode, int use_uos, void* stream) {
+                  int hadamard, const int8_t* signs, const uint8_t* perm, int clip_mode, int use_uos, void* stream, int flags = 0) {
   if (ld_row_codes == 0) ld_row_codes = C / 2;
   if (ld_col_codes == 0) ld_col_codes = M / 2;
   ALTO_REQUIRE(row_codes == nullptr || (ld_row_codes >= C / 2 && ld_row_codes % 4 == 0), "quantize: ld_row_codes must be >= C/2 and a multiple of 4 bytes");
@@ -680,6 +712,14 @@ int quantize_impl(const void* x, int dtype, int64_t batch, int64_t M, int64_t C,
   }
   ALTO_REQUIRE(!hadamard || (!is_2d && do_col), "quantize: the Hadamard transform applies to a 1D column output only");
   ALTO_REQUIRE(clip_mode == ALTO_CLIP_NONE || clip_mode == ALTO_CLIP_STATIC || clip_mode == ALTO_CLIP_DYNAMIC, "quantize: bad clip_mode %d", clip_mode);
+  const bool pack_rs = (flags & 1) != 0, pack_cs = (flags & 2) != 0;
+  if (pack_rs || pack_cs) {
+    ALTO_REQUIRE(batch <= 1 && !is_2d && clip_mode != ALTO_CLIP_DYNAMIC, "quantize: packed scales are written for one matrix with 1D blocks (no dynamic clip)");
+    ALTO_REQUIRE((!pack_rs || row_codes) && (!pack_cs || col_codes), "quantize: packed scales asked for an output that is not produced");
+    ALTO_REQUIRE(M % 32 == 0 && M * C < (1ll << 36), "quantize: packed scales need M %% 32 == 0 and M * C < 2^36");
+    ALTO_REQUIRE(((reinterpret_cast<uintptr_t>(pack_rs ? row_scales : nullptr) | reinterpret_cast<uintptr_t>(pack_cs ? col_scales : nullptr)) & 15) == 0,
+                 "quantize: packed scales must be 16-byte aligned");
+  }
   if (batch == 0 || M == 0 || C == 0) return ALTO_MXFP4_OK;
   if (clip_mode == ALTO_CLIP_DYNAMIC) {   // std-based scale: separate plain kernel, quantisation along the contiguous dim
     ALTO_REQUIRE(do_row && !do_col && !hadamard,
@@ -712,6 +752,8 @@ int quantize_impl(const void* x, int dtype, int64_t batch, int64_t M, int64_t C,
   if (!do_col) p.clip_col = 0;
   if (!do_row) p.clip_row = 0;
   p.uos = use_uos ? 1 : 0;
+  p.pack_rs = pack_rs ? 1 : 0;
+  p.pack_cs = pack_cs ? 1 : 0;
   const bool gen = p.clip_row || p.clip_col || p.uos;
 
   dim3 grid((unsigned)((C + TILE_C - 1) / TILE_C), (unsigned)((M + 31) / 32), (unsigned)batch);
@@ -774,6 +816,22 @@ extern "C" int alto_mxfp4_quantize_sr_hw(const void* x, int dtype, int64_t batch
 extern "C" int64_t alto_mxfp4_quantize_sr_hw_words(int dtype, int64_t batch, int64_t M, int64_t C) {
   const int64_t nb = (M + 31) / 32;
   return 4 * (dtype == ALTO_DT_BF16 ? 2 : 8) * batch * nb * C;
+}
+
+extern "C" int alto_mxfp4_quantize_ex(const void* x, int dtype, int64_t batch, int64_t M, int64_t C, int64_t ld_x, int64_t bs_x,
+                                      uint8_t* row_codes, uint8_t* row_scales, uint8_t* col_codes, uint8_t* col_scales,
+                                      int64_t ld_row_codes, int64_t ld_col_codes, int is_2d, int sr_mode,
+                                      const uint32_t* rand_bits, int64_t ld_rand, int64_t bs_rand, uint64_t seed, uint64_t offset,
+                                      const uint64_t* philox_state, int hadamard, const int8_t* signs, const uint8_t* perm,
+                                      int clip_mode, int use_uos, int flags, void* stream) {
+  using namespace alto;
+  ALTO_REQUIRE(sr_mode >= 0 && sr_mode <= 3, "quantize_ex: sr_mode %d is not 0 (nearest even), 1 (words given), 2 (Philox in the kernel) or 3 (hardware converts)", sr_mode);
+  ALTO_REQUIRE((flags & ~3) == 0, "quantize_ex: unknown flags 0x%x", flags);
+  ALTO_REQUIRE(sr_mode < 2 || C < (1ll << 26), "quantize_ex: C (%lld) out of range for words made in the kernel", (long long)C);
+  ALTO_REQUIRE(sr_mode < 2 || philox_state == nullptr || (reinterpret_cast<uintptr_t>(philox_state) & 7) == 0, "quantize_ex: philox_state must be 8-byte aligned");
+  return quantize_impl(x, dtype, batch, M, C, ld_x, bs_x, row_codes, row_scales, col_codes, col_scales, ld_row_codes, ld_col_codes, is_2d, sr_mode,
+                       sr_mode == 1 ? rand_bits : nullptr, ld_rand, bs_rand, seed, offset, sr_mode >= 2 ? philox_state : nullptr, hadamard, signs, perm,
+                       clip_mode, use_uos, stream, flags);
 }
 
 extern "C" int alto_mxfp4_philox_advance(uint64_t* philox_state, uint64_t words, void* stream) {

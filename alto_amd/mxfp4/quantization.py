@@ -49,23 +49,34 @@ def _code_buffer(B: int, R: int, nbytes: int, dev, pad: bool) -> torch.Tensor:
 
 def _quantize_call(x3: torch.Tensor, want_row: bool, want_col: bool, is_2d: bool, use_sr: bool,
                    rand3: Optional[torch.Tensor], hadamard: Optional[HadamardTransform], clip: int, use_uos: bool,
-                   pad_codes: bool = False, philox: Optional[Tuple[int, int]] = None, hw_sr: bool = False):
+                   pad_codes: bool = False, philox: Optional[Tuple[int, int]] = None, hw_sr: bool = False,
+                   pack_row_scales: bool = False, pack_col_scales: bool = False):
     """x3: [B, M, C] with unit stride along C and uniform row / batch strides. Returns the outputs (or None): dense, or
     with ``pad_codes`` code tensors whose rows are padded to whole 128-byte cache lines (for GEMM operands).
     ``philox = (seed, offset)`` with ``use_sr`` and no ``rand3``: the kernel makes the random words itself, element
     (b, i, j) taking word (b M + i) C + j of the stream ``alto_mxfp4_random_bits(.., seed, offset)`` writes.
     ``philox`` = an int64[2] device tensor {key, counter}: the same, with key and counter read on the device and the
     counter moved past the B M C words afterwards (nothing about the draw is a kernel argument: safe under graph capture).
-    ``hw_sr``: round with the hardware's stochastic converts (``alto_mxfp4_quantize_sr_hw``; needs ``philox``)."""
+    ``hw_sr``: round with the hardware's stochastic converts (``alto_mxfp4_quantize_sr_hw``; needs ``philox``).
+    ``pack_row_scales`` / ``pack_col_scales`` (one matrix, 1D blocks): that scale output comes in the packed form of
+    ``linear.pack_scales`` -- [1, ceil(C/512), M, 16] resp. [1, ceil(M/512), C, 16] -- written by the kernel itself."""
     B, M, C = x3.shape
     dev = x3.device
+    packed = pack_row_scales or pack_col_scales
+    assert not packed or (B == 1 and not is_2d), "packed scales: one matrix with 1D blocks"
     row_codes = row_scales = col_codes = col_scales = None
     if want_row:
         row_codes = _code_buffer(B, M, C // 2, dev, pad_codes)
-        row_scales = torch.empty((B, M // 32, C // 32) if is_2d else (B, M, C // 32), dtype=torch.uint8, device=dev)
+        if pack_row_scales:
+            row_scales = torch.empty((1, -(-(C // 32) // 16), M, 16), dtype=torch.uint8, device=dev)
+        else:
+            row_scales = torch.empty((B, M // 32, C // 32) if is_2d else (B, M, C // 32), dtype=torch.uint8, device=dev)
     if want_col:
         col_codes = _code_buffer(B, C, M // 2, dev, pad_codes)
-        col_scales = torch.empty((B, C // 32, M // 32) if is_2d else (B, C, M // 32), dtype=torch.uint8, device=dev)
+        if pack_col_scales:
+            col_scales = torch.empty((1, -(-(M // 32) // 16), C, 16), dtype=torch.uint8, device=dev)
+        else:
+            col_scales = torch.empty((B, C // 32, M // 32) if is_2d else (B, C, M // 32), dtype=torch.uint8, device=dev)
     had, sp, pp = _signs_perm_ptrs(hadamard)
     ld_x = x3.stride(1) if M > 1 else C
     bs_x = x3.stride(0) if B > 1 else M * ld_x
@@ -73,6 +84,25 @@ def _quantize_call(x3: torch.Tensor, want_row: bool, want_col: bool, is_2d: bool
     if use_sr and rand3 is not None:
         ld_r = rand3.stride(1) if M > 1 else C
         bs_r = rand3.stride(0) if B > 1 else M * ld_r
+    if packed:   # the general entry point: every rounding mode plus the layout flags
+        state, seed, offset, sr_mode = None, 0, 0, 0
+        if use_sr and rand3 is not None:
+            sr_mode = 1
+        elif use_sr:
+            assert philox is not None, "stochastic rounding needs rand_bits or a Philox (seed, offset)"
+            state = philox if isinstance(philox, torch.Tensor) else None
+            seed, offset = (0, 0) if state is not None else (philox[0] & (2 ** 64 - 1), philox[1] & (2 ** 64 - 1))
+            sr_mode = 3 if hw_sr else 2
+        rc = rt.lib().alto_mxfp4_quantize_ex(
+            x3.data_ptr(), rt.dtype_code(x3.dtype), B, M, C, ld_x, bs_x,
+            rt.ptr(row_codes), rt.ptr(row_scales), rt.ptr(col_codes), rt.ptr(col_scales),
+            row_codes.stride(1) if want_row else 0, col_codes.stride(1) if want_col else 0,
+            int(is_2d), sr_mode, rt.ptr(rand3) if sr_mode == 1 else None, ld_r, bs_r, seed, offset, rt.ptr(state),
+            had, sp, pp, clip, int(use_uos), int(pack_row_scales) | (int(pack_col_scales) << 1), rt.stream_ptr(dev))
+        check(rc, "alto_mxfp4_quantize_ex")
+        if state is not None:
+            rt.philox_advance(state, rt.lib().alto_mxfp4_quantize_sr_hw_words(rt.dtype_code(x3.dtype), B, M, C) if hw_sr else B * M * C)
+        return row_codes, row_scales, col_codes, col_scales
     if use_sr and rand3 is None:
         assert philox is not None, "stochastic rounding needs rand_bits or a Philox (seed, offset)"
         state = philox if isinstance(philox, torch.Tensor) else None
@@ -282,6 +312,8 @@ def quantize_rowcol(
     use_uos: bool = False,
     pad_codes: bool = False,
     use_asm: Optional[bool] = None,
+    pack_row_scales: bool = False,
+    pack_col_scales: bool = False,
 ):
     """One pass over a 2D ``x [M, C]`` producing BOTH quantisations the linear layer needs.
 
@@ -290,6 +322,10 @@ def quantize_rowcol(
     ``clip_mode`` applied there) and the row pair equals ``convert_to_mxfp4(x, axis=-1, ...)`` (no transform, no
     clipping).  Fuses mxfp_linear.py:310-315 with :383-396 (forward, x) and
     :466-494 (backward, dY); for 2D blocks it yields both packings of a weight from one read.
+
+    ``pack_row_scales`` / ``pack_col_scales`` (1D blocks, no dynamic clip): that scale output is the packed tensor
+    ``linear.pack_scales`` would make of it -- ``[ceil(C/512), M, 16]`` resp. ``[ceil(M/512), C, 16]`` -- written by the
+    quantizer itself, for ``linear.gemm_packed`` / ``grouped_gemm.grouped_forward_packed``.
     """
     assert x.dim() == 2 and x.dtype in (torch.float32, torch.bfloat16)
     rt.require_gpu(x)
@@ -310,6 +346,8 @@ def quantize_rowcol(
                 philox = rt.philox_seed_offset(None, None)
         else:
             rand_bits = rt.draw_rand_bits(x.shape, x.device)
+    torch._check(not (pack_row_scales or pack_col_scales) or (not is_2d_block and clip_mode != "dynamic"),
+                 lambda: "packed scales come with 1D blocks and without the dynamic clip")
     if clip_mode == "dynamic":   # the row pair is never clipped; the column pair takes the plain path
         rc, rs = convert_to_mxfp4(x, axis=-1, is_2d_block=is_2d_block, use_sr=use_sr, use_uos=use_uos, rand_bits=rand_bits)
         cc, cs = convert_to_mxfp4(x, axis=0, is_2d_block=is_2d_block, use_sr=use_sr, clip_mode="dynamic", use_uos=use_uos,
@@ -321,8 +359,9 @@ def quantize_rowcol(
         assert rand_bits.shape == x.shape
         r3 = _as_i32(rand_bits)
         r3 = _batched_view(r3 if r3.stride(-1) == 1 and r3.stride(0) % 4 == 0 and r3.data_ptr() % 16 == 0 else r3.contiguous())
-    rc, rs, cc, cs = _quantize_call(x3, True, True, is_2d_block, use_sr, r3, hadamard, clip, use_uos, pad_codes, philox=philox, hw_sr=hw_sr)
-    return rc[0], rs[0], cc[0].transpose(0, 1), cs[0].transpose(0, 1)
+    rc, rs, cc, cs = _quantize_call(x3, True, True, is_2d_block, use_sr, r3, hadamard, clip, use_uos, pad_codes, philox=philox, hw_sr=hw_sr,
+                                    pack_row_scales=pack_row_scales, pack_col_scales=pack_col_scales)
+    return rc[0], rs[0], cc[0].transpose(0, 1), cs[0] if pack_col_scales else cs[0].transpose(0, 1)
 
 
 def hadamard_apply(x: torch.Tensor, h: HadamardTransform, inverse: bool = False, left_mul: bool = False) -> torch.Tensor:

@@ -150,6 +150,27 @@ int alto_mxfp4_quantize_sr_hw(const void* x, int dtype, int64_t batch, int64_t M
 int64_t alto_mxfp4_quantize_sr_hw_words(int dtype, int64_t batch, int64_t M, int64_t C);
 
 /*
+ * The quantizer with every rounding mode behind one signature, plus output-layout flags.  sr_mode: 0 = nearest even
+ * (alto_mxfp4_quantize_pitched with use_sr = 0), 1 = stochastic with the words in rand_bits (the same call with use_sr =
+ * 1), 2 = alto_mxfp4_quantize_sr_philox, 3 = alto_mxfp4_quantize_sr_hw; arguments a mode does not use are ignored.
+ * Codes, and scales where no flag asks otherwise, are those calls' bit for bit.
+ * flags (one matrix: batch <= 1; 1D blocks: is_2d = 0; clip_mode not dynamic; ALTO_MXFP4_EINVAL / ENOTIMPL otherwise):
+ *   ALTO_QUANT_PACK_ROW_SCALES (1): row_scales receives the packed layout of alto_mxfp4_pack_scales for rows = M, K = C
+ *     (alto_mxfp4_packed_scales_bytes(M, C) bytes), pads included, instead of [M][C/32];
+ *   ALTO_QUANT_PACK_COL_SCALES (2): col_scales likewise for rows = C, K = M.
+ * The GEMMs on packed scales (alto_mxfp4_gemm_ps, alto_mxfp4_grouped_gemm_ps) then take the quantizer's output as it is.
+ * The reference has one layout only (mxfp_quantization.py:340-420 writes [M][C/32]); the flags have no counterpart there.
+ */
+#define ALTO_QUANT_PACK_ROW_SCALES 1
+#define ALTO_QUANT_PACK_COL_SCALES 2
+int alto_mxfp4_quantize_ex(const void* x, int dtype, int64_t batch, int64_t M, int64_t C, int64_t ld_x, int64_t bs_x,
+                           uint8_t* row_codes, uint8_t* row_scales, uint8_t* col_codes, uint8_t* col_scales,
+                           int64_t ld_row_codes, int64_t ld_col_codes, int is_2d, int sr_mode,
+                           const uint32_t* rand_bits, int64_t ld_rand, int64_t bs_rand, uint64_t seed, uint64_t offset,
+                           const uint64_t* philox_state, int hadamard, const int8_t* signs, const uint8_t* perm,
+                           int clip_mode, int use_uos, int flags, void* stream);
+
+/*
  * Moves the counter of a device-resident Philox state {key, counter} past `words` random words (counter += ceil(words / 4)),
  * enqueued on `stream` after the quantizer call that consumed them.  A one-thread kernel; it can be captured together
  * with that call.  No counterpart in the reference (its Philox offsets are host integers).
@@ -223,7 +244,7 @@ int alto_mxfp4_gemm(const uint8_t* a, int64_t lda, const uint8_t* a_scales, int6
  *   (kb < ceil(K / 512); h, ms in {0, 1}; j < 4), and 127 where that group lies beyond K.
  * alto_mxfp4_pack_scales builds it from plain scales (1D: element (row, g) at scales[row * ss_r + g * ss_k]; 2D: row / 32
  * instead of row); alto_mxfp4_packed_scales_bytes is its size.  The quantizers write it directly when asked to
- * (alto_mxfp4_quantize_packed below).
+ * (alto_mxfp4_quantize_ex, flags).
  */
 int64_t alto_mxfp4_packed_scales_bytes(int64_t rows, int64_t K);
 int alto_mxfp4_pack_scales(const uint8_t* scales, int64_t ss_r, int64_t ss_k, int is_2d, int64_t rows, int64_t K, uint8_t* packed, void* stream);

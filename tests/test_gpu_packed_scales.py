@@ -5,7 +5,7 @@ import pytest
 import torch
 
 import oracle as O
-from tests.helpers import assert_bytes_equal, randn_outliers
+from tests.helpers import assert_bytes_equal, hadamard_from_seed, randn_outliers
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -97,3 +97,52 @@ def test_grouped_gemm_with_packed_scales_equals_the_plain_call(m, N, K, sorted_f
     assert torch.equal(got, want)
     again = G.grouped_forward_packed(aq, a_ps, wq, w_ps, groups, plan=plan)
     assert torch.equal(again, want)
+
+
+@pytest.mark.parametrize("M,C", [(512, 512), (96, 1056), (1024, 2880), (544, 32), (32, 4096)])
+@pytest.mark.parametrize("mode", ["rne", "sr_words", "sr_philox", "sr_hw"])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_quantizer_writes_the_packed_scales_itself(m, M, C, mode, dtype):
+    """Codes and scales of the call with the layout flags equal those of the plain call, the scales after
+    ``pack_scales``: every rounding mode, with the Hadamard transform, static clip and K tails of both outputs."""
+    from alto_amd.mxfp4.linear import pack_scales
+    from alto_amd.mxfp4.quantization import _prep, _quantize_call
+    x = randn_outliers((M, C), dtype, seed=M + C).to(DEV)
+    h = m.HadamardTransform(*hadamard_from_seed(77))
+    rand = torch.randint(-2 ** 31, 2 ** 31 - 1, (1, M, C), dtype=torch.int32, generator=torch.Generator().manual_seed(3)).to(DEV)
+    kw = dict(use_sr=mode != "rne", rand3=rand if mode == "sr_words" else None, hadamard=h, clip=1, use_uos=False,
+              philox=(1234, 5678) if mode in ("sr_philox", "sr_hw") else None, hw_sr=mode == "sr_hw")
+    x3 = _prep(x)
+    rc, rs, cc, cs = _quantize_call(x3, True, True, False, **kw)
+    for pr, pc in [(True, True), (True, False), (False, True)]:
+        rc2, rs2, cc2, cs2 = _quantize_call(x3, True, True, False, pack_row_scales=pr, pack_col_scales=pc, **kw)
+        assert_bytes_equal(rc2.cpu(), rc.cpu(), "row codes")
+        assert_bytes_equal(cc2.cpu(), cc.cpu(), "column codes")
+        assert_bytes_equal(rs2[0].cpu(), (pack_scales(rs[0], M, C) if pr else rs[0]).cpu(), "row scales")
+        assert_bytes_equal(cs2[0].cpu(), (pack_scales(cs[0], C, M) if pc else cs[0]).cpu(), "column scales")
+    # one output only
+    rc3, rs3, _, _ = _quantize_call(x3, True, False, False, pack_row_scales=True, **{**kw, "hadamard": None, "clip": 0})
+    rc4, rs4, _, _ = _quantize_call(x3, True, False, False, **{**kw, "hadamard": None, "clip": 0})
+    assert_bytes_equal(rc3.cpu(), rc4.cpu(), "row codes alone")
+    assert_bytes_equal(rs3[0].cpu(), pack_scales(rs4[0], M, C).cpu(), "row scales alone")
+
+
+def test_quantize_rowcol_packed_feeds_the_packed_gemm(m):
+    from alto_amd.mxfp4.linear import gemm_packed
+    M, N, K = 384, 256, 1056
+    a = randn_outliers((M, K), torch.bfloat16, seed=1).to(DEV)
+    b = randn_outliers((N, K), torch.bfloat16, seed=2).to(DEV)
+    aq, as_, _, _ = m.quantize_rowcol(a)
+    bq, bs, _, _ = m.quantize_rowcol(b)
+    aq2, aps, _, _ = m.quantize_rowcol(a, pack_row_scales=True)
+    bq2, bps, _, _ = m.quantize_rowcol(b, pack_row_scales=True)
+    want = m.blockwise_mxfp4_gemm(aq, as_, bq, bs, trans_b=True, output_dtype=torch.bfloat16)
+    assert torch.equal(gemm_packed(aq2, aps, bq2, bps), want)
+
+
+def test_packed_flags_are_rejected_where_they_do_not_apply(m):
+    x = torch.randn(64, 64, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(RuntimeError, match="packed scales"):
+        m.quantize_rowcol(x, is_2d_block=True, pack_row_scales=True)
+    with pytest.raises(RuntimeError, match="packed scales"):
+        m.quantize_rowcol(x, clip_mode="dynamic", pack_col_scales=True)
