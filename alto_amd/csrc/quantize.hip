@@ -38,7 +38,7 @@ struct QuantParams {
   int clip_row;          // 1: multiply by 3/4 (in the input dtype) before encoding the row output
   int clip_col;
   int uos;
-  int pack_rs, pack_cs;  // 1: the 1D row / column scales go out in the packed form of alto_mxfp4_pack_scales (batch == 1)
+  int pack_rs, pack_cs;  // 1: the row / column scales go out in the packed form of alto_mxfp4_pack_scales, matrix after matrix
 };
 
 // byte position of K group g16 (0..15) inside the 16 bytes of a row and 512-K block of packed scales: 4 (2 h + ms) + j with
@@ -257,15 +257,17 @@ __global__ __launch_bounds__(256) void quant_kernel(const QuantParams p) {
     // descriptors of the row outputs start at the tile's first row
     const __amdgpu_buffer_rsrc_t rsrc_rc = __builtin_amdgcn_make_buffer_rsrc(
         DO_ROW ? p.row_codes + (b * M + row0) * p.ld_rc : nullptr, 0, DO_ROW ? 0x7FFFFFFF : 0, 0x00020000);
-    // Row scales, plain: [M][C/32], the byte of (row, group g) at row * (C/32) + g.  Packed (one matrix): the 16 groups of
+    // Row scales, plain: [M][C/32], the byte of (row, group g) at row * (C/32) + g.  Packed (per matrix): the 16 groups of
     // a row's 512-element block share 16 bytes, ((g / 16) M + row) 16 + packed_scale_pos(g % 16).  One store serves both:
     // the row pitch and the lane's column term are chosen here, outside the loop.
-    const bool prs = DO_ROW && !B2D && p.pack_rs;
+    // With 2D blocks the packed form repeats the block's scale for each of its 32 rows (the GEMM reads one layout).
+    const bool prs = DO_ROW && p.pack_rs;
+    const bool rs_rows = DO_ROW && (!B2D || prs);   // a scale byte per row goes out
     const int ldrs = prs ? 16 : C / 32;
     const int rs_col = prs ? ((c >> 9) * M) * 16 + packed_scale_pos((c >> 5) & 15) : (c >> 5);
     const __amdgpu_buffer_rsrc_t rsrc_rs = __builtin_amdgcn_make_buffer_rsrc(
-        (DO_ROW && !B2D) ? p.row_scales + (prs ? (int64_t)row0 * 16 : (b * M + row0) * (int64_t)(C / 32)) : nullptr, 0,
-        (DO_ROW && !B2D) ? 0x7FFFFFFF : 0, 0x00020000);
+        rs_rows ? p.row_scales + (prs ? (b * (int64_t)((C + 511) >> 9) * M + row0) * 16 : (b * M + row0) * (int64_t)(C / 32)) : nullptr, 0,
+        rs_rows ? 0x7FFFFFFF : 0, 0x00020000);
     const int ldrc = (int)p.ld_rc;
     if (prs && ((C >> 5) & 15) != 0 && col0 + TILE_C >= C) {   // packed: the groups of the last block beyond C read as 127
       const bool last = (tid & 3) == 0 && (c >> 5) == (C >> 5) - 1;
@@ -283,13 +285,11 @@ __global__ __launch_bounds__(256) void quant_kernel(const QuantParams p) {
       if (GEN && p.uos) s = e8m0_uos(BF ? u2f(a << 16) : u2f(a));
       else s = BF ? e8m0_from_bf16_bits(a) : e8m0_from_f32_bits(a);
       // scales
-      if (!B2D) {
-        if (DO_ROW) {
-          __builtin_amdgcn_raw_buffer_store_b8((uint8_t)s, rsrc_rs, (valid[i] && (tid & 3) == 0) ? rsub * ldrs + rs_col : OOB, 8 * i * ldrs, 0);
-        }
-      } else if (i == 0 && rsub == 0 && (tid & 3) == 0 && valid[0]) {
-        if (DO_ROW) p.row_scales[(b * (M / 32) + blockIdx.y) * (C / 32) + (c >> 5)] = (uint8_t)s;
-        if (DO_COL) p.col_scales[(b * (C / 32) + (c >> 5)) * (M / 32) + blockIdx.y] = (uint8_t)s;
+      if (!B2D || prs)   // (descriptor without range when no per-row byte is due)
+        __builtin_amdgcn_raw_buffer_store_b8((uint8_t)s, rsrc_rs, (valid[i] && (tid & 3) == 0) ? rsub * ldrs + rs_col : OOB, 8 * i * ldrs, 0);
+      if (B2D && i == 0 && rsub == 0 && (tid & 3) == 0 && valid[0]) {
+        if (DO_ROW && !prs) p.row_scales[(b * (M / 32) + blockIdx.y) * (C / 32) + (c >> 5)] = (uint8_t)s;
+        if (DO_COL && !p.pack_cs) p.col_scales[(b * (C / 32) + (c >> 5)) * (M / 32) + blockIdx.y] = (uint8_t)s;
       }
       if constexpr (ROW_CODES) {
       const float scale_f = u2f(s << 23);
@@ -397,14 +397,17 @@ __global__ __launch_bounds__(256) void quant_kernel(const QuantParams p) {
       for (int k = 0; k < 32; k += 2) am = __builtin_fmaxf(__builtin_fmaxf(am, __builtin_fabsf(z[k])), __builtin_fabsf(z[k + 1]));
       if (GEN && p.uos) s = e8m0_uos(am);
       else s = BF ? e8m0_from_bf16_bits(f2u(am) >> 16) : e8m0_from_f32_bits(f2u(am));
-      // plain: [C][M/32], this band's byte of column cc at cc (M/32) + band.  Packed (one matrix): ((band / 16) C + cc) 16 +
-      // packed_scale_pos(band % 16); the last band also writes the 127s of the groups beyond M.
+    }
+    // Column scales, plain 1D: [C][M/32], this band's byte of column cc at cc (M/32) + band (2D blocks: the row phase wrote
+    // the block's byte).  Packed (per matrix, 1D or 2D blocks): ((band / 16) C + cc) 16 + packed_scale_pos(band % 16); the
+    // last band also writes the 127s of the groups beyond M.
+    {
       const bool pcs = p.pack_cs;
       const int by = blockIdx.y, cs_pitch = pcs ? 16 : M / 32;
-      const uint8_t* cs_blk = p.col_scales + ((int64_t)(by >> 4) * C + col0) * 16;
+      const uint8_t* cs_blk = p.col_scales + ((b * (int64_t)((M + 511) >> 9) + (by >> 4)) * C + col0) * 16;
       const __amdgpu_buffer_rsrc_t rsrc_cs = __builtin_amdgcn_make_buffer_rsrc(
           const_cast<uint8_t*>(pcs ? cs_blk + packed_scale_pos(by & 15) : p.col_scales + (b * C + col0) * (int64_t)(M / 32) + by), 0, 0x7FFFFFFF, 0x00020000);
-      __builtin_amdgcn_raw_buffer_store_b8((uint8_t)s, rsrc_cs, cvalid ? tid * cs_pitch : OOB, 0, 0);
+      if (!B2D || pcs) __builtin_amdgcn_raw_buffer_store_b8((uint8_t)s, rsrc_cs, cvalid ? tid * cs_pitch : OOB, 0, 0);
       if (pcs && by == (M >> 5) - 1 && ((M >> 5) & 15) != 0) {
         const __amdgpu_buffer_rsrc_t rsrc_pad = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(cs_blk), 0, 0x7FFFFFFF, 0x00020000);
         for (int gp = (M >> 5) & 15; gp < 16; ++gp)
@@ -714,7 +717,7 @@ int quantize_impl(const void* x, int dtype, int64_t batch, int64_t M, int64_t C,
   ALTO_REQUIRE(clip_mode == ALTO_CLIP_NONE || clip_mode == ALTO_CLIP_STATIC || clip_mode == ALTO_CLIP_DYNAMIC, "quantize: bad clip_mode %d", clip_mode);
   const bool pack_rs = (flags & 1) != 0, pack_cs = (flags & 2) != 0;
   if (pack_rs || pack_cs) {
-    ALTO_REQUIRE(batch <= 1 && !is_2d && clip_mode != ALTO_CLIP_DYNAMIC, "quantize: packed scales are written for one matrix with 1D blocks (no dynamic clip)");
+    ALTO_REQUIRE(clip_mode != ALTO_CLIP_DYNAMIC, "quantize: packed scales are not written with the dynamic clip");
     ALTO_REQUIRE((!pack_rs || row_codes) && (!pack_cs || col_codes), "quantize: packed scales asked for an output that is not produced");
     ALTO_REQUIRE(M % 32 == 0 && M * C < (1ll << 36), "quantize: packed scales need M %% 32 == 0 and M * C < 2^36");
     ALTO_REQUIRE(((reinterpret_cast<uintptr_t>(pack_rs ? row_scales : nullptr) | reinterpret_cast<uintptr_t>(pack_cs ? col_scales : nullptr)) & 15) == 0,

@@ -6,7 +6,7 @@ from .grouped_gemm import (ALIGN_SIZE_M, MXFP4GroupedGEMM, _quantize_then_mxfp_s
                            mxfp4_grouped_gemm_backward_weights, mxfp4_grouped_gemm_forward)
 from .hadamard import HadamardFactory, HadamardTransform
 from .linear import (MXFP4LinearFunction, _to_mxfp4_then_scaled_mm, blockwise_mxfp4_gemm, clear_weight_cache, enable_weight_cache,
-                     transpose_codes, weight_cache_stats)
+                     transpose_codes, use_packed_scales, weight_cache_stats)
 from .ops import register_torch_ops
 from .qdq import _make_qdq_fn_for, quantize_dequantize
 from .quantization import BLOCK_SIZE_DEFAULT, convert_from_mxfp4, convert_to_mxfp4, hadamard_left, quantize_rowcol
@@ -41,6 +41,7 @@ __all__ = (
     "TrainingWeightWrapperBaseTensor",
     "swap_params",
     "enable_weight_cache",
+    "use_packed_scales",
     "clear_weight_cache",
     "weight_cache_stats",
     "quantize_dequantize",

@@ -19,7 +19,7 @@ import torch
 from . import _runtime as rt
 from .._lib import check
 from .hadamard import HadamardFactory, HadamardTransform
-from .linear import _wgrad_scale, cached_weight_quantisation, transpose_codes, unwrap_weight_wrapper
+from .linear import _wgrad_scale, cached_weight_quantisation, packed_scales_enabled, transpose_codes, unwrap_weight_wrapper
 from .quantization import convert_to_mxfp4, quantize_rowcol
 
 ALIGN_SIZE_M = 128
@@ -117,6 +117,16 @@ def grouped_forward_packed(a_q, a_ps, w_q, w_ps, groups: Groups, plan=None, retu
         ws.data_ptr(), ws.numel(), int(plan is not None), rt.stream_ptr(a_q.device))
     check(rc, "alto_mxfp4_grouped_gemm_ps")
     return (out, ws) if return_plan else out
+
+
+def grouped_packed_supported(M: int, N: int, K: int, num_groups: int, lda: Optional[int] = None, ldw: Optional[int] = None) -> bool:
+    """Shapes :func:`grouped_forward_packed` serves (the conditions of the grouped 256x256 tile kernel); ``lda`` / ``ldw`` are
+    the row pitches of the codes in bytes (default: K/2 rounded up to 16)."""
+    pitch = -(-(K // 2) // 16) * 16
+    lda = pitch if lda is None else lda
+    ldw = pitch if ldw is None else ldw
+    return (M >= 128 and N >= 128 and K >= 512 and N % 8 == 0 and M * lda < 2 ** 31 and N * ldw < 2 ** 31
+            and -(-(K // 32) // 16) * max(M, N) * 16 < 2 ** 31 and (-(-M // 256) + num_groups + 2) * -(-N // 256) < 2 ** 28)
 
 
 def grouped_plan(groups: Groups, num_experts: int, m_total: int) -> torch.Tensor:
@@ -239,18 +249,30 @@ class MXFP4GroupedGEMM(torch.autograd.Function):
             groups = groups_from_offsets(offsets)
         torch._check(M_buf % 32 == 0)
         x = inputs if inputs.is_contiguous() else inputs.contiguous()
-        if use_2dblock_x:   # one 2D-block quantisation, both packings: K-packed for the forward, token-packed for dW
-            a_q, a_s, a_qm, a_sm = quantize_rowcol(x, True, use_uos=use_uos, pad_codes=True)
-        else:               # row copy for the forward; Hadamard + clip on the token-axis copy saved for dW
-            a_q, a_s, a_qm, a_sm = quantize_rowcol(x, False, hadamard=hadamard_transform, clip_mode=clip_mode, use_uos=use_uos, pad_codes=True)
-        # weights: codes packed along K [E, N, K/2] for the forward, packed along N [E, K, N/2] for dX
         w = expert_weights if trans_weights else expert_weights.transpose(1, 2)   # logical [E, N, K]
+        N, K = w.shape[1], w.shape[2]
+        # Packed scales for the forward and dX where the grouped tile kernel serves the shape: the quantizers write that
+        # layout themselves.  (dW reads plain scales: its operands' scales are read once per tile, not per K step.)
+        can_pack = (packed_scales_enabled() and original_dtype == torch.bfloat16 and clip_mode != "dynamic"
+                    and M_buf * max(N, K) < 2 ** 36 and N * K < 2 ** 36)
+        pk_f = can_pack and grouped_packed_supported(M_buf, N, K, groups.n)
+        pk_d = can_pack and grouped_packed_supported(M_buf, K, N, groups.n)
+        if use_2dblock_x:   # one 2D-block quantisation, both packings: K-packed for the forward, token-packed for dW
+            a_q, a_s, a_qm, a_sm = quantize_rowcol(x, True, use_uos=use_uos, pad_codes=True, pack_row_scales=pk_f)
+        else:               # row copy for the forward; Hadamard + clip on the token-axis copy saved for dW
+            a_q, a_s, a_qm, a_sm = quantize_rowcol(x, False, hadamard=hadamard_transform, clip_mode=clip_mode, use_uos=use_uos, pad_codes=True,
+                                                   pack_row_scales=pk_f)
+        # weights: codes packed along K [E, N, K/2] for the forward, packed along N [E, K, N/2] for dX
         if w.stride(2) == 1:
-            wq_nk, ws_nk, wq_kn, ws_kn = _quantize_experts(weights_owner, w, use_2dblock_w, use_uos)
+            wq_nk, ws_nk, wq_kn, ws_kn = _quantize_experts(weights_owner, w, use_2dblock_w, use_uos, pk_f, pk_d)
         else:                                                                     # stored [E, K, N]: same pass, roles swapped
-            wq_kn, ws_kn, wq_nk, ws_nk = _quantize_experts(weights_owner, w.transpose(1, 2), use_2dblock_w, use_uos)
-        out, plan = grouped_forward(a_q, a_s, wq_nk, ws_nk, groups, use_2dblock_x, use_2dblock_w, original_dtype, return_plan=True)
+            wq_kn, ws_kn, wq_nk, ws_nk = _quantize_experts(weights_owner, w.transpose(1, 2), use_2dblock_w, use_uos, pk_d, pk_f)
+        if pk_f:
+            out, plan = grouped_forward_packed(a_q, a_s, wq_nk, ws_nk, groups, return_plan=True)
+        else:
+            out, plan = grouped_forward(a_q, a_s, wq_nk, ws_nk, groups, use_2dblock_x, use_2dblock_w, original_dtype, return_plan=True)
         ctx.save_for_backward(a_qm, a_sm, wq_kn, ws_kn, groups.offs, groups.expert, plan)   # (plan: the pass list, reused by dX)
+        ctx.packed_dx = pk_d
         ctx.num_groups = groups.n
         ctx.trans_weights = trans_weights
         ctx.original_dtype = original_dtype
@@ -272,27 +294,33 @@ class MXFP4GroupedGEMM(torch.autograd.Function):
         sr = bool(ctx.use_sr_grad)
         # random words: made inside the quantizer (Philox) unless a source of explicit words is installed
         rand = rt.draw_rand_bits(go.shape, go.device) if (sr and not rt.philox_in_kernel()) else None
+        pk_d = ctx.packed_dx
         if ctx.use_2dblock_x:
-            go_q, go_s, go_qm, go_sm = quantize_rowcol(go, True, use_sr=sr, rand_bits=rand, use_uos=ctx.use_uos, pad_codes=True)
+            go_q, go_s, go_qm, go_sm = quantize_rowcol(go, True, use_sr=sr, rand_bits=rand, use_uos=ctx.use_uos, pad_codes=True, pack_row_scales=pk_d)
         else:
             go_q, go_s, go_qm, go_sm = quantize_rowcol(go, False, use_sr=sr, rand_bits=rand, hadamard=ctx.hadamard_transform,
-                                                       clip_mode=ctx.clip_mode, use_uos=ctx.use_uos, pad_codes=True)
-        grad_inputs = grouped_forward(go_q, go_s, wq_kn, ws_kn, groups, ctx.use_2dblock_x, ctx.use_2dblock_w, ctx.original_dtype, plan=plan)
+                                                       clip_mode=ctx.clip_mode, use_uos=ctx.use_uos, pad_codes=True, pack_row_scales=pk_d)
+        if pk_d:
+            grad_inputs = grouped_forward_packed(go_q, go_s, wq_kn, ws_kn, groups, plan=plan)
+        else:
+            grad_inputs = grouped_forward(go_q, go_s, wq_kn, ws_kn, groups, ctx.use_2dblock_x, ctx.use_2dblock_w, ctx.original_dtype, plan=plan)
         grad_weights = grouped_dw(go_qm.transpose(0, 1), go_sm.transpose(0, 1), a_qm.transpose(0, 1), a_sm.transpose(0, 1),
                                   groups, ctx.num_experts, ctx.original_dtype, ctx.trans_weights,
                                   _wgrad_scale(ctx.clip_mode, ctx.use_dge), is_2d=ctx.use_2dblock_x)
         return (grad_inputs, grad_weights) + (None,) * 11
 
 
-def _quantize_experts(owner: torch.Tensor, w: torch.Tensor, is_2d: bool, use_uos: bool):
+def _quantize_experts(owner: torch.Tensor, w: torch.Tensor, is_2d: bool, use_uos: bool, pack_rows: bool = False, pack_cols: bool = False):
     """w [E, R, C] (unit stride along C; ``owner`` or a transposed view of it) -> codes packed along C [E,R,C/2] with
     their scales, and codes packed along R [E,C,R/2] with theirs (each operand of a GEMM wants unit stride along its
     reduction dim).  2D blocks: one quantisation, scales [E,R/32,C/32] and the same values stored transposed
     [E,C/32,R/32].  1D blocks: two quantisations (blocks along C: scales [E,R,C/32]; blocks along R: [E,C,R/32]), still one
-    pass over the weights.  The cache entry belongs to ``owner``, the tensor object the caller keeps."""
+    pass over the weights.  ``pack_rows`` / ``pack_cols``: the first / second scale tensor comes packed, [E, ceil(C/512), R, 16]
+    / [E, ceil(R/512), C, 16].  The cache entry belongs to ``owner``, the tensor object the caller keeps."""
     from .quantization import _prep, _quantize_call
-    return cached_weight_quantisation(owner, ("experts", bool(is_2d), bool(use_uos), tuple(w.shape), tuple(w.stride())),
-                                      lambda: _quantize_call(_prep(w), True, True, bool(is_2d), False, None, None, 0, use_uos, True))
+    return cached_weight_quantisation(owner, ("experts", bool(is_2d), bool(use_uos), tuple(w.shape), tuple(w.stride()), bool(pack_rows), bool(pack_cols)),
+                                      lambda: _quantize_call(_prep(w), True, True, bool(is_2d), False, None, None, 0, use_uos, True,
+                                                             pack_row_scales=pack_rows, pack_col_scales=pack_cols))
 
 
 def mxfp4_grouped_gemm(inputs, expert_weights, expert_indices, *, trans_weights=True, use_2dblock_x=False, use_2dblock_w=True,

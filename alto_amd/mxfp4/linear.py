@@ -5,6 +5,7 @@ Mirrors ``alto/kernels/fp4/mxfp4/mxfp_linear.py``: ``blockwise_mxfp4_gemm`` (:14
 """
 from __future__ import annotations
 
+import os
 import weakref
 from typing import Optional
 
@@ -76,13 +77,18 @@ def cached_weight_quantisation(weight: torch.Tensor, tag, make):
     return out
 
 
-def _quantize_weight_2d(weight: torch.Tensor, use_uos: bool, owner: Optional[torch.Tensor] = None):
+def _quantize_weight_2d(weight: torch.Tensor, use_uos: bool, owner: Optional[torch.Tensor] = None,
+                        pack_fprop: bool = False, pack_dgrad: bool = False):
     """(w_q, w_s, w_qt, w_st) of a 2D-block quantisation, from the cache when the weight is unchanged.  ``owner`` is the
     object the CALLER keeps alive (the ``nn.Parameter`` or wrapper tensor): ``weight`` itself may be a plain-tensor alias
     made for this call only (``unwrap_weight_wrapper`` of a Parameter is a new object every time), on which an entry
-    would never be found again.  The alias shares the owner's storage and version counter."""
-    return cached_weight_quantisation(weight if owner is None else owner, ("linear2d", bool(use_uos)),
-                                      lambda: quantize_rowcol(weight, True, use_uos=use_uos, pad_codes=True))
+    would never be found again.  The alias shares the owner's storage and version counter.
+
+    ``pack_fprop`` / ``pack_dgrad``: ``w_s`` / ``w_st`` come in the packed form of :func:`pack_scales` (rows N, reduction K
+    resp. rows K, reduction N), written by the quantizer."""
+    return cached_weight_quantisation(weight if owner is None else owner, ("linear2d", bool(use_uos), bool(pack_fprop), bool(pack_dgrad)),
+                                      lambda: quantize_rowcol(weight, True, use_uos=use_uos, pad_codes=True,
+                                                              pack_row_scales=pack_fprop, pack_col_scales=pack_dgrad))
 
 
 def transpose_codes(codes: torch.Tensor) -> torch.Tensor:
@@ -130,6 +136,27 @@ def pack_scales(scales: torch.Tensor, rows: int, K: int, is_2d_block: bool = Fal
 def packed_gemm_supported(M: int, N: int, K: int) -> bool:
     """Shapes the packed-scale kernel serves (the 256x256 tile kernel's conditions; anything else takes plain scales)."""
     return M >= 128 and N >= 128 and K >= 512 and N % 8 == 0 and M * (K // 2) < 2 ** 31 and N * (K // 2) < 2 ** 31
+
+
+_PACKED_SCALES = os.environ.get("ALTO_MXFP4_PACKED_SCALES", "1") != "0"   # the process-wide default; see use_packed_scales
+
+
+def use_packed_scales(enabled: bool = True) -> None:
+    """The linear and grouped autograd functions hand scales to their GEMMs in the packed form wherever the tile kernel
+    serves the shape (default), or always in the reference's plain form.  Results are the same bit for bit."""
+    global _PACKED_SCALES
+    _PACKED_SCALES = bool(enabled)
+
+
+def packed_scales_enabled() -> bool:
+    return _PACKED_SCALES
+
+
+def _k_major(codes: torch.Tensor) -> torch.Tensor:
+    """Codes [rows, K/2] with unit stride along K and 16-byte aligned rows (a copy only when the view is not)."""
+    if codes.stride(1) != 1 or codes.stride(0) % 16 != 0 or codes.data_ptr() % 16 != 0:
+        return codes.contiguous()
+    return codes
 
 
 def gemm_packed(a_q: torch.Tensor, a_ps: torch.Tensor, b_q: torch.Tensor, b_ps: torch.Tensor, out_scale: float = 1.0) -> torch.Tensor:
@@ -237,8 +264,17 @@ class MXFP4LinearFunction(torch.autograd.Function):
         M = x2.shape[0]
 
         fuse_x = (not use_2dblock_x) and M % 32 == 0
+        # Packed scales: each of the three GEMMs takes them when the tile kernel serves its shape; the quantizers then
+        # write that layout directly, so nothing is converted on the way.
+        N, K = weight.shape
+        can_pack = (_PACKED_SCALES and fuse_x and clip_mode != "dynamic" and original_dtype == torch.bfloat16
+                    and weight.dtype in (torch.bfloat16, torch.float32) and M * max(N, K) < 2 ** 36 and N * K < 2 ** 36)
+        pk_f = can_pack and packed_gemm_supported(M, N, K)   # fprop: y [M, N], reduction K
+        pk_d = can_pack and packed_gemm_supported(M, K, N)   # dgrad: dx [M, K], reduction N
+        pk_w = can_pack and packed_gemm_supported(N, K, M)   # wgrad: dw [N, K], reduction M
         if fuse_x:
-            x_q, x_s, x_qm, x_sm = quantize_rowcol(x2, False, hadamard=hadamard_transform, clip_mode=clip_mode, use_uos=use_uos, pad_codes=True)
+            x_q, x_s, x_qm, x_sm = quantize_rowcol(x2, False, hadamard=hadamard_transform, clip_mode=clip_mode, use_uos=use_uos, pad_codes=True,
+                                                   pack_row_scales=pk_f, pack_col_scales=pk_w)
         else:
             x_q, x_s = convert_to_mxfp4(x2, axis=-1, is_2d_block=use_2dblock_x, use_uos=use_uos)
             if use_2dblock_x:
@@ -247,17 +283,25 @@ class MXFP4LinearFunction(torch.autograd.Function):
                 x_qm, x_sm = convert_to_mxfp4(x2, axis=0, clip_mode=clip_mode, use_uos=use_uos, hadamard=hadamard_transform)
 
         if use_2dblock_w:
-            w_q, w_s, w_qt, w_st = _quantize_weight_2d(weight, use_uos, owner=weight_owner)
+            w_q, w_s, w_qt, w_st = _quantize_weight_2d(weight, use_uos, owner=weight_owner, pack_fprop=pk_f, pack_dgrad=pk_d)
             # [N/2, K] view over [K][N/2] memory; scales [N/32, K/32] as a view over [K/32][N/32] memory (same values as
-            # w_s, stored so that the dgrad GEMM reads them with unit stride along its reduction dim N)
+            # w_s, stored so that the dgrad GEMM reads them with unit stride along its reduction dim N), or packed
             w_bwd, w_bwd_s = w_qt, w_st
         else:
             w_q, w_s = convert_to_mxfp4(weight, axis=-1, is_2d_block=False, use_uos=use_uos)
             w_bwd, w_bwd_s = convert_to_mxfp4(weight, axis=0, is_2d_block=False, use_uos=use_uos)
+            if pk_f:
+                w_s = pack_scales(w_s, N, K)
+            if pk_d:
+                w_bwd_s = pack_scales(w_bwd_s.transpose(0, 1), K, N)
 
-        y = blockwise_mxfp4_gemm(x_q, x_s, w_q, w_s, use_2dblock_a=use_2dblock_x, use_2dblock_b=use_2dblock_w,
-                                 trans_b=True, output_dtype=original_dtype)
+        if pk_f:
+            y = gemm_packed(_k_major(x_q), x_s, _k_major(w_q), w_s)
+        else:
+            y = blockwise_mxfp4_gemm(x_q, x_s, w_q, w_s, use_2dblock_a=use_2dblock_x, use_2dblock_b=use_2dblock_w,
+                                     trans_b=True, output_dtype=original_dtype)
         ctx.save_for_backward(x_qm, x_sm, w_bwd, w_bwd_s)
+        ctx.packed = (pk_d, pk_w)
         ctx.use_2dblock_x = use_2dblock_x
         ctx.use_2dblock_w = use_2dblock_w
         ctx.original_dtype = original_dtype
@@ -273,6 +317,7 @@ class MXFP4LinearFunction(torch.autograd.Function):
         original_shape = grad_output.shape
         go = grad_output.reshape(-1, original_shape[-1])
         x_qm, x_sm, w_bwd, w_bwd_s = ctx.saved_tensors
+        pk_d, pk_w = ctx.packed
         sr = bool(ctx.use_sr_grad)
         # random words: made inside the quantizer (Philox) unless a source of explicit words is installed
         rand = rt.draw_rand_bits(go.shape, go.device) if (sr and not rt.philox_in_kernel()) else None
@@ -281,17 +326,25 @@ class MXFP4LinearFunction(torch.autograd.Function):
             go_qm, go_sm = go_q, go_s
         else:
             go_q, go_s, go_qm, go_sm = quantize_rowcol(go, False, use_sr=sr, rand_bits=rand, hadamard=ctx.hadamard_transform,
-                                                       clip_mode=ctx.clip_mode, use_uos=ctx.use_uos, pad_codes=True)
+                                                       clip_mode=ctx.clip_mode, use_uos=ctx.use_uos, pad_codes=True,
+                                                       pack_row_scales=pk_d, pack_col_scales=pk_w)
         # dgrad: reduction over N.  The saved weight operand is already packed along N (both layouts of a 2D-block
         # quantisation hold the same codes), so no k_pack=False repack is needed here.
-        grad_inputs = blockwise_mxfp4_gemm(go_q, go_s, w_bwd, w_bwd_s, use_2dblock_a=ctx.use_2dblock_x,
-                                           use_2dblock_b=ctx.use_2dblock_w, k_pack_b=True, output_dtype=ctx.original_dtype)
+        if pk_d:
+            grad_inputs = gemm_packed(_k_major(go_q), go_s, _k_major(w_bwd.transpose(0, 1)), w_bwd_s)
+        else:
+            grad_inputs = blockwise_mxfp4_gemm(go_q, go_s, w_bwd, w_bwd_s, use_2dblock_a=ctx.use_2dblock_x,
+                                               use_2dblock_b=ctx.use_2dblock_w, k_pack_b=True, output_dtype=ctx.original_dtype)
         # wgrad: reduction over tokens
-        grad_weights = blockwise_mxfp4_gemm(go_qm, go_sm, x_qm, x_sm, use_2dblock_a=ctx.use_2dblock_x,
-                                            use_2dblock_b=ctx.use_2dblock_x, trans_a=True,
-                                            k_pack_a=not ctx.use_2dblock_x, k_pack_b=not ctx.use_2dblock_x,
-                                            output_dtype=ctx.original_dtype,
-                                            out_scale=_wgrad_scale(ctx.clip_mode, ctx.use_dge))
+        if pk_w:
+            grad_weights = gemm_packed(_k_major(go_qm.transpose(0, 1)), go_sm, _k_major(x_qm.transpose(0, 1)), x_sm,
+                                       out_scale=_wgrad_scale(ctx.clip_mode, ctx.use_dge))
+        else:
+            grad_weights = blockwise_mxfp4_gemm(go_qm, go_sm, x_qm, x_sm, use_2dblock_a=ctx.use_2dblock_x,
+                                                use_2dblock_b=ctx.use_2dblock_x, trans_a=True,
+                                                k_pack_a=not ctx.use_2dblock_x, k_pack_b=not ctx.use_2dblock_x,
+                                                output_dtype=ctx.original_dtype,
+                                                out_scale=_wgrad_scale(ctx.clip_mode, ctx.use_dge))
         return grad_inputs.view(*original_shape[:-1], -1), grad_weights, None, None, None, None, None, None, None, None
 
 

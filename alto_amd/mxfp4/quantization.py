@@ -58,23 +58,22 @@ def _quantize_call(x3: torch.Tensor, want_row: bool, want_col: bool, is_2d: bool
     ``philox`` = an int64[2] device tensor {key, counter}: the same, with key and counter read on the device and the
     counter moved past the B M C words afterwards (nothing about the draw is a kernel argument: safe under graph capture).
     ``hw_sr``: round with the hardware's stochastic converts (``alto_mxfp4_quantize_sr_hw``; needs ``philox``).
-    ``pack_row_scales`` / ``pack_col_scales`` (one matrix, 1D blocks): that scale output comes in the packed form of
-    ``linear.pack_scales`` -- [1, ceil(C/512), M, 16] resp. [1, ceil(M/512), C, 16] -- written by the kernel itself."""
+    ``pack_row_scales`` / ``pack_col_scales``: that scale output comes in the packed form of ``linear.pack_scales`` --
+    [B, ceil(C/512), M, 16] resp. [B, ceil(M/512), C, 16] -- written by the kernel itself."""
     B, M, C = x3.shape
     dev = x3.device
     packed = pack_row_scales or pack_col_scales
-    assert not packed or (B == 1 and not is_2d), "packed scales: one matrix with 1D blocks"
     row_codes = row_scales = col_codes = col_scales = None
     if want_row:
         row_codes = _code_buffer(B, M, C // 2, dev, pad_codes)
         if pack_row_scales:
-            row_scales = torch.empty((1, -(-(C // 32) // 16), M, 16), dtype=torch.uint8, device=dev)
+            row_scales = torch.empty((B, -(-(C // 32) // 16), M, 16), dtype=torch.uint8, device=dev)
         else:
             row_scales = torch.empty((B, M // 32, C // 32) if is_2d else (B, M, C // 32), dtype=torch.uint8, device=dev)
     if want_col:
         col_codes = _code_buffer(B, C, M // 2, dev, pad_codes)
         if pack_col_scales:
-            col_scales = torch.empty((1, -(-(M // 32) // 16), C, 16), dtype=torch.uint8, device=dev)
+            col_scales = torch.empty((B, -(-(M // 32) // 16), C, 16), dtype=torch.uint8, device=dev)
         else:
             col_scales = torch.empty((B, C // 32, M // 32) if is_2d else (B, C, M // 32), dtype=torch.uint8, device=dev)
     had, sp, pp = _signs_perm_ptrs(hadamard)
@@ -323,7 +322,7 @@ def quantize_rowcol(
     clipping).  Fuses mxfp_linear.py:310-315 with :383-396 (forward, x) and
     :466-494 (backward, dY); for 2D blocks it yields both packings of a weight from one read.
 
-    ``pack_row_scales`` / ``pack_col_scales`` (1D blocks, no dynamic clip): that scale output is the packed tensor
+    ``pack_row_scales`` / ``pack_col_scales`` (no dynamic clip): that scale output is the packed tensor
     ``linear.pack_scales`` would make of it -- ``[ceil(C/512), M, 16]`` resp. ``[ceil(M/512), C, 16]`` -- written by the
     quantizer itself, for ``linear.gemm_packed`` / ``grouped_gemm.grouped_forward_packed``.
     """
@@ -346,8 +345,7 @@ def quantize_rowcol(
                 philox = rt.philox_seed_offset(None, None)
         else:
             rand_bits = rt.draw_rand_bits(x.shape, x.device)
-    torch._check(not (pack_row_scales or pack_col_scales) or (not is_2d_block and clip_mode != "dynamic"),
-                 lambda: "packed scales come with 1D blocks and without the dynamic clip")
+    torch._check(not (pack_row_scales or pack_col_scales) or clip_mode != "dynamic", lambda: "packed scales come without the dynamic clip")
     if clip_mode == "dynamic":   # the row pair is never clipped; the column pair takes the plain path
         rc, rs = convert_to_mxfp4(x, axis=-1, is_2d_block=is_2d_block, use_sr=use_sr, use_uos=use_uos, rand_bits=rand_bits)
         cc, cs = convert_to_mxfp4(x, axis=0, is_2d_block=is_2d_block, use_sr=use_sr, clip_mode="dynamic", use_uos=use_uos,

@@ -154,7 +154,8 @@ int64_t alto_mxfp4_quantize_sr_hw_words(int dtype, int64_t batch, int64_t M, int
  * (alto_mxfp4_quantize_pitched with use_sr = 0), 1 = stochastic with the words in rand_bits (the same call with use_sr =
  * 1), 2 = alto_mxfp4_quantize_sr_philox, 3 = alto_mxfp4_quantize_sr_hw; arguments a mode does not use are ignored.
  * Codes, and scales where no flag asks otherwise, are those calls' bit for bit.
- * flags (one matrix: batch <= 1; 1D blocks: is_2d = 0; clip_mode not dynamic; ALTO_MXFP4_EINVAL / ENOTIMPL otherwise):
+ * flags (clip_mode not dynamic; M % 32 == 0; M C < 2^36; ALTO_MXFP4_EINVAL otherwise; with is_2d a block's scale is
+ * repeated for its 32 rows, as alto_mxfp4_pack_scales does; with batch > 1 the packed matrices follow one another):
  *   ALTO_QUANT_PACK_ROW_SCALES (1): row_scales receives the packed layout of alto_mxfp4_pack_scales for rows = M, K = C
  *     (alto_mxfp4_packed_scales_bytes(M, C) bytes), pads included, instead of [M][C/32];
  *   ALTO_QUANT_PACK_COL_SCALES (2): col_scales likewise for rows = C, K = M.

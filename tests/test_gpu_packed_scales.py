@@ -140,9 +140,108 @@ def test_quantize_rowcol_packed_feeds_the_packed_gemm(m):
     assert torch.equal(gemm_packed(aq2, aps, bq2, bps), want)
 
 
+@pytest.mark.parametrize("M,C", [(512, 512), (96, 1056), (1056, 2880), (544, 32)])
+@pytest.mark.parametrize("mode", ["rne", "sr_hw"])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_quantizer_writes_packed_scales_of_2d_blocks(m, M, C, mode, dtype):
+    """2D blocks (the weight): both packings' scales, packed, repeat a block's scale for its 32 rows."""
+    from alto_amd.mxfp4.linear import pack_scales
+    from alto_amd.mxfp4.quantization import _prep, _quantize_call
+    x3 = _prep(randn_outliers((M, C), dtype, seed=M * 3 + C).to(DEV))
+    kw = dict(use_sr=mode != "rne", rand3=None, hadamard=None, clip=0, use_uos=False, philox=(9, 8) if mode == "sr_hw" else None, hw_sr=mode == "sr_hw")
+    rc, rs, cc, cs = _quantize_call(x3, True, True, True, **kw)
+    for pr, pc in [(True, True), (True, False), (False, True)]:
+        rc2, rs2, cc2, cs2 = _quantize_call(x3, True, True, True, pack_row_scales=pr, pack_col_scales=pc, **kw)
+        assert_bytes_equal(rc2.cpu(), rc.cpu(), "row codes")
+        assert_bytes_equal(cc2.cpu(), cc.cpu(), "column codes")
+        assert_bytes_equal(rs2[0].cpu(), (pack_scales(rs[0], M, C, True) if pr else rs[0]).cpu(), "row scales")
+        assert_bytes_equal(cs2[0].cpu(), (pack_scales(cs[0], C, M, True) if pc else cs[0]).cpu(), "column scales")
+    rc3, rs3, _, _ = _quantize_call(x3, True, False, True, pack_row_scales=True, **kw)
+    assert_bytes_equal(rc3.cpu(), rc.cpu(), "row codes alone")
+    assert_bytes_equal(rs3[0].cpu(), pack_scales(rs[0], M, C, True).cpu(), "row scales alone")
+    _, _, cc4, cs4 = _quantize_call(x3, False, True, True, pack_col_scales=True, **kw)
+    assert_bytes_equal(cc4.cpu(), cc.cpu(), "column codes alone")
+    assert_bytes_equal(cs4[0].cpu(), pack_scales(cs[0], C, M, True).cpu(), "column scales alone")
+
+
 def test_packed_flags_are_rejected_where_they_do_not_apply(m):
     x = torch.randn(64, 64, dtype=torch.bfloat16, device=DEV)
     with pytest.raises(RuntimeError, match="packed scales"):
-        m.quantize_rowcol(x, is_2d_block=True, pack_row_scales=True)
-    with pytest.raises(RuntimeError, match="packed scales"):
         m.quantize_rowcol(x, clip_mode="dynamic", pack_col_scales=True)
+
+
+def _count_calls(monkeypatch, module, name):
+    calls = []
+    real = getattr(module, name)
+
+    def spy(*a, **k):
+        calls.append(1)
+        return real(*a, **k)
+    monkeypatch.setattr(module, name, spy)
+    return calls
+
+
+@pytest.mark.parametrize("M,N,K,expect", [(512, 768, 1024, 3), (1056, 512, 2880, 3), (256, 160, 544, 1), (96, 256, 512, 0), (256, 64, 512, 0),
+                                          (128, 512, 160, 1), (512, 544, 512, 3)])
+@pytest.mark.parametrize("w2d", [True, False])
+@pytest.mark.parametrize("mode", ["rne", "sr", "sr_hw", "static_clip"])
+def test_linear_autograd_is_the_same_on_packed_scales(m, monkeypatch, M, N, K, expect, w2d, mode):
+    """y, dx and dw of the linear function with packed scales switched on equal those with the switch off, bit for bit, and
+    the packed GEMM serves exactly the GEMMs whose shape the tile kernel takes."""
+    from alto_amd.mxfp4 import linear as L
+    assert expect == sum(L.packed_gemm_supported(*s) for s in ((M, N, K), (M, K, N), (N, K, M)))
+    x = randn_outliers((M, K), torch.bfloat16, seed=5).to(DEV)
+    w = randn_outliers((N, K), torch.bfloat16, seed=6).to(DEV)
+    go = (randn_outliers((M, N), torch.bfloat16, seed=7) / (M * N)).to(DEV)
+    h = m.HadamardTransform(*hadamard_from_seed(11))
+    calls = _count_calls(monkeypatch, L, "gemm_packed")
+    res = []
+    m.use_hardware_stochastic_rounding(mode == "sr_hw")
+    try:
+        for on in (True, False):
+            L.use_packed_scales(on)
+            torch.manual_seed(99)   # the Philox key of the backward quantizer
+            xg, wg = x.clone().requires_grad_(True), w.clone().requires_grad_(True)
+            y = m.MXFP4LinearFunction.apply(xg, wg, False, w2d, mode.startswith("sr"), False, "static" if mode == "static_clip" else "none", False, h, False)
+            y.backward(go)
+            res.append((y.detach(), xg.grad, wg.grad))
+            if on:
+                assert len(calls) == expect
+    finally:
+        L.use_packed_scales(True)
+        m.use_hardware_stochastic_rounding(False)
+    assert len(calls) == expect
+    for got, want, what in zip(res[0], res[1], ("y", "dx", "dw")):
+        assert torch.equal(got, want), what
+
+
+@pytest.mark.parametrize("N,K", [(768, 1280), (512, 2880), (288, 512), (128, 96)])
+@pytest.mark.parametrize("x2d,w2d", [(False, True), (False, False), (True, True)])
+@pytest.mark.parametrize("trans_weights", [True, False])
+def test_grouped_autograd_is_the_same_on_packed_scales(m, monkeypatch, N, K, x2d, w2d, trans_weights):
+    from alto_amd.mxfp4 import grouped_gemm as G
+    from alto_amd.mxfp4 import linear as L
+    E, Mt = 4, 1024
+    a = randn_outliers((Mt, K), torch.bfloat16, seed=31).to(DEV)
+    wts = randn_outliers((E, N, K) if trans_weights else (E, K, N), torch.bfloat16, seed=32).to(DEV)
+    idx = torch.randint(0, E, (Mt // 128,), generator=torch.Generator().manual_seed(33), dtype=torch.int32).repeat_interleave(128).to(DEV)
+    go = (randn_outliers((Mt, N), torch.bfloat16, seed=34) / (Mt * N)).to(DEV)
+    calls = _count_calls(monkeypatch, G, "grouped_forward_packed")
+    expect = int(G.grouped_packed_supported(Mt, N, K, E)) + int(G.grouped_packed_supported(Mt, K, N, E))
+    res = []
+    try:
+        for on in (True, False):
+            L.use_packed_scales(on)
+            torch.manual_seed(99)
+            m.HadamardFactory.configure(seed=1234)
+            ag, wg = a.clone().requires_grad_(True), wts.clone().requires_grad_(True)
+            out = m.mxfp4_grouped_gemm(ag, wg, idx, trans_weights=trans_weights, use_2dblock_x=x2d, use_2dblock_w=w2d, use_sr_grad=True, use_hadamard=not x2d)
+            out.backward(go)
+            res.append((out.detach(), ag.grad, wg.grad))
+            if on:
+                assert len(calls) == expect
+    finally:
+        L.use_packed_scales(True)
+    assert len(calls) == expect
+    for got, want, what in zip(res[0], res[1], ("out", "dx", "dw")):
+        assert torch.equal(got, want), what
