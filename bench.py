@@ -504,6 +504,54 @@ class LinearStep(Workload):
         raise NotImplementedError("the end-to-end step is reported beside the per-kernel workloads, without its own CPU leg")
 
 
+class GroupedStep(Workload):
+    """Config 5 end to end: the grouped autograd function forward and backward at the GPT-OSS expert shape (1D activation
+    blocks, 2D weight blocks, Hadamard on the dW operands, stochastic rounding of dY, ragged offsets): per step the
+    quantizer passes over x, the 32 expert weights (unless cached) and dY, and the three grouped GEMMs."""
+    bound = "mfma"
+    kernel = "grouped_gemm"
+    E, N, K, T, TOPK = 32, 5760, 2880, 16384, 4
+
+    def __init__(self, cached, hw_sr=False):
+        self.cached = cached
+        self.hw_sr = hw_sr
+        self.name = f"cfg5_grouped_fwd_bwd[65536x2880->5760,E=32,{'cached' if cached else 'requantized'} weights{', hardware SR converts' if hw_sr else ''}]"
+        self.work = 3 * 2.0 * self.T * self.TOPK * self.K * self.N
+
+    def setup(self, dev, gen):
+        import torch
+        import alto_amd.mxfp4 as m
+        self.m = m
+        rows = self.T * self.TOPK
+        logits = torch.randn(self.T, self.E, device=dev, generator=gen)
+        skew = torch.log(1.0 / torch.arange(1, self.E + 1, device=dev).float() ** 1.1)
+        top = torch.topk(torch.softmax(logits + skew, dim=-1), self.TOPK, dim=-1).indices.reshape(-1)
+        counts = torch.bincount(top, minlength=self.E)
+        self.offs = torch.cat([torch.zeros(1, dtype=torch.int64, device=dev), counts.cumsum(0)]).to(torch.int32)
+        self.x = torch.randn(rows, self.K, device=dev, generator=gen).bfloat16().requires_grad_(True)
+        self.w = (torch.randn(self.E, self.N, self.K, device=dev, generator=gen) * 0.02).bfloat16().requires_grad_(True)
+        self.go = _laplace((rows, self.N), 1e-3, dev, gen)
+        m.HadamardFactory.configure(seed=1234)
+
+    def step(self):
+        m = self.m
+        m.enable_weight_cache(self.cached)
+        m.use_hardware_stochastic_rounding(self.hw_sr)
+        try:
+            self.x.grad = self.w.grad = None
+            y = m.mxfp4_grouped_gemm(self.x, self.w, None, use_2dblock_x=False, use_2dblock_w=True, use_sr_grad=True, use_hadamard=True,
+                                     offsets=self.offs)
+            y.backward(self.go)
+        finally:
+            m.use_hardware_stochastic_rounding(False)
+            if not self.cached:
+                m.enable_weight_cache(False)
+        return y
+
+    def cpu_sample(self):
+        raise NotImplementedError("the end-to-end step is reported beside the per-kernel workloads, without its own CPU leg")
+
+
 class CopyCalibration(Workload):
     """Plain device copy of 256 MiB (torch's elementwise copy kernel): the known-size launch against which the
     FETCH_SIZE / WRITE_SIZE counters of the other kernels are scaled.  Not part of the product path."""
@@ -592,6 +640,9 @@ def make_workloads():
         "linear_step_cached": LinearStep(True),
         "linear_step_hw_sr": LinearStep(False, hw_sr=True),
         "linear_step_cached_hw_sr": LinearStep(True, hw_sr=True),
+        "grouped_step": GroupedStep(False),
+        "grouped_step_hw_sr": GroupedStep(False, hw_sr=True),
+        "grouped_step_cached_hw_sr": GroupedStep(True, hw_sr=True),
         "copy_calib": CopyCalibration(),
         "mfma_probe_const": MfmaProbe(False),
         "mfma_probe_random": MfmaProbe(True),
