@@ -38,6 +38,7 @@ struct QuantParams {
   int clip_row;          // 1: multiply by 3/4 (in the input dtype) before encoding the row output
   int clip_col;
   int uos;
+  int unit_shift;        // column-output launches: log2 of the bands per unit of the workgroup mapping (3 .. 7)
   int pack_rs, pack_cs;  // 1: the row / column scales go out in the packed form of alto_mxfp4_pack_scales, matrix after matrix
 };
 
@@ -131,16 +132,18 @@ __global__ __launch_bounds__(256) void quant_kernel(const QuantParams p) {
   const int tid = threadIdx.x;
   const int M = p.M, C = p.C;
   // Workgroup -> (column tile bx, 32-row band by).  With a column output the grid is one-dimensional per matrix: consecutive
-  // workgroups go to the 8 XCDs in turn, so 64 consecutive ones are laid out as 8 XCDs (one unit = column tile x group of
-  // 8 bands each, neighbouring column tiles first) x the unit's 8 consecutive bands, and the eight 16-byte pieces that make
-  // up a 128-byte line of the column codes are written through one XCD's L2 within a short time of each other and leave it
-  // as a whole line (measured: 65536 x 5760 in 280 us instead of 403).  Without one: (column tiles, bands).
+  // workgroups go to the 8 XCDs in turn, so 8 x 2^unit_shift consecutive ones are laid out as 8 XCDs (one unit = column tile
+  // x group of 2^unit_shift bands each, neighbouring column tiles first) x the unit's consecutive bands.  The 16-byte pieces
+  // that make up a 128-byte line of the column codes (8 bands), and the bytes of a line of plain column scales (128 bands),
+  // are then written through one XCD's L2 within a short time of each other and leave it as whole lines (measured: 65536 x
+  // 5760 in 260-300 us instead of 403).  Without a column output: (column tiles, bands).
   const int nby = (M + 31) >> 5;
   int bx, by;
   if constexpr (DO_COL) {
-    const unsigned wg = blockIdx.x, unit = (wg >> 6) * 8 + (wg & 7), tiles_x = (unsigned)(C + TILE_C - 1) / TILE_C;
+    const unsigned wg = blockIdx.x, us = (unsigned)p.unit_shift;
+    const unsigned unit = (wg >> (3 + us)) * 8 + (wg & 7), tiles_x = (unsigned)(C + TILE_C - 1) / TILE_C;
     bx = (int)(unit % tiles_x);
-    by = (int)(unit / tiles_x) * 8 + (int)((wg >> 3) & 7);
+    by = (int)(((unit / tiles_x) << us) + ((wg >> 3) & ((1u << us) - 1)));
     if (by >= nby) return;   // (whole workgroup: padding of the last group of bands / of the units to a multiple of 8)
   } else {
     bx = (int)blockIdx.x;
@@ -776,10 +779,14 @@ int quantize_impl(const void* x, int dtype, int64_t batch, int64_t M, int64_t C,
   const bool gen = p.clip_row || p.clip_col || p.uos;
 
   const int64_t tiles_x = (C + TILE_C - 1) / TILE_C, bands = (M + 31) / 32;
-  const int64_t units = tiles_x * ((bands + 7) / 8);   // with a column output: 8 workgroups per unit, units padded to 8
-  ALTO_REQUIRE(do_col ? (units + 7) / 8 * 64 < (1ll << 31) : (tiles_x < (1ll << 31) && bands <= 65535),
-               "quantize: %lld x %lld exceeds the grid", (long long)M, (long long)C);
-  const dim3 grid = do_col ? dim3((unsigned)((units + 7) / 8 * 64), 1, (unsigned)batch) : dim3((unsigned)tiles_x, (unsigned)bands, (unsigned)batch);
+  // With a column output: 2^unit_shift workgroups per unit, units padded to a multiple of 8.  The largest unit (up to the
+  // 128 bands of a line of plain column scales) whose padding launches at most 5 % more workgroups than there are tiles.
+  int us = 7;
+  auto padded = [&](int sh) { return ((tiles_x * ((bands + (1ll << sh) - 1) >> sh) + 7) / 8 * 8) << sh; };
+  while (us > 3 && padded(us) * 20 > tiles_x * bands * 21) --us;
+  p.unit_shift = us;
+  ALTO_REQUIRE(do_col ? padded(us) < (1ll << 31) : (tiles_x < (1ll << 31) && bands <= 65535), "quantize: %lld x %lld exceeds the grid", (long long)M, (long long)C);
+  const dim3 grid = do_col ? dim3((unsigned)padded(us), 1, (unsigned)batch) : dim3((unsigned)tiles_x, (unsigned)bands, (unsigned)batch);
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   if (dtype == ALTO_DT_BF16) dispatch<__bf16>(p, grid, st, do_row, do_col, hadamard != 0, is_2d != 0, sr_mode, gen);
   else dispatch<float>(p, grid, st, do_row, do_col, hadamard != 0, is_2d != 0, sr_mode, gen);
