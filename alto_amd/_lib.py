@@ -72,6 +72,8 @@ SIGNATURES = {
                                            c_vp, c_i64, c_vp, c_i64, c_i64, c_int,
                                            c_vp, c_vp, c_int, c_int, c_i64, c_i64, c_i64,
                                            c_vp, c_int, c_i64, c_i64, c_i64, c_f32, c_vp]),
+    "alto_mxfp4_grouped_gemm_dw_ps": (c_int, [c_vp, c_i64, c_vp, c_vp, c_i64, c_vp, c_vp, c_vp, c_int, c_int, c_i64, c_i64, c_i64,
+                                              c_vp, c_i64, c_i64, c_i64, c_f32, c_vp]),
     "alto_mxfp4_probe_mfma": (c_int, [c_int, c_int, c_int, c_vp, c_vp, c_vp]),
     "alto_mxfp4_attention_fwd": (c_int, [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64,
                                          c_f32, c_int, c_vp]),

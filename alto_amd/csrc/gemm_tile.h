@@ -48,6 +48,8 @@ struct TileArgs {
   int k_lead = 0;              // the first k_lead (< 8) K groups of the reduction read as zero codes: a reduction over a
                                // sub-range of K starts at the 128-byte line that holds its first group, so that every
                                // operand load is one whole line, and the groups before the range drop out this way
+  int ps_q0 = 0;               // packed scales, reduction over a sub-range of K: the 512-K block of the packed layout that
+  int ps_sh = 0;               // holds the range's first stage, and 1 when that stage is the block's second half
 };
 
 // Every field of TileArgs is the same for all lanes.  When the struct arrives through memory (a real function call) the
@@ -79,6 +81,7 @@ __device__ __forceinline__ TileArgs uniform_args(const TileArgs& t) {
   o.as_bytes = uniform_i64(t.as_bytes); o.bs_bytes = uniform_i64(t.bs_bytes);
   o.s_k0 = __builtin_amdgcn_readfirstlane(t.s_k0); o.s_row = __builtin_amdgcn_readfirstlane(t.s_row);
   o.k_lead = __builtin_amdgcn_readfirstlane(t.k_lead);
+  o.ps_q0 = __builtin_amdgcn_readfirstlane(t.ps_q0); o.ps_sh = __builtin_amdgcn_readfirstlane(t.ps_sh);
   return o;
 }
 
@@ -252,9 +255,10 @@ struct TileLoader {
 // OperandView::ss_k the bytes from one block to the next (rows x 16).  A block of a tile's 256 + 256 rows is then 8 runs of
 // 1 KB, which the eight waves move straight into LDS with one load each (no registers, no fix-up, no ds_write; 8 cache
 // lines per load instead of the 64 of per-row scale rows).  Needs the end of K at compile time (LMS >= 0, or no K tail).
-template <bool KTAIL, int LMS = -1, int NST = 4, bool PS = false>
+template <bool KTAIL, int LMS = -1, int NST = 4, int PS = 0>
 __device__ __forceinline__ void gemm_tile_mainloop(const TileArgs& ta, TileAcc& acc, uint8_t* smem) {
-  static_assert(!PS || !KTAIL || LMS >= 0, "packed scales: the end of K must be known at compile time");
+  static_assert(PS != 1 || !KTAIL || LMS >= 0, "packed scales: the end of K must be known at compile time");
+  static_assert(PS != 2 || (KTAIL && LMS < 0), "packed scales of a sub-range of K: the generic endings only");
   constexpr int SP = PS ? 4 : GT_SCALE_PITCH;   // dwords per row of a scale buffer in LDS
   TileLoader ld;
   v4i_t sraw;   // scale bytes of a later block, as loaded
@@ -307,6 +311,26 @@ __device__ __forceinline__ void gemm_tile_mainloop(const TileArgs& ta, TileAcc& 
       fb[u] = v8i_t{(int)b4.x, (int)b4.y, (int)b4.z, (int)b4.w, 0, 0, 0, 0};
     }
   };
+  // PS == 2: the reduction starts at stage ps_sh (0 / 1) of packed block ps_q0, so block kn of this loop takes its first
+  // stage's bytes from packed block kn, dword 2 h + sh, and its second stage's from packed block kn + sh, dword 2 h + 1 - sh
+  // (packed block q sits in scale buffer q & 1).
+  const int sh = PS == 2 ? ta.ps_sh : 0;
+  auto read_scales2 = [&](int kn, int (&xa)[4][2], int (&xb)[2][2]) {
+    const uint32_t o0 = (uint32_t)((kn & 1) * (GT_TM + GT_TN) * SP * 4 + 4 * sh);
+    const uint32_t o1 = (uint32_t)(((kn + sh) & 1) * (GT_TM + GT_TN) * SP * 4 + 4 - 4 * sh);
+    const uint8_t* sb8 = reinterpret_cast<const uint8_t*>(sscale);
+    const uint8_t *a0 = sb8 + (sa_off + o0), *a1 = sb8 + (sa_off + o1), *b0 = sb8 + (sb_off + o0), *b1 = sb8 + (sb_off + o1);
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      xa[t][0] = *reinterpret_cast<const int*>(a0 + t * 32 * SP * 4);
+      xa[t][1] = *reinterpret_cast<const int*>(a1 + t * 32 * SP * 4);
+    }
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      xb[u][0] = *reinterpret_cast<const int*>(b0 + u * 32 * SP * 4);
+      xb[u][1] = *reinterpret_cast<const int*>(b1 + u * 32 * SP * 4);
+    }
+  };
   auto read_scales = [&](const uint8_t* sblock, int (&xa)[4][2], int (&xb)[2][2]) {
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
@@ -327,9 +351,10 @@ __device__ __forceinline__ void gemm_tile_mainloop(const TileArgs& ta, TileAcc& 
                                                                            (int)(ps_a ? ta.as_bytes : ta.bs_bytes), 0x00020000);
   const int ps_row0 = __builtin_amdgcn_readfirstlane((int)((ps_a ? ta.m0 + 64 * wave : ta.n0 + 64 * (wave - GT_TM / 64)) * 16));
   const int ps_blk = __builtin_amdgcn_readfirstlane((int)(ps_a ? ta.A.ss_k : ta.B.ss_k));
-  auto sdma = [&](int kb) {
+  const int ps_q0 = PS == 2 ? ta.ps_q0 : 0;
+  auto sdma = [&](int kb) {   // packed block ps_q0 + kb -> scale buffer kb & 1
     typedef __attribute__((address_space(3))) uint8_t lds_u8s;
-    const int so = __builtin_amdgcn_readfirstlane(kb * ps_blk + ps_row0);
+    const int so = __builtin_amdgcn_readfirstlane((kb + ps_q0) * ps_blk + ps_row0);
     __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_ps, (__attribute__((address_space(3))) void*)((lds_u8s*)sscale + (kb & 1) * (GT_TM + GT_TN) * SP * 4 + wave * 1024), 16,
                                              lane * 16, so, 0, 0);
   };
@@ -394,7 +419,7 @@ __device__ __forceinline__ void gemm_tile_mainloop(const TileArgs& ta, TileAcc& 
     __builtin_amdgcn_s_setprio(3);
     if constexpr (MS == 0 && !PEN) {
       if constexpr (PS) {
-        sdma(kb + 1);            // block kb+1 -> the other scale buffer; this block's second stage waits for it
+        sdma(kb + 1 + sh);       // block kb+1 (+1 with a half-block shift) -> the buffer whose bytes are all in registers; this block's second stage waits for it
       } else {
         swrite(kb + 1, fastc);   // block kb+1 -> the other scale buffer (last read at the end of block kb-1)
         ld.template sload<KTAIL>(kb + 2, sraw);
@@ -402,8 +427,10 @@ __device__ __forceinline__ void gemm_tile_mainloop(const TileArgs& ta, TileAcc& 
       __builtin_amdgcn_sched_barrier(0);
     }
     if constexpr (!PEN) ld.gload(smem, s + 2, MS, 0, 4);
-    if constexpr (MS == 1)   // the next block's scales (in LDS since this stage's barrier) ride along with the last step
-      read_scales(reinterpret_cast<const uint8_t*>(sscale + ((kb + 1) & 1) * (GT_TM + GT_TN) * SP), sa_next, sb_next);
+    if constexpr (MS == 1) {   // the next block's scales (in LDS since this stage's barrier) ride along with the last step
+      if constexpr (PS == 2) read_scales2(kb + 1, sa_next, sb_next);
+      else read_scales(reinterpret_cast<const uint8_t*>(sscale + ((kb + 1) & 1) * (GT_TM + GT_TN) * SP), sa_next, sb_next);
+    }
     mfma8(msc, std::integral_constant<int, 3>{}, fa1, fb1);
     read_frags(MS ^ 1, 0, fa0, fb0);
     if constexpr (PEN) interleave();
@@ -417,6 +444,7 @@ __device__ __forceinline__ void gemm_tile_mainloop(const TileArgs& ta, TileAcc& 
   ld.init(ta);
   if constexpr (PS) {
     sdma(0);
+    if constexpr (PS == 2) sdma(sh);   // with the shift, block 0 also needs packed block 1 (without: block 0 once more)
     ld.gload(smem, 0, 0, 0, 8);
     (void)sraw;
   } else {
@@ -428,7 +456,8 @@ __device__ __forceinline__ void gemm_tile_mainloop(const TileArgs& ta, TileAcc& 
   ld.gload(smem, 1, 1, 0, 4);   // the other half goes out in the first step of the loop
   asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)\n\ts_barrier" ::: "memory");   // all but stage 1's four loads
   read_frags(0, 0, fa0, fb0);
-  read_scales(reinterpret_cast<const uint8_t*>(sscale), sa, sb);
+  if constexpr (PS == 2) read_scales2(0, sa, sb);
+  else read_scales(reinterpret_cast<const uint8_t*>(sscale), sa, sb);
 
   // ---- main loop: one iteration = one 512-K block = 2 macro stages
   const int NS = (ta.G + 7) / 8;         // macro stages that hold any K at all
@@ -567,7 +596,7 @@ __device__ __forceinline__ void gemm_tile_store(const TileArgs& ta, TileAcc& acc
 }
 
 // LMS / NST: how the reduction ends, as in gemm_tile_mainloop.
-template <typename OutT, bool KTAIL, int LMS = -1, int NST = 4, bool PS = false>
+template <typename OutT, bool KTAIL, int LMS = -1, int NST = 4, int PS = 0>
 __device__ __forceinline__ void gemm_tile_256x256(const TileArgs& ta, OutT* __restrict__ c, int64_t ldc, uint8_t* smem) {
   TileAcc acc;
   gemm_tile_zero(acc);

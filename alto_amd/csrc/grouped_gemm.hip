@@ -332,7 +332,9 @@ constexpr int GT_DW_LDS_BYTES = GT_LDS_BYTES + 2 * (GT_DW_MAX_GROUPS / 64) * 8; 
 // memory operation in here, the global->LDS loads of the K loop included, as not aliasing the output, and only with that
 // mark does the compiler's wait insertion keep those loads in flight across the LDS reads that follow them (unmarked, it
 // puts an `s_waitcnt vmcnt(0)` before the next fragment read, twice per stage, and the loop runs at the load latency).
-template <typename OutT>
+// PS: the operands' scales are in the packed form of alto_mxfp4_pack_scales along the tokens ([M_total / 512 blocks][rows][16],
+// P.ss_k / Q.ss_k = bytes per block); a run starts at a 256-token line, i.e. at the first or the second half of a block.
+template <typename OutT, bool PS>
 __device__ __forceinline__ void grouped_dw_tile(const OperandView& P, const OperandView& Q, int64_t NP, int64_t NQ,
                                                 const int32_t* offs, const int32_t* group_expert, int num_groups,
                                                 int64_t M_total, OutT* __restrict__ dw, int64_t s_e, int64_t ld, float out_scale,
@@ -355,7 +357,8 @@ __device__ __forceinline__ void grouped_dw_tile(const OperandView& P, const Oper
   TileAcc acc;
   gemm_tile_zero(acc);
   const int64_t p_bytes = (NP - 1) * P.ld + M_total / 2, q_bytes = (NQ - 1) * Q.ld + M_total / 2;
-  const int64_t ps_bytes = ((P.is_2d ? NP / 32 : NP) - 1) * P.ss_r + M_total / 32, qs_bytes = ((Q.is_2d ? NQ / 32 : NQ) - 1) * Q.ss_r + M_total / 32;
+  const int64_t ps_bytes = PS ? ((M_total + 511) / 512) * P.ss_k : ((P.is_2d ? NP / 32 : NP) - 1) * P.ss_r + M_total / 32;
+  const int64_t qs_bytes = PS ? ((M_total + 511) / 512) * Q.ss_k : ((Q.is_2d ? NQ / 32 : NQ) - 1) * Q.ss_r + M_total / 32;
   // Boundaries of this expert's token runs; one that is not a multiple of 32 would share an MX block along the token dim
   // with another expert: the tile is then poisoned with NaN instead of being silently wrong.
   int bad = 0;
@@ -430,8 +433,9 @@ __device__ __forceinline__ void grouped_dw_tile(const OperandView& P, const Oper
     Pv.codes += ta0 / 2;
     Qv.codes += ta0 / 2;
     TileArgs ta{Pv, Qv, (int64_t)tm * GT_TM, (int64_t)tn * GT_TN, 0, NP, NQ, (int)((t1 - ta0) / 32), out_scale,
-                p_bytes - ta0 / 2, q_bytes - ta0 / 2, ps_bytes, qs_bytes, (int)(ta0 / 32), (int)(M_total / 32), (int)((t0 - ta0) / 32)};
-    gemm_tile_mainloop<true, -2>(ta, acc, smem);
+                p_bytes - ta0 / 2, q_bytes - ta0 / 2, ps_bytes, qs_bytes, (int)(ta0 / 32), (int)(M_total / 32), (int)((t0 - ta0) / 32),
+                (int)(ta0 >> 9), (int)(ta0 >> 8) & 1};
+    gemm_tile_mainloop<true, -2, 4, PS ? 2 : 0>(ta, acc, smem);
   }
   if (bad) {
 #pragma unroll
@@ -445,13 +449,13 @@ __device__ __forceinline__ void grouped_dw_tile(const OperandView& P, const Oper
   gemm_tile_store<OutT>(ta, acc, dw + e * s_e, ld, smem);
 }
 
-template <typename OutT>
+template <typename OutT, bool PS = false>
 __global__ __launch_bounds__(GT_THREADS) void grouped_dw_tiled_kernel(OperandView P, OperandView Q, int64_t NP, int64_t NQ,
                                                                       const int32_t* offs, const int32_t* group_expert, int num_groups,
                                                                       int64_t M_total, OutT* dw, int64_t s_e, int64_t ld, float out_scale,
                                                                       int tiles_p, int tiles_q, int xq_log2) {
   extern __shared__ __align__(16) uint8_t smem[];
-  grouped_dw_tile<OutT>(P, Q, NP, NQ, offs, group_expert, num_groups, M_total, dw, s_e, ld, out_scale, tiles_p, tiles_q, xq_log2, smem);
+  grouped_dw_tile<OutT, PS>(P, Q, NP, NQ, offs, group_expert, num_groups, M_total, dw, s_e, ld, out_scale, tiles_p, tiles_q, xq_log2, smem);
 }
 
 // upper bound on the number of passes: every band is one, every group start inside a band adds one, plus the unrouted head and tail
@@ -478,10 +482,10 @@ int launch_grouped_tiled(const OperandView& A, const uint8_t* w, int64_t w_strid
   return 0;
 }
 
-template <typename OutT>
+template <typename OutT, bool PS = false>
 int launch_dw_tiled(const OperandView& P, const OperandView& Q, int64_t NP, int64_t NQ, const int32_t* offs, const int32_t* group_expert,
                     int num_groups, int num_experts, int64_t M_total, void* dw, int64_t s_e, int64_t ld, float out_scale, hipStream_t st) {
-  auto kern = grouped_dw_tiled_kernel<OutT>;
+  auto kern = grouped_dw_tiled_kernel<OutT, PS>;
   static std::once_flag once;
   static hipError_t attr_rc = hipSuccess;
   std::call_once(once, [&] { attr_rc = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, GT_DW_LDS_BYTES); });
@@ -718,12 +722,14 @@ extern "C" int alto_mxfp4_grouped_gemm_noalloc(const uint8_t* a, int64_t lda, co
                            num_groups, num_experts, M_total, N, K, out, out_dtype, ldo, plan, ALTO_NOALLOC_SCRATCH_BYTES, "the built-in scratch array", true, stream);
 }
 
-extern "C" int alto_mxfp4_grouped_gemm_dw(const uint8_t* go, int64_t ld_go, const uint8_t* go_scales, int64_t gs_r, int64_t gs_k, int go_is_2d,
-                                          const uint8_t* x, int64_t ld_xq, const uint8_t* x_scales, int64_t xs_r, int64_t xs_k, int x_is_2d,
-                                          const int32_t* offs, const int32_t* group_expert, int num_groups, int num_experts,
-                                          int64_t M_total, int64_t N, int64_t K, void* dw, int dw_dtype, int64_t dw_stride_e, int64_t dw_stride_n, int64_t dw_stride_k,
-                                          float out_scale, void* stream) {
-  using namespace alto;
+namespace alto {
+namespace {
+// ps: go_scales / x_scales are packed along the tokens ([ceil(M_total / 512)][N or K][16]); tile kernel and bf16 only
+int grouped_dw_impl(const uint8_t* go, int64_t ld_go, const uint8_t* go_scales, int64_t gs_r, int64_t gs_k, int go_is_2d,
+                    const uint8_t* x, int64_t ld_xq, const uint8_t* x_scales, int64_t xs_r, int64_t xs_k, int x_is_2d,
+                    const int32_t* offs, const int32_t* group_expert, int num_groups, int num_experts,
+                    int64_t M_total, int64_t N, int64_t K, void* dw, int dw_dtype, int64_t dw_stride_e, int64_t dw_stride_n, int64_t dw_stride_k,
+                    float out_scale, void* stream, bool ps) {
   ALTO_REQUIRE(go && go_scales && x && x_scales && offs && dw, "grouped_gemm_dw: NULL pointer");
   ALTO_REQUIRE(num_experts > 0 && num_experts <= 65535, "grouped_gemm_dw: num_experts (%d) out of range", num_experts);
   ALTO_REQUIRE(num_groups > 0 && num_groups <= 65536, "grouped_gemm_dw: num_groups (%d) out of range", num_groups);
@@ -746,12 +752,17 @@ extern "C" int alto_mxfp4_grouped_gemm_dw(const uint8_t* go, int64_t ld_go, cons
     const int64_t NP = n_major ? N : K, NQ = n_major ? K : N;
     const int64_t ld = n_major ? dw_stride_n : dw_stride_k;
     const bool unit = n_major || dw_stride_n == 1;
-    const bool tiled = unit && M_total >= 512 && N >= 128 && K >= 128 && gs_k == 1 && xs_k == 1 && NQ % 8 == 0 && ld % 8 == 0 && dw_stride_e % 8 == 0 &&
+    const bool tiled = unit && M_total >= 512 && N >= 128 && K >= 128 && (ps || (gs_k == 1 && xs_k == 1)) && NQ % 8 == 0 && ld % 8 == 0 && dw_stride_e % 8 == 0 &&
                        (reinterpret_cast<uintptr_t>(dw) & 15) == 0 && N * ld_go < (1ll << 31) && K * ld_xq < (1ll << 31) &&
                        N * gs_r < (1ll << 31) && K * xs_r < (1ll << 31) && num_groups <= GT_DW_MAX_GROUPS && num_experts <= 65535 &&
                        ((NP + GT_TM - 1) / GT_TM) * ((NQ + GT_TN - 1) / GT_TN) < (1ll << 28);
+    if (ps && !(tiled && dw_dtype == ALTO_DT_BF16)) {
+      set_error("grouped_gemm_dw_ps: shape (%lld tokens, %lld, %lld) is not served by the tile kernel; use plain scales", (long long)M_total, (long long)N, (long long)K);
+      return ALTO_MXFP4_ENOTIMPL;
+    }
     if (tiled) {
-      const int rc = dw_dtype == ALTO_DT_BF16
+      const int rc = ps ? launch_dw_tiled<__bf16, true>(P, Q, NP, NQ, offs, group_expert, num_groups, num_experts, M_total, dw, dw_stride_e, ld, out_scale, st)
+                     : dw_dtype == ALTO_DT_BF16
                          ? launch_dw_tiled<__bf16>(P, Q, NP, NQ, offs, group_expert, num_groups, num_experts, M_total, dw, dw_stride_e, ld, out_scale, st)
                          : launch_dw_tiled<float>(P, Q, NP, NQ, offs, group_expert, num_groups, num_experts, M_total, dw, dw_stride_e, ld, out_scale, st);
       if (rc != 0) {
@@ -768,4 +779,27 @@ extern "C" int alto_mxfp4_grouped_gemm_dw(const uint8_t* go, int64_t ld_go, cons
   else
     hipLaunchKernelGGL(grouped_dw_simple_kernel<float>, grid, dim3(256), 0, st, GO, X, offs, group_expert, num_groups, M_total, N, K, (float*)dw, dw_stride_e, dw_stride_n, dw_stride_k, out_scale);
   return check_launch("grouped_gemm_dw");
+}
+}  // namespace
+}  // namespace alto
+
+extern "C" int alto_mxfp4_grouped_gemm_dw(const uint8_t* go, int64_t ld_go, const uint8_t* go_scales, int64_t gs_r, int64_t gs_k, int go_is_2d,
+                                          const uint8_t* x, int64_t ld_xq, const uint8_t* x_scales, int64_t xs_r, int64_t xs_k, int x_is_2d,
+                                          const int32_t* offs, const int32_t* group_expert, int num_groups, int num_experts,
+                                          int64_t M_total, int64_t N, int64_t K, void* dw, int dw_dtype, int64_t dw_stride_e, int64_t dw_stride_n, int64_t dw_stride_k,
+                                          float out_scale, void* stream) {
+  return alto::grouped_dw_impl(go, ld_go, go_scales, gs_r, gs_k, go_is_2d, x, ld_xq, x_scales, xs_r, xs_k, x_is_2d, offs, group_expert, num_groups, num_experts,
+                               M_total, N, K, dw, dw_dtype, dw_stride_e, dw_stride_n, dw_stride_k, out_scale, stream, false);
+}
+
+extern "C" int alto_mxfp4_grouped_gemm_dw_ps(const uint8_t* go, int64_t ld_go, const uint8_t* go_packed, const uint8_t* x, int64_t ld_xq, const uint8_t* x_packed,
+                                             const int32_t* offs, const int32_t* group_expert, int num_groups, int num_experts,
+                                             int64_t M_total, int64_t N, int64_t K, void* dw, int64_t dw_stride_e, int64_t dw_stride_n, int64_t dw_stride_k,
+                                             float out_scale, void* stream) {
+  using namespace alto;
+  ALTO_REQUIRE(((reinterpret_cast<uintptr_t>(go_packed) | reinterpret_cast<uintptr_t>(x_packed)) & 15) == 0, "grouped_gemm_dw_ps: packed scales must be 16-byte aligned");
+  ALTO_REQUIRE(M_total >= 0 && ((M_total + 511) / 512) * (N > K ? N : K) * 16 < (1ll << 31), "grouped_gemm_dw_ps: packed scales beyond 2 GiB");
+  // go: [blocks][N][16], x: [blocks][K][16]; ss_k carries the bytes from block to block
+  return grouped_dw_impl(go, ld_go, go_packed, 16, N * 16, 0, x, ld_xq, x_packed, 16, K * 16, 0, offs, group_expert, num_groups, num_experts,
+                         M_total, N, K, dw, ALTO_DT_BF16, dw_stride_e, dw_stride_n, dw_stride_k, out_scale, stream, true);
 }

@@ -201,6 +201,37 @@ def grouped_dw(go_qm, go_sm, x_qm, x_sm, groups: Groups, num_experts, output_dty
     return dw
 
 
+def grouped_dw_packed_supported(M_total: int, N: int, K: int, num_groups: int, num_experts: int) -> bool:
+    """Shapes :func:`grouped_dw_packed` serves (the conditions of the 256x256 dW tile kernel, dW stored [E, N, K] or [E, K, N]
+    contiguous, code rows of M_total / 2 bytes rounded up to 16)."""
+    pitch = -(-(M_total // 2) // 16) * 16
+    return (M_total >= 512 and M_total % 32 == 0 and N >= 128 and K >= 128 and N % 8 == 0 and K % 8 == 0 and N * pitch < 2 ** 31 and K * pitch < 2 ** 31
+            and num_groups <= 32768 and num_experts <= 65535 and -(-M_total // 512) * max(N, K) * 16 < 2 ** 31)
+
+
+def grouped_dw_packed(go_qm, go_ps, x_qm, x_ps, groups: Groups, num_experts, trans_weights=True, out_scale=1.0):
+    """:func:`grouped_dw` on scales packed along the tokens (bf16 dW): ``go_ps`` [ceil(M/512), N, 16], ``x_ps`` [ceil(M/512), K, 16]
+    -- the column scales ``quantize_rowcol(..., pack_col_scales=True)`` writes."""
+    N, K = go_qm.shape[0], x_qm.shape[0]
+    M_total = go_qm.shape[1] * 2
+    assert x_qm.shape[1] * 2 == M_total
+    if go_qm.stride(1) != 1 or go_qm.stride(0) % 16:
+        go_qm = go_qm.contiguous()
+    if x_qm.stride(1) != 1 or x_qm.stride(0) % 16:
+        x_qm = x_qm.contiguous()
+    KB = -(-M_total // 512)
+    assert go_ps.shape == (KB, N, 16) and x_ps.shape == (KB, K, 16) and go_ps.is_contiguous() and x_ps.is_contiguous()
+    shape = (num_experts, N, K) if trans_weights else (num_experts, K, N)
+    dw = torch.empty(shape, dtype=torch.bfloat16, device=go_qm.device)
+    s_e, s_n, s_k = (dw.stride(0), dw.stride(1), dw.stride(2)) if trans_weights else (dw.stride(0), dw.stride(2), dw.stride(1))
+    rc = rt.lib().alto_mxfp4_grouped_gemm_dw_ps(
+        go_qm.data_ptr(), go_qm.stride(0), go_ps.data_ptr(), x_qm.data_ptr(), x_qm.stride(0), x_ps.data_ptr(),
+        groups.offs.data_ptr(), rt.ptr(groups.expert), groups.n, num_experts, M_total, N, K, dw.data_ptr(), s_e, s_n, s_k,
+        float(out_scale), rt.stream_ptr(go_qm.device))
+    check(rc, "alto_mxfp4_grouped_gemm_dw_ps")
+    return dw
+
+
 def _token_packed(codes: torch.Tensor, k_pack: bool) -> torch.Tensor:
     """An operand of the weight gradient as [features, M/2] codes with unit stride along the tokens: a transposed view
     when it arrives packed along the tokens ([M/2, features], ``k_pack``), a nibble transpose when it arrives packed along
@@ -251,17 +282,18 @@ class MXFP4GroupedGEMM(torch.autograd.Function):
         x = inputs if inputs.is_contiguous() else inputs.contiguous()
         w = expert_weights if trans_weights else expert_weights.transpose(1, 2)   # logical [E, N, K]
         N, K = w.shape[1], w.shape[2]
-        # Packed scales for the forward and dX where the grouped tile kernel serves the shape: the quantizers write that
-        # layout themselves.  (dW reads plain scales: its operands' scales are read once per tile, not per K step.)
+        # Packed scales for the three grouped GEMMs where their tile kernels serve the shape: the quantizers write that
+        # layout themselves.
         can_pack = (packed_scales_enabled() and original_dtype == torch.bfloat16 and clip_mode != "dynamic"
                     and M_buf * max(N, K) < 2 ** 36 and N * K < 2 ** 36)
         pk_f = can_pack and grouped_packed_supported(M_buf, N, K, groups.n)
         pk_d = can_pack and grouped_packed_supported(M_buf, K, N, groups.n)
+        pk_w = can_pack and grouped_dw_packed_supported(M_buf, N, K, groups.n, E)
         if use_2dblock_x:   # one 2D-block quantisation, both packings: K-packed for the forward, token-packed for dW
-            a_q, a_s, a_qm, a_sm = quantize_rowcol(x, True, use_uos=use_uos, pad_codes=True, pack_row_scales=pk_f)
+            a_q, a_s, a_qm, a_sm = quantize_rowcol(x, True, use_uos=use_uos, pad_codes=True, pack_row_scales=pk_f, pack_col_scales=pk_w)
         else:               # row copy for the forward; Hadamard + clip on the token-axis copy saved for dW
             a_q, a_s, a_qm, a_sm = quantize_rowcol(x, False, hadamard=hadamard_transform, clip_mode=clip_mode, use_uos=use_uos, pad_codes=True,
-                                                   pack_row_scales=pk_f)
+                                                   pack_row_scales=pk_f, pack_col_scales=pk_w)
         # weights: codes packed along K [E, N, K/2] for the forward, packed along N [E, K, N/2] for dX
         if w.stride(2) == 1:
             wq_nk, ws_nk, wq_kn, ws_kn = _quantize_experts(weights_owner, w, use_2dblock_w, use_uos, pk_f, pk_d)
@@ -273,6 +305,7 @@ class MXFP4GroupedGEMM(torch.autograd.Function):
             out, plan = grouped_forward(a_q, a_s, wq_nk, ws_nk, groups, use_2dblock_x, use_2dblock_w, original_dtype, return_plan=True)
         ctx.save_for_backward(a_qm, a_sm, wq_kn, ws_kn, groups.offs, groups.expert, plan)   # (plan: the pass list, reused by dX)
         ctx.packed_dx = pk_d
+        ctx.packed_dw = pk_w
         ctx.num_groups = groups.n
         ctx.trans_weights = trans_weights
         ctx.original_dtype = original_dtype
@@ -294,19 +327,24 @@ class MXFP4GroupedGEMM(torch.autograd.Function):
         sr = bool(ctx.use_sr_grad)
         # random words: made inside the quantizer (Philox) unless a source of explicit words is installed
         rand = rt.draw_rand_bits(go.shape, go.device) if (sr and not rt.philox_in_kernel()) else None
-        pk_d = ctx.packed_dx
+        pk_d, pk_w = ctx.packed_dx, ctx.packed_dw
         if ctx.use_2dblock_x:
-            go_q, go_s, go_qm, go_sm = quantize_rowcol(go, True, use_sr=sr, rand_bits=rand, use_uos=ctx.use_uos, pad_codes=True, pack_row_scales=pk_d)
+            go_q, go_s, go_qm, go_sm = quantize_rowcol(go, True, use_sr=sr, rand_bits=rand, use_uos=ctx.use_uos, pad_codes=True, pack_row_scales=pk_d,
+                                                       pack_col_scales=pk_w)
         else:
             go_q, go_s, go_qm, go_sm = quantize_rowcol(go, False, use_sr=sr, rand_bits=rand, hadamard=ctx.hadamard_transform,
-                                                       clip_mode=ctx.clip_mode, use_uos=ctx.use_uos, pad_codes=True, pack_row_scales=pk_d)
+                                                       clip_mode=ctx.clip_mode, use_uos=ctx.use_uos, pad_codes=True, pack_row_scales=pk_d, pack_col_scales=pk_w)
         if pk_d:
             grad_inputs = grouped_forward_packed(go_q, go_s, wq_kn, ws_kn, groups, plan=plan)
         else:
             grad_inputs = grouped_forward(go_q, go_s, wq_kn, ws_kn, groups, ctx.use_2dblock_x, ctx.use_2dblock_w, ctx.original_dtype, plan=plan)
-        grad_weights = grouped_dw(go_qm.transpose(0, 1), go_sm.transpose(0, 1), a_qm.transpose(0, 1), a_sm.transpose(0, 1),
-                                  groups, ctx.num_experts, ctx.original_dtype, ctx.trans_weights,
-                                  _wgrad_scale(ctx.clip_mode, ctx.use_dge), is_2d=ctx.use_2dblock_x)
+        if pk_w:
+            grad_weights = grouped_dw_packed(go_qm.transpose(0, 1), go_sm, a_qm.transpose(0, 1), a_sm, groups, ctx.num_experts, ctx.trans_weights,
+                                             _wgrad_scale(ctx.clip_mode, ctx.use_dge))
+        else:
+            grad_weights = grouped_dw(go_qm.transpose(0, 1), go_sm.transpose(0, 1), a_qm.transpose(0, 1), a_sm.transpose(0, 1),
+                                      groups, ctx.num_experts, ctx.original_dtype, ctx.trans_weights,
+                                      _wgrad_scale(ctx.clip_mode, ctx.use_dge), is_2d=ctx.use_2dblock_x)
         return (grad_inputs, grad_weights) + (None,) * 11
 
 

@@ -428,6 +428,20 @@ class GroupedGemmDw(GroupedGemm):
         raise NotImplementedError("reported beside the forward workload, which carries the CPU leg")
 
 
+class GroupedGemmDwPacked(GroupedGemmDw):
+    """Config 5 weight gradient on operands whose scales are packed along the tokens (written that way by the quantizer)."""
+    name = "cfg5_grouped_dw_packed_scales[32x5760x2880 over 65536 tokens]"
+
+    def setup(self, dev, gen):
+        super().setup(dev, gen)
+        from alto_amd.mxfp4.linear import pack_scales
+        self.gps = pack_scales(self.gs, self.N, self.rows)
+        self.xps = pack_scales(self.xs, self.K, self.rows)
+
+    def step(self):
+        return self.G.grouped_dw_packed(self.gq, self.gps, self.xq, self.xps, self.groups, self.E)
+
+
 class AttentionFwd(Workload):
     """MXFP4 flash-attention forward on pre-quantised Q, K, V: the largest case of the reference's own test list
     (tests/unittest/mxfp4/test_mxfp_attention.py:64: batch 4, 2048 tokens, 64 query / 8 KV heads, head dim 128, causal)."""
@@ -635,6 +649,7 @@ def make_workloads():
         "cfg5_grouped_packed": GroupedGemmPacked(),
         "cfg5_grouped_dx_packed": GroupedGemmDxPacked(),
         "cfg5_grouped_dw": GroupedGemmDw(),
+        "cfg5_grouped_dw_packed": GroupedGemmDwPacked(),
         "attn_fwd": AttentionFwd(),
         "linear_step": LinearStep(False),
         "linear_step_cached": LinearStep(True),

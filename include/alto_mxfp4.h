@@ -365,6 +365,20 @@ int alto_mxfp4_grouped_gemm_dw(const uint8_t* go, int64_t ld_go, const uint8_t* 
                                float out_scale, void* stream);
 
 /*
+ * alto_mxfp4_grouped_gemm_dw on operands whose scales are packed along the tokens (alto_mxfp4_pack_scales with rows = N
+ * resp. K and the M_total tokens as the reduction: go_packed [ceil(M_total / 512)][N][16], x_packed [...][K][16] -- what
+ * alto_mxfp4_quantize_ex writes as column scales with ALTO_QUANT_PACK_COL_SCALES), bf16 dW.  Same results bit for bit.
+ * A run of tokens may start anywhere the plain call allows: the kernel starts at the 256-token line that holds the run's
+ * first token, i.e. at the first or second half of a packed block, and reads its scale bytes from there.  Serves the shapes
+ * of the tile kernel only (M_total >= 512, N, K >= 128, unit stride along the output's last dim, ...):
+ * ALTO_MXFP4_ENOTIMPL otherwise, and the caller keeps plain scales for those.
+ */
+int alto_mxfp4_grouped_gemm_dw_ps(const uint8_t* go, int64_t ld_go, const uint8_t* go_packed, const uint8_t* x, int64_t ld_xq, const uint8_t* x_packed,
+                                  const int32_t* offs, const int32_t* group_expert, int num_groups, int num_experts,
+                                  int64_t M_total, int64_t N, int64_t K, void* dw, int64_t dw_stride_e, int64_t dw_stride_n, int64_t dw_stride_k,
+                                  float out_scale, void* stream);
+
+/*
  * Fused quantize -> dequantize: y = convert_from_mxfp4(convert_to_mxfp4(x, axis=-1, is_2d_block), output_dtype = dtype
  * of x), round to nearest even, no clipping, in one pass (no codes or scales are written).  Replaces the pair of
  * launches in the weight de-oscillation hook (alto/components/optimizer.py:123-158, which calls

@@ -227,7 +227,9 @@ def test_grouped_autograd_is_the_same_on_packed_scales(m, monkeypatch, N, K, x2d
     idx = torch.randint(0, E, (Mt // 128,), generator=torch.Generator().manual_seed(33), dtype=torch.int32).repeat_interleave(128).to(DEV)
     go = (randn_outliers((Mt, N), torch.bfloat16, seed=34) / (Mt * N)).to(DEV)
     calls = _count_calls(monkeypatch, G, "grouped_forward_packed")
+    dw_calls = _count_calls(monkeypatch, G, "grouped_dw_packed")
     expect = int(G.grouped_packed_supported(Mt, N, K, E)) + int(G.grouped_packed_supported(Mt, K, N, E))
+    expect_dw = int(G.grouped_dw_packed_supported(Mt, N, K, G.groups_from_indices(idx).n, E))
     res = []
     try:
         for on in (True, False):
@@ -239,9 +241,59 @@ def test_grouped_autograd_is_the_same_on_packed_scales(m, monkeypatch, N, K, x2d
             out.backward(go)
             res.append((out.detach(), ag.grad, wg.grad))
             if on:
-                assert len(calls) == expect
+                assert len(calls) == expect and len(dw_calls) == expect_dw
     finally:
         L.use_packed_scales(True)
-    assert len(calls) == expect
+    assert len(calls) == expect and len(dw_calls) == expect_dw
     for got, want, what in zip(res[0], res[1], ("out", "dx", "dw")):
         assert torch.equal(got, want), what
+
+
+@pytest.mark.parametrize("N,K", [(256, 384), (512, 2880), (288, 160)])
+@pytest.mark.parametrize("layout", ["sorted", "per_group", "ragged32"])
+@pytest.mark.parametrize("trans_weights,is_2d", [(True, False), (False, False), (True, True)])
+def test_grouped_dw_with_packed_scales_equals_the_plain_call(m, N, K, layout, trans_weights, is_2d):
+    """Token-packed scales ([M/512][rows][16]): runs that start in the first and in the second half of a packed block, at
+    128- and 32-token boundaries, empty experts, runs of one expert in several places; NaN poisoning of a split MX block
+    included (same bits as the plain call everywhere)."""
+    from alto_amd.mxfp4 import grouped_gemm as G
+    from alto_amd.mxfp4.linear import pack_scales
+    E = 6
+    if layout == "sorted":      # 128-token boundaries, some in the second half of a 512 block, one empty expert
+        offs = torch.tensor([0, 384, 384, 1280, 1408, 2304, 2560], dtype=torch.int32)
+        groups = G.groups_from_offsets(offs.to(DEV))
+    elif layout == "per_group":  # the reference's contract: one expert id per 128 rows, unsorted
+        idx = torch.randint(0, E, (2560 // 128,), generator=torch.Generator().manual_seed(5), dtype=torch.int32).repeat_interleave(128)
+        groups = G.groups_from_indices(idx.to(DEV))
+    else:                        # boundaries at multiples of 32 only, one of them splitting a block (poisoned)
+        offs = torch.tensor([0, 96, 800, 832, 1999, 2528, 2560], dtype=torch.int32)
+        groups = G.groups_from_offsets(offs.to(DEV))
+    Mt = 2560
+    go = (randn_outliers((Mt, N), torch.bfloat16, seed=3) / 64).to(DEV)
+    x = randn_outliers((Mt, K), torch.bfloat16, seed=4).to(DEV)
+    h = None if is_2d else m.HadamardTransform(*hadamard_from_seed(8))
+    _, _, gqm, gsm = m.quantize_rowcol(go, is_2d, hadamard=h, pad_codes=True)
+    _, _, xqm, xsm = m.quantize_rowcol(x, is_2d, hadamard=h, pad_codes=True)
+    _, _, gqm2, gps = m.quantize_rowcol(go, is_2d, hadamard=h, pad_codes=True, pack_col_scales=True)
+    _, _, xqm2, xps = m.quantize_rowcol(x, is_2d, hadamard=h, pad_codes=True, pack_col_scales=True)
+    assert_bytes_equal(gps.cpu(), pack_scales(gsm.transpose(0, 1), N, Mt, is_2d).cpu(), "dY scales packed along the tokens")
+    assert G.grouped_dw_packed_supported(Mt, N, K, groups.n, E)
+    want = G.grouped_dw(gqm.transpose(0, 1), gsm.transpose(0, 1), xqm.transpose(0, 1), xsm.transpose(0, 1), groups, E, torch.bfloat16, trans_weights, 16.0 / 9.0,
+                        is_2d=is_2d)
+    got = G.grouped_dw_packed(gqm2.transpose(0, 1), gps, xqm2.transpose(0, 1), xps, groups, E, trans_weights, 16.0 / 9.0)
+    assert got.shape == want.shape
+    assert torch.equal(torch.isnan(got), torch.isnan(want))
+    if layout == "ragged32":
+        assert bool(torch.isnan(want[3]).all()) and bool(torch.isnan(want[4]).all())
+    assert torch.equal(torch.nan_to_num(got), torch.nan_to_num(want))
+
+
+def test_packed_dw_rejects_what_the_tile_kernel_does_not_serve(m):
+    from alto_amd.mxfp4 import grouped_gemm as G
+    Mt, N, K, E = 256, 64, 64, 2
+    assert not G.grouped_dw_packed_supported(Mt, N, K, E, E)
+    z = torch.zeros(Mt, N, dtype=torch.bfloat16, device=DEV)
+    _, _, q, ps = m.quantize_rowcol(z, False, pad_codes=True, pack_col_scales=True)
+    groups = G.groups_from_offsets(torch.tensor([0, 128, 256], dtype=torch.int32, device=DEV))
+    with pytest.raises(NotImplementedError, match="not served by the tile kernel"):
+        G.grouped_dw_packed(q.transpose(0, 1), ps, q.transpose(0, 1), ps, groups, E)
