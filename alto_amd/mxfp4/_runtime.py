@@ -1,6 +1,7 @@
 """Small helpers shared by the host wrappers: device checks, pointers, stream, random bits."""
 from __future__ import annotations
 
+import os
 from typing import Callable, Optional
 
 import torch
@@ -52,20 +53,28 @@ def set_rand_bits_source(fn: Optional[Callable[[torch.Size, torch.device], torch
     _rand_source = fn
 
 
-# The reference picks the gfx950 hardware converts whenever ``use_asm`` is left at None (mxfp_quantization.py:426-427).
-# Here None means the exact software rule unless this switch is on; ``use_asm=True`` / ``False`` always win.
-_hw_rounding_default = False
+# The reference picks the gfx950 hardware converts whenever ``use_asm`` is left at None (mxfp_quantization.py:426-427:
+# USE_ASM = is_cdna4()); this library runs on gfx950 only, so None means the hardware converts here as well.  The switch
+# below moves that default to the exact software rule of triton_fp4_ops.py:49-61 (what the reference runs on other parts
+# and what its PyTorch twin restates); ``use_asm=True`` / ``False`` on a call always win, and so do explicit ``rand_bits``
+# (words per element, which only the software rule consumes).
+_hw_rounding_default = os.environ.get("ALTO_MXFP4_HW_SR", "1") != "0"
 
 
 def use_hardware_stochastic_rounding(on: bool = True) -> None:
-    """Make stochastic rounding with ``use_asm=None`` (what the autograd functions pass) use the hardware converts
-    (``v_cvt_scalef32_sr_pk_fp4_*``, one random dword per pair of elements) instead of the software rule."""
+    """Stochastic rounding with ``use_asm=None`` (what the autograd functions pass): the hardware converts
+    (``v_cvt_scalef32_sr_pk_fp4_*``, one random dword per pair of elements; the default, as in the reference on gfx950) or,
+    with ``on=False``, the software rule."""
     global _hw_rounding_default
     _hw_rounding_default = bool(on)
 
 
 def hardware_stochastic_rounding(use_asm: Optional[bool] = None) -> bool:
-    return _hw_rounding_default if use_asm is None else bool(use_asm)
+    """What a call with this ``use_asm`` rounds with.  None: the session default -- unless a source of explicit words is
+    installed (``set_rand_bits_source``): only the software rule consumes those."""
+    if use_asm is None:
+        return _hw_rounding_default and _rand_source is None
+    return bool(use_asm)
 
 
 def philox_in_kernel() -> bool:

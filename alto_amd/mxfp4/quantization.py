@@ -188,8 +188,9 @@ def convert_to_mxfp4(
     results equal the software rule bit for bit): ``True`` rounds with ``v_cvt_scalef32_sr_pk_fp4_{bf16,f32}``, one random
     dword per pair of neighbouring elements, cut from the Philox stream ``(philox_seed, philox_offset)`` inside the kernel
     (mxfp_quantization.py:133-182; ``rand_bits`` cannot be given, ``clip_mode="dynamic"`` is not offered); ``False`` runs
-    the software rule of triton_fp4_ops.py:49-61 with 32 random bits per element; ``None`` (the reference: hardware on
-    gfx950) follows ``use_hardware_stochastic_rounding()``, off by default.
+    the software rule of triton_fp4_ops.py:49-61 with 32 random bits per element; ``None`` means the hardware converts, as in the
+    reference on gfx950 (``USE_ASM = is_cdna4()``, mxfp_quantization.py:426-427), unless ``rand_bits`` are given, the clip is
+    dynamic, or ``use_hardware_stochastic_rounding(False)`` / ``ALTO_MXFP4_HW_SR=0`` moved the default to the software rule.
     ``use_sr`` (software rule) consumes ``rand_bits`` (int32/uint32, same shape as ``data_hp``; element ``[i, j]`` uses
     ``rand_bits[i, j]``); when omitted they come from the library's Philox4x32-10 fill kernel (key and
     counter start ``philox_seed``/``philox_offset`` if given, else a draw from torch's CPU generator).  ``hadamard`` fuses ``hadamard(x, left_mul=True)`` in front of

@@ -486,13 +486,14 @@ class LinearStep(Workload):
     def __init__(self, cached, hw_sr=False):
         self.cached = cached
         self.hw_sr = hw_sr
-        self.name = f"cfg3+4_linear_fwd_bwd[8192x4096->14336,{'cached' if cached else 'requantized'} weight{', hardware SR converts' if hw_sr else ''}]"
+        self.name = f"cfg3+4_linear_fwd_bwd[8192x4096->14336,{'cached' if cached else 'requantized'} weight, {'hardware SR converts (the library default)' if hw_sr else 'software SR rule'}]"
         self.work = 3 * 2.0 * self.M * self.K * self.N
 
     def setup(self, dev, gen):
         import torch
         import alto_amd.mxfp4 as m
-        self.m = m
+        from alto_amd.mxfp4 import _runtime
+        self.m, self.rt = m, _runtime
         self.x = torch.randn(self.M, self.K, device=dev, generator=gen).bfloat16().requires_grad_(True)
         self.w = (torch.randn(self.N, self.K, device=dev, generator=gen) * 0.02).bfloat16().requires_grad_(True)
         self.go = _laplace((self.M, self.N), 1e-3, dev, gen)
@@ -503,13 +504,14 @@ class LinearStep(Workload):
     def step(self):
         m = self.m
         m.enable_weight_cache(self.cached)
+        before = self.rt.hardware_stochastic_rounding()
         m.use_hardware_stochastic_rounding(self.hw_sr)
         try:   # the random words of the stochastic rounding are drawn inside the step (Philox fill kernel), as in training
             self.x.grad = self.w.grad = None
             y = m.MXFP4LinearFunction.apply(self.x, self.w, False, True, True, False, "none", False, self.h, False)
             y.backward(self.go)
         finally:
-            m.use_hardware_stochastic_rounding(False)
+            m.use_hardware_stochastic_rounding(before)
             if not self.cached:
                 m.enable_weight_cache(False)
         return y
@@ -529,13 +531,14 @@ class GroupedStep(Workload):
     def __init__(self, cached, hw_sr=False):
         self.cached = cached
         self.hw_sr = hw_sr
-        self.name = f"cfg5_grouped_fwd_bwd[65536x2880->5760,E=32,{'cached' if cached else 'requantized'} weights{', hardware SR converts' if hw_sr else ''}]"
+        self.name = f"cfg5_grouped_fwd_bwd[65536x2880->5760,E=32,{'cached' if cached else 'requantized'} weights, {'hardware SR converts (the library default)' if hw_sr else 'software SR rule'}]"
         self.work = 3 * 2.0 * self.T * self.TOPK * self.K * self.N
 
     def setup(self, dev, gen):
         import torch
         import alto_amd.mxfp4 as m
-        self.m = m
+        from alto_amd.mxfp4 import _runtime
+        self.m, self.rt = m, _runtime
         rows = self.T * self.TOPK
         logits = torch.randn(self.T, self.E, device=dev, generator=gen)
         skew = torch.log(1.0 / torch.arange(1, self.E + 1, device=dev).float() ** 1.1)
@@ -550,6 +553,7 @@ class GroupedStep(Workload):
     def step(self):
         m = self.m
         m.enable_weight_cache(self.cached)
+        before = self.rt.hardware_stochastic_rounding()
         m.use_hardware_stochastic_rounding(self.hw_sr)
         try:
             self.x.grad = self.w.grad = None
@@ -557,7 +561,7 @@ class GroupedStep(Workload):
                                      offsets=self.offs)
             y.backward(self.go)
         finally:
-            m.use_hardware_stochastic_rounding(False)
+            m.use_hardware_stochastic_rounding(before)
             if not self.cached:
                 m.enable_weight_cache(False)
         return y

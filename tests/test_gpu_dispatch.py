@@ -247,7 +247,7 @@ def test_forward_replays_from_a_hip_graph(m):
         (x.float() @ w.float().T).sum().item()   # unrelated eager work and a host sync between replays
 
 
-def test_captured_stochastic_rounding_draws_fresh_words_on_every_replay(m):
+def test_captured_stochastic_rounding_draws_fresh_words_on_every_replay(m, software_sr):
     """With the device-resident Philox state nothing about the random words is a kernel argument: a captured SR
     quantizer (fused row + column copies with the Hadamard transform) draws new words on every replay, and every replay
     equals the eager call keyed with the (key, counter) the state held before it."""

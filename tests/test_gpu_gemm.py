@@ -166,7 +166,7 @@ def test_linear_autograd(m, shape, use_2dblock_x, use_2dblock_w, use_sr, use_h, 
     _linear_autograd_case(m, shape, use_2dblock_x, use_2dblock_w, use_sr, use_h, clip_mode, dtype, use_uos, floors=not use_uos)
 
 
-def test_autograd_with_words_made_in_the_kernel(m):
+def test_autograd_with_words_made_in_the_kernel(m, software_sr):
     """The default backward path: no source of explicit words installed, the quantizer of dY draws its words itself from
     the device-resident Philox stream.  The words are rebuilt from (key, counter) and the gradients compared with the
     oracle's flow on those words -- once for the linear function, once for the grouped one."""

@@ -147,7 +147,7 @@ def test_session_default_routes_the_autograd_function(m):
             y = m.MXFP4LinearFunction.apply(x, w, False, True, True, False, "none", False, h, False)
             gx, gw = torch.autograd.grad(y, (x, w), go)
         finally:
-            m.use_hardware_stochastic_rounding(False)
+            m.use_hardware_stochastic_rounding(True)
         outs[hw] = (gx.float(), gw.float())
     ref_gx = go.float() @ w.float().detach()
     ref_gw = go.float().t() @ x.float().detach()
@@ -155,3 +155,24 @@ def test_session_default_routes_the_autograd_function(m):
         gx, gw = outs[hw]
         assert float((gx - ref_gx).norm() / ref_gx.norm()) < 0.25 and float((gw - ref_gw).norm() / ref_gw.norm()) < 0.25
     assert not torch.equal(outs[False][0], outs[True][0])
+
+
+def test_use_asm_left_at_none_means_the_hardware_converts(m):
+    """The reference's default on gfx950 (USE_ASM = is_cdna4(), mxfp_quantization.py:426-427): a call that leaves ``use_asm``
+    at None rounds with the hardware converts; explicit words, or the switch, select the software rule."""
+    from alto_amd.mxfp4 import _runtime as rt
+    assert rt.hardware_stochastic_rounding() is True
+    x = laplace((128, 256), 1e-3, torch.bfloat16, seed=9).to(DEV)
+    dflt = m.convert_to_mxfp4(x, use_sr=True, philox_seed=3, philox_offset=8)
+    hw = m.convert_to_mxfp4(x, use_sr=True, use_asm=True, philox_seed=3, philox_offset=8)
+    sw = m.convert_to_mxfp4(x, use_sr=True, use_asm=False, philox_seed=3, philox_offset=8)
+    assert torch.equal(dflt[0], hw[0]) and torch.equal(dflt[1], hw[1]) and not torch.equal(dflt[0], sw[0])
+    words = rt.draw_rand_bits(x.shape, x.device, 3, 8)
+    given = m.convert_to_mxfp4(x, use_sr=True, rand_bits=words)          # explicit words: only the software rule reads them
+    assert torch.equal(given[0], sw[0])
+    m.use_hardware_stochastic_rounding(False)
+    try:
+        off = m.convert_to_mxfp4(x, use_sr=True, philox_seed=3, philox_offset=8)
+    finally:
+        m.use_hardware_stochastic_rounding(True)
+    assert torch.equal(off[0], sw[0])

@@ -209,7 +209,7 @@ def test_linear_autograd_is_the_same_on_packed_scales(m, monkeypatch, M, N, K, e
                 assert len(calls) == expect
     finally:
         L.use_packed_scales(True)
-        m.use_hardware_stochastic_rounding(False)
+        m.use_hardware_stochastic_rounding(True)
     assert len(calls) == expect
     for got, want, what in zip(res[0], res[1], ("y", "dx", "dw")):
         assert torch.equal(got, want), what

@@ -322,7 +322,7 @@ def test_random_bits_kernel_is_philox4x32_10(m, n, seed, offset):
     assert np.all(got[n:] == 0x55555555)
 
 
-def test_default_random_bits_follow_the_torch_seed(m):
+def test_default_random_bits_follow_the_torch_seed(m, software_sr):
     """Without supplied bits, stochastic rounding draws from the Philox kernel keyed by torch's CPU generator."""
     x = laplace((64, 96), 1e-3, torch.bfloat16, seed=3).to(DEV)
     torch.manual_seed(123)
@@ -344,7 +344,7 @@ def test_default_random_bits_follow_the_torch_seed(m):
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("shape", [(256, 512), (3, 64, 96), (8192, 4096)])
-def test_in_kernel_philox_equals_supplied_words(m, dtype, shape):
+def test_in_kernel_philox_equals_supplied_words(m, dtype, shape, software_sr):
     """Stochastic rounding with the random words made inside the kernel (Philox4x32-10, counter = element index / 4) gives
     the bytes of the supplied-words path when the tensor is filled by alto_mxfp4_random_bits with the same key and
     counter start -- which the oracle checks in turn: row copy, Hadamard column copy, 2D blocks, column copy alone."""
