@@ -48,25 +48,39 @@ __device__ __forceinline__ float pair_max(float v) {   // max over the two lanes
 
 // NK = D / 64 (MFMA K steps of Q K^T), ND = Dv / 32 (output tiles).
 // The four waves of a workgroup own 128 consecutive query rows of one head and walk the key blocks together: a block's
-// K codes (64 rows x D/2 bytes) and V codes (Dv rows x 32 bytes) are fetched once per workgroup with coalesced 16-byte
-// loads one block ahead, parked in registers during the softmax and written to the other half of a two-slot LDS ring;
+// K codes (64 rows x D/2 bytes) and V codes (Dv rows x 32 bytes) are fetched once per workgroup, two blocks ahead, with
+// direct-to-LDS loads (16 bytes per lane, 1 KB per wave instruction, no registers in between) into a three-slot ring;
 // one barrier per block.  (Fetching the pieces per wave straight from global memory made the vector-memory path the
-// bound: 8 KB per wave and block in scattered 16-byte accesses.)
+// bound: 8 KB per wave and block in scattered 16-byte accesses.  One block ahead through registers left the waves
+// waiting for the load at the end of every block: the kernel ran at 38 % VALU issue with the matrix pipes at 11 %.)
+constexpr int ATTN_RING = 3;
 template <int NK, int ND>
-__global__ __launch_bounds__(256, ATTN_WG_PER_CU) void attn_fwd_kernel(AttnArgs a) {
+struct AttnTile {
+  static constexpr int D = NK * 64, DV = ND * 32;
+  static constexpr int K_BYTES = 64 * (D / 2), V_BYTES = DV * 32;       // one block of K codes, of V codes
+  static constexpr int SLOT = K_BYTES + V_BYTES;
+};
+
+// The body of the kernel as a function of its own because of the `__restrict__` on the outputs: inlining then marks the
+// direct-to-LDS loads as not aliasing them, and only with that mark does the compiler's wait insertion keep those loads
+// in flight across the LDS reads that follow (unmarked, it puts an `s_waitcnt vmcnt(0)` before the next LDS read).
+template <int NK, int ND>
+__device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, __bf16* __restrict__ out, float* __restrict__ lse_out, uint8_t* ring) {
   constexpr int D = NK * 64, DV = ND * 32;
-  constexpr int K_BYTES = 64 * (D / 2), V_BYTES = DV * 32;       // one block of K codes, of V codes
+  constexpr int K_BYTES = AttnTile<NK, ND>::K_BYTES, V_BYTES = AttnTile<NK, ND>::V_BYTES, SLOT = AttnTile<NK, ND>::SLOT;
   constexpr int K_PIECES = K_BYTES / 16, V_PIECES = V_BYTES / 16;
-  constexpr int K_PER_THREAD = (K_PIECES + 255) / 256, V_PER_THREAD = (V_PIECES + 255) / 256;
-  __shared__ __attribute__((aligned(16))) uint8_t ring[2][K_BYTES + V_BYTES];
+  constexpr int PIECES = K_PIECES + V_PIECES;             // 16-byte pieces of one block, K first; both multiples of 64
+  constexpr int DMA_MAX = (PIECES + 255) / 256;           // loads per wave and block: DMA_MAX, or one less for the last waves
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r = lane & 31, h = lane >> 5;
-  const int qblk = a.causal ? (int)(gridDim.x - 1 - blockIdx.x) : (int)blockIdx.x;   // causal: long rows are dispatched first
+  // grid (heads, batch, row blocks): with a causal mask every head's longest rows are dispatched before anybody's shorter
+  // ones, so the launch ends with the cheapest workgroups
+  const int qblk = a.causal ? (int)(gridDim.z - 1 - blockIdx.z) : (int)blockIdx.z;
   const int q0 = (qblk * 4 + wave) * 32;
   const bool live = q0 < a.Sq;                    // a wave past the last row still helps with loads and barriers
-  const int hq = blockIdx.y, b = blockIdx.z;
+  const int hq = blockIdx.x, b = blockIdx.y;
   const int hk = hq / (a.Hq / a.Hk);
   const int64_t bhq = (int64_t)b * a.Hq + hq, bhk = (int64_t)b * a.Hk + hk;
   const int qrow = live ? q0 + r : 0;
@@ -106,34 +120,33 @@ __global__ __launch_bounds__(256, ATTN_WG_PER_CU) void attn_fwd_kernel(AttnArgs 
   }
   if (!live) nblk = 0;
 
-  // ---- cooperative fetch of one block: thread -> 16-byte pieces (K is contiguous; V is DV rows of 32 bytes)
-  uint4 kreg[K_PER_THREAD], vreg[V_PER_THREAD];
-  auto fetch = [&](int kb) {
-    const uint8_t* kblk = a.k + (bhk * a.Sk + kb * 64) * (D / 2);
-    const uint8_t* vblk = a.vt + bhk * DV * (int64_t)(a.Sk / 2) + kb * 32;
+  // ---- cooperative fetch of one block: wave instruction j moves pieces [256 j + 64 wave, + 64) of the block, K pieces
+  // first (contiguous in memory), then V pieces (piece p = 16 bytes of row p / 2, half p % 2); the piece index is also the
+  // position in the slot.  Blocks beyond the keys are out of the descriptors' range and arrive as zeros.
+  typedef __attribute__((address_space(3))) uint8_t lds_u8;
+  const __amdgpu_buffer_rsrc_t rsrc_k = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(a.k + bhk * a.Sk * (D / 2)), 0, a.Sk * (D / 2), 0x00020000);
+  const __amdgpu_buffer_rsrc_t rsrc_v = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(a.vt + bhk * DV * (int64_t)(a.Sk / 2)), 0, DV * (a.Sk / 2), 0x00020000);
+  const int n_dma = (PIECES - 64 * wave + 255) / 256;   // this wave's loads per block (wave-uniform)
+  auto dma = [&](int kb, int slot) {
+    lds_u8* base = (lds_u8*)ring + slot * SLOT;
 #pragma unroll
-    for (int i = 0; i < K_PER_THREAD; ++i) {
-      const int piece = tid + 256 * i;
-      if (K_PIECES % 256 == 0 || piece < K_PIECES) kreg[i] = *reinterpret_cast<const uint4*>(kblk + (uint32_t)piece * 16);
-    }
-#pragma unroll
-    for (int i = 0; i < V_PER_THREAD; ++i) {
-      const int piece = tid + 256 * i;
-      if (V_PIECES % 256 == 0 || piece < V_PIECES)
-        vreg[i] = *reinterpret_cast<const uint4*>(vblk + (uint32_t)(piece >> 1) * (uint32_t)(a.Sk / 2) + (piece & 1) * 16);
+    for (int j = 0; j < DMA_MAX; ++j) {
+      const int p0 = 256 * j + 64 * wave;   // wave-uniform
+      if (PIECES % 256 != 0 && p0 >= PIECES) continue;
+      if (p0 < K_PIECES) {
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_k, (__attribute__((address_space(3))) void*)(base + p0 * 16), 16, (p0 + lane) * 16,
+                                                 __builtin_amdgcn_readfirstlane(kb * K_BYTES), 0, 0);
+      } else {
+        const int p = p0 - K_PIECES + lane;
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_v, (__attribute__((address_space(3))) void*)(base + p0 * 16), 16,
+                                                 (p >> 1) * (a.Sk / 2) + (p & 1) * 16, __builtin_amdgcn_readfirstlane(kb * 32), 0, 0);
+      }
     }
   };
-  auto park = [&](int slot) {
-#pragma unroll
-    for (int i = 0; i < K_PER_THREAD; ++i) {
-      const int piece = tid + 256 * i;
-      if (K_PIECES % 256 == 0 || piece < K_PIECES) *reinterpret_cast<uint4*>(&ring[slot][piece * 16]) = kreg[i];
-    }
-#pragma unroll
-    for (int i = 0; i < V_PER_THREAD; ++i) {
-      const int piece = tid + 256 * i;
-      if (V_PIECES % 256 == 0 || piece < V_PIECES) *reinterpret_cast<uint4*>(&ring[slot][K_BYTES + piece * 16]) = vreg[i];
-    }
+  auto wait_dma = [&](bool one_block_in_flight) {   // this wave's loads are done, except the youngest block's if asked
+    if (!one_block_in_flight) __builtin_amdgcn_s_waitcnt(0x0070 | 0x0F00 | 0);                      // vmcnt(0)
+    else if (n_dma == DMA_MAX) __builtin_amdgcn_s_waitcnt(0x0070 | 0x0F00 | (DMA_MAX & 15));        // vmcnt(DMA_MAX)
+    else __builtin_amdgcn_s_waitcnt(0x0070 | 0x0F00 | ((DMA_MAX - 1) & 15));
   };
   // Scale bytes of a block: 2 D/32 bytes of K (key tile t, 32-column block j at byte t D/32 + j) and 2 Dv/32 bytes of V
   // (key tile t, column block d at byte t Dv/32 + d) sit at wave-uniform, 4-byte aligned addresses: whole dwords, one
@@ -149,23 +162,27 @@ __global__ __launch_bounds__(256, ATTN_WG_PER_CU) void attn_fwd_kernel(AttnArgs 
     for (int i = 0; i < VS_DW; ++i) vw[i] = vp[i];
   };
   if (wg_blk > 0) {
-    fetch(0);
     fetch_scales(0, ksw_next, vsw_next);
-    park(0);
+    dma(0, 0);
+    if (wg_blk > 1) dma(1, 1);
   }
-  __syncthreads();
+  // (the bare barrier instruction: `__syncthreads()` would first wait for every outstanding load, the prefetched block's
+  // included; the ring is written by the direct-to-LDS loads only, and wait_dma has waited for this wave's part)
+  wait_dma(wg_blk > 1);
+  asm volatile("s_barrier" ::: "memory");
 
+  int slot = 0;   // of block kb
   for (int kb = 0; kb < wg_blk; ++kb) {
     const int key0 = kb * 64;
-    const uint8_t* tile = ring[kb & 1];
+    const uint8_t* tile = ring + slot * SLOT;
 #pragma unroll
     for (int i = 0; i < KS_DW; ++i) ksw[i] = ksw_next[i];
 #pragma unroll
     for (int i = 0; i < VS_DW; ++i) vsw[i] = vsw_next[i];
-    if (kb + 1 < wg_blk) {                         // travels during this block's arithmetic
-      fetch(kb + 1);
-      fetch_scales(kb + 1, ksw_next, vsw_next);
-    }
+    // the next block's scale bytes, then the codes of the block after it (into the slot the previous block used: every wave
+    // left it at the last barrier); both travel during this block's arithmetic
+    if (kb + 1 < wg_blk) fetch_scales(kb + 1, ksw_next, vsw_next);
+    if (kb + 2 < wg_blk) dma(kb + 2, slot == 0 ? ATTN_RING - 1 : slot - 1);
     if (kb < nblk) {
       // ---- S = Q K^T for two 32-key tiles; K scale of (tile t, step s, half h) = byte t D/32 + 2 s + h
       v16f_t S[2];
@@ -256,15 +273,16 @@ __global__ __launch_bounds__(256, ATTN_WG_PER_CU) void attn_fwd_kernel(AttnArgs 
         acc_o[d] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(vf, pf, acc_o[d], 4, 4, d, vsh, 0, pscale);
       });
     }
-    if (kb + 1 < wg_blk) park((kb + 1) & 1);
-    __syncthreads();
+    wait_dma(kb + 2 < wg_blk);   // block kb + 1 has landed (this wave's part; the barrier collects the others')
+    asm volatile("s_barrier" ::: "memory");
+    slot = slot == ATTN_RING - 1 ? 0 : slot + 1;
   }
   if (!live) return;
 
   // ---- O = acc / l, bf16; log-sum-exp
   const float l = acc_l[0];
   const float rl = 1.0f / l;
-  __bf16* orow = reinterpret_cast<__bf16*>(a.out) + (bhq * a.Sq + qrow) * DV;
+  __bf16* orow = out + (bhq * a.Sq + qrow) * DV;
 #pragma unroll
   for (int d = 0; d < ND; ++d)
 #pragma unroll
@@ -279,12 +297,18 @@ __global__ __launch_bounds__(256, ATTN_WG_PER_CU) void attn_fwd_kernel(AttnArgs 
       w.y = __builtin_bit_cast(uint32_t, hi);
       *reinterpret_cast<uint2*>(orow + 32 * d + 8 * g + 4 * h) = w;
     }
-  if (h == 0) a.lse[bhq * a.Sq + qrow] = (m_i + log2f(l)) * ATTN_LN2;
+  if (h == 0) lse_out[bhq * a.Sq + qrow] = (m_i + log2f(l)) * ATTN_LN2;
+}
+
+template <int NK, int ND>
+__global__ __launch_bounds__(256, ATTN_WG_PER_CU) void attn_fwd_kernel(AttnArgs a) {
+  __shared__ __attribute__((aligned(16))) uint8_t ring[ATTN_RING * AttnTile<NK, ND>::SLOT];
+  attn_fwd_body<NK, ND>(a, reinterpret_cast<__bf16*>(a.out), a.lse, ring);
 }
 
 template <int NK, int ND>
 static int launch_attn(const AttnArgs& a, int B, hipStream_t st) {
-  dim3 grid((unsigned)((a.Sq + 127) / 128), (unsigned)a.Hq, (unsigned)B);
+  dim3 grid((unsigned)a.Hq, (unsigned)B, (unsigned)((a.Sq + 127) / 128));
   hipLaunchKernelGGL((attn_fwd_kernel<NK, ND>), grid, dim3(256), 0, st, a);
   return check_launch("attention_fwd");
 }
@@ -314,7 +338,7 @@ extern "C" int alto_mxfp4_attention_fwd(const void* q_codes, const void* q_scale
   ALTO_REQUIRE(Sk_used > 0 && Sk_used <= Sk && Sk - Sk_used < 64 && Sk_used % 32 == 0,
                "attention_fwd: Sk_used=%lld must be a multiple of 32 in (Sk - 64, Sk]", (long long)Sk_used);
   ALTO_REQUIRE(!causal || Sq <= Sk_used, "attention_fwd: causal attention needs Sq <= Sk (got %lld > %lld)", (long long)Sq, (long long)Sk_used);
-  ALTO_REQUIRE(B <= 65535 && Hq <= 65535, "attention_fwd: B and Hq must fit a grid dimension");
+  ALTO_REQUIRE(B <= 65535 && (Sq + 127) / 128 <= 65535, "attention_fwd: B and Sq / 128 must fit a grid dimension");
   ALTO_REQUIRE(B * Hq * Sq * (D > Dv ? D : Dv) < (1ll << 40), "attention_fwd: tensor too large");
   ALTO_REQUIRE(((uintptr_t)q_codes | (uintptr_t)k_codes | (uintptr_t)vt_codes) % 16 == 0 && (uintptr_t)out % 8 == 0,
                "attention_fwd: code pointers must be 16-byte aligned, out 8-byte aligned");
