@@ -126,6 +126,12 @@ __device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, __bf16* __restr
   typedef __attribute__((address_space(3))) uint8_t lds_u8;
   const __amdgpu_buffer_rsrc_t rsrc_k = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(a.k + bhk * a.Sk * (D / 2)), 0, a.Sk * (D / 2), 0x00020000);
   const __amdgpu_buffer_rsrc_t rsrc_v = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(a.vt + bhk * DV * (int64_t)(a.Sk / 2)), 0, DV * (a.Sk / 2), 0x00020000);
+  // Where a piece sits inside its row of the slot: the LDS serves a 16-byte read of 16 lanes per pass from 64 banks
+  // (256 bytes), and the 16 lanes of a fragment read ask for the same piece of 16 consecutive rows.  With PR pieces per
+  // row, 16 / PR rows share a 256-byte line; piece c of row `row` goes to position c ^ ((row / (16 / PR)) % PR), which
+  // spreads those 16 reads over all banks.  (Rows of 96 bytes, D = 192, keep the plain order.)  The loads put the pieces
+  // there: lane i of a load fills position p0 + i and fetches the piece that belongs there.
+  constexpr int KPR = D / 32, KSW = (KPR == 2 || KPR == 4 || KPR == 8) ? 16 / KPR : 0;   // pieces per K row; rows per swizzle step
   const int n_dma = (PIECES - 64 * wave + 255) / 256;   // this wave's loads per block (wave-uniform)
   auto dma = [&](int kb, int slot) {
     lds_u8* base = (lds_u8*)ring + slot * SLOT;
@@ -134,15 +140,19 @@ __device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, __bf16* __restr
       const int p0 = 256 * j + 64 * wave;   // wave-uniform
       if (PIECES % 256 != 0 && p0 >= PIECES) continue;
       if (p0 < K_PIECES) {
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_k, (__attribute__((address_space(3))) void*)(base + p0 * 16), 16, (p0 + lane) * 16,
+        const int p = p0 + lane, row = p / KPR;
+        const int c = KSW ? (p % KPR) ^ ((row / (KSW ? KSW : 1)) % KPR) : p % KPR;
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_k, (__attribute__((address_space(3))) void*)(base + p0 * 16), 16, (row * KPR + c) * 16,
                                                  __builtin_amdgcn_readfirstlane(kb * K_BYTES), 0, 0);
       } else {
-        const int p = p0 - K_PIECES + lane;
+        const int p = p0 - K_PIECES + lane, row = p >> 1;
         __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_v, (__attribute__((address_space(3))) void*)(base + p0 * 16), 16,
-                                                 (p >> 1) * (a.Sk / 2) + (p & 1) * 16, __builtin_amdgcn_readfirstlane(kb * 32), 0, 0);
+                                                 row * (a.Sk / 2) + (((p & 1) ^ ((row >> 3) & 1)) * 16), __builtin_amdgcn_readfirstlane(kb * 32), 0, 0);
       }
     }
   };
+  const int k_swz = KSW ? ((r / (KSW ? KSW : 1)) % KPR) * 16 : 0;   // XOR on the byte offset of a piece inside its K row
+  const int v_swz = ((r >> 3) & 1) * 16;                            // and inside its 32-byte V row
   auto wait_dma = [&](bool one_block_in_flight) {   // this wave's loads are done, except the youngest block's if asked
     if (!one_block_in_flight) __builtin_amdgcn_s_waitcnt(0x0070 | 0x0F00 | 0);                      // vmcnt(0)
     else if (n_dma == DMA_MAX) __builtin_amdgcn_s_waitcnt(0x0070 | 0x0F00 | (DMA_MAX & 15));        // vmcnt(DMA_MAX)
@@ -196,7 +206,7 @@ __device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, __bf16* __restr
         static_for<NK>([&](auto sc) {
           constexpr int s = decltype(sc)::value;
           constexpr int byte = t * (D / 32) + 2 * s;
-          const v8i_t kf = frag16(tile + (32 * t + r) * (D / 2) + 32 * s + 16 * h);
+          const v8i_t kf = frag16(tile + (32 * t + r) * (D / 2) + ((32 * s + 16 * h) ^ k_swz));
           S[t] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(kf, qf[s], S[t], 4, 4, byte % 4, ksh[byte / 4], 0, qsc[s]);
         });
       });
@@ -269,7 +279,7 @@ __device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, __bf16* __restr
       const int vsh = DV == 128 ? (int)(h ? vsw[VS_DW - 1] : vsw[0]) : (int)(vsw[0] >> (16 * h));
       static_for<ND>([&](auto dc) {
         constexpr int d = decltype(dc)::value;
-        const v8i_t vf = frag16(tile + K_BYTES + (32 * d + r) * 32 + 16 * h);
+        const v8i_t vf = frag16(tile + K_BYTES + (32 * d + r) * 32 + ((16 * h) ^ v_swz));
         acc_o[d] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(vf, pf, acc_o[d], 4, 4, d, vsh, 0, pscale);
       });
     }
