@@ -69,8 +69,8 @@ def triton_attention_mxfp4(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, al
                            bias: Optional[torch.Tensor] = None, sm_scale: Optional[float] = None, dropout_p: float = 0.0,
                            cu_seqlens_q=0, cu_seqlens_k=0, max_seqlens_q: Optional[int] = None, max_seqlens_k: Optional[int] = None,
                            causal: bool = True, return_scores: bool = False, use_exp2: bool = True, layout: str = "bhsd"):
-    """(q, k, v) [B,H,S,D] (or [B,S,H,D] with ``layout="bshd"``) -> (out bf16 in the layout of q, softmax_lse fp32 [B,H,S],
-    exp_scores placeholder), as :1206-1239.
+    """(q, k, v) [B,H,S,D] (or [B,S,H,D] with ``layout="bshd"``, or packed [T,H,D] with ``layout="thd"`` and ``cu_seqlens_*``)
+    -> (out bf16 in the layout of q, softmax_lse fp32 [B,H,S] ([T,H] for 'thd'), exp_scores placeholder), as :1206-1239.
 
     ``use_exp2`` is accepted either way: both settings evaluate exp(x) as exp2(x * log2 e) on the GPU's exp unit.
     """
@@ -83,8 +83,31 @@ def triton_attention_mxfp4(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, al
                                                   dropout_p, cu_seqlens_q, cu_seqlens_k, max_seqlens_q, max_seqlens_k, causal, return_scores,
                                                   use_exp2, "bhsd")
         return out.transpose(1, 2), lse, scores
+    if layout == "thd":
+        # Variable-length sequences packed along the tokens: q [Tq, Hq, D], k / v [Tk, Hk, D], boundaries cu_seqlens_q /
+        # cu_seqlens_k (int [n + 1], leading 0); out [Tq, Hq, Dv], softmax_lse [Tq, Hq] (the shapes of :1199-1203).  Every
+        # sequence is the 'bhsd' attention of its own rows: its 32 x 32 quantisation blocks start at its first token, so the
+        # boundaries must be multiples of 32 (no block may belong to two sequences), and a causal mask is aligned to the
+        # bottom-right corner of each sequence's own score matrix.  One launch per sequence.
+        cq = [int(c) for c in (cu_seqlens_q.tolist() if isinstance(cu_seqlens_q, torch.Tensor) else cu_seqlens_q)]
+        ck = [int(c) for c in (cu_seqlens_k.tolist() if isinstance(cu_seqlens_k, torch.Tensor) else cu_seqlens_k)]
+        torch._check(q.dim() == 3 and k.dim() == 3 and v.dim() == 3, lambda: "layout 'thd' takes [tokens, heads, head dim] tensors")
+        torch._check(len(cq) == len(ck) and len(cq) >= 2 and cq[0] == 0 and ck[0] == 0 and cq[-1] == q.shape[0] and ck[-1] == k.shape[0],
+                     lambda: "cu_seqlens_q / cu_seqlens_k must start at 0, end at the token counts and describe the same number of sequences")
+        torch._check(all(c % 32 == 0 for c in cq) and all(c % 32 == 0 for c in ck), lambda: "sequence boundaries must be multiples of 32 tokens")
+        out = torch.empty((q.shape[0], q.shape[1], v.shape[2]), dtype=torch.bfloat16, device=q.device)
+        lse = torch.empty((q.shape[0], q.shape[1]), dtype=torch.float32, device=q.device)
+        for i in range(len(cq) - 1):
+            q0, q1, k0, k1 = cq[i], cq[i + 1], ck[i], ck[i + 1]
+            torch._check(q1 > q0 and k1 > k0, lambda: "empty sequences are not supported")
+            o_i, l_i, _ = triton_attention_mxfp4(q[q0:q1].transpose(0, 1).unsqueeze(0), k[k0:k1].transpose(0, 1).unsqueeze(0),
+                                                 v[k0:k1].transpose(0, 1).unsqueeze(0), alibi_slopes, bias, sm_scale, dropout_p, 0, 0,
+                                                 q1 - q0, k1 - k0, causal, return_scores, use_exp2, "bhsd")
+            out[q0:q1] = o_i[0].transpose(0, 1)
+            lse[q0:q1] = l_i[0].transpose(0, 1)
+        return out, lse, torch.empty([], device=q.device, dtype=torch.float32)
     if layout != "bhsd":
-        raise NotImplementedError(f"layout {layout!r}: 'bhsd' and 'bshd' are implemented ('thd' packs variable-length sequences)")
+        raise NotImplementedError(f"layout {layout!r}: 'bhsd', 'bshd' and 'thd' are implemented")
     if alibi_slopes is not None or bias is not None:
         raise NotImplementedError("alibi slopes and bias are not implemented")
     if dropout_p != 0.0:

@@ -141,10 +141,39 @@ def test_layout_bshd_is_the_same_attention_on_permuted_views(m):
     assert torch.equal(o2.transpose(1, 2), o) and torch.equal(lse2, lse)
 
 
+@pytest.mark.parametrize("causal", [True, False])
+def test_layout_thd_is_the_attention_of_every_sequence(m, causal):
+    """Packed variable-length sequences (layout 'thd', cu_seqlens): each sequence's rows equal the 'bhsd' attention of that
+    sequence alone and match the CPU model; lengths of 32, 96 (half a key block), 256 and 160 / 192 (Sq < Sk)."""
+    Hq, Hk, D, Dv = 4, 2, 128, 128
+    lens_q, lens_k = [32, 96, 256, 160], [32, 96, 256, 192]
+    cq = [0] + list(torch.tensor(lens_q).cumsum(0).tolist())
+    ck = [0] + list(torch.tensor(lens_k).cumsum(0).tolist())
+    g = torch.Generator().manual_seed(17)
+    q = torch.randn(cq[-1], Hq, D, generator=g).to(torch.bfloat16)
+    k = torch.randn(ck[-1], Hk, D, generator=g).to(torch.bfloat16)
+    v = torch.randn(ck[-1], Hk, Dv, generator=g).to(torch.bfloat16)
+    out, lse, _ = m.triton_attention_mxfp4(q.to(DEV), k.to(DEV), v.to(DEV), sm_scale=D ** -0.5, cu_seqlens_q=torch.tensor(cq, dtype=torch.int32),
+                                           cu_seqlens_k=ck, max_seqlens_q=max(lens_q), max_seqlens_k=max(lens_k), causal=causal, layout="thd")
+    assert out.shape == (cq[-1], Hq, Dv) and out.dtype == torch.bfloat16 and lse.shape == (cq[-1], Hq)
+    for i in range(len(lens_q)):
+        qi, ki, vi = (t.transpose(0, 1).unsqueeze(0) for t in (q[cq[i]:cq[i + 1]], k[ck[i]:ck[i + 1]], v[ck[i]:ck[i + 1]]))
+        o1, l1, _ = m.triton_attention_mxfp4(qi.to(DEV), ki.to(DEV), vi.to(DEV), sm_scale=D ** -0.5, causal=causal)
+        assert torch.equal(out[cq[i]:cq[i + 1]].transpose(0, 1), o1[0]) and torch.equal(lse[cq[i]:cq[i + 1]].transpose(0, 1), l1[0])
+        ref, ref_lse = attention_fwd_ref(qi, ki, vi, causal=causal)
+        assert _rel(o1.cpu(), ref) <= REL_L2 and float((l1.cpu() - ref_lse).abs().max()) <= 1e-4
+
+
 def test_rejected_arguments(m):
     q, k, v = (t.to(DEV) for t in _qkv(1, 2, 2, 64, 64, 64, 64, seed=1))
     with pytest.raises(NotImplementedError):
-        m.triton_attention_mxfp4(q, k, v, layout="thd")
+        m.triton_attention_mxfp4(q, k, v, layout="hsd")
+    with pytest.raises(RuntimeError, match="multiples of 32"):
+        m.triton_attention_mxfp4(q[0].transpose(0, 1), k[0].transpose(0, 1), v[0].transpose(0, 1), cu_seqlens_q=[0, 40, 64], cu_seqlens_k=[0, 32, 64],
+                                 layout="thd")
+    with pytest.raises(RuntimeError, match="same number of sequences"):
+        m.triton_attention_mxfp4(q[0].transpose(0, 1), k[0].transpose(0, 1), v[0].transpose(0, 1), cu_seqlens_q=[0, 64], cu_seqlens_k=[0, 32, 64],
+                                 layout="thd")
     with pytest.raises(NotImplementedError):
         m.triton_attention_mxfp4(q, k, v, dropout_p=0.1)
     with pytest.raises(NotImplementedError):
