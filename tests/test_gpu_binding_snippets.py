@@ -27,7 +27,13 @@ def lib():
     _lib.alto_mxfp4_grouped_gemm_workspace_bytes.argtypes = [i64, i32]
     _lib.alto_mxfp4_grouped_gemm.argtypes = [vp, i64, vp, i64, i64, i32, vp, i64, i64, vp, i64, i64, i64, i32,
                                              vp, vp, i32, i32, i64, i64, i64, vp, i32, i64, vp, i64, vp]
+    _lib.alto_mxfp4_quantize_ex.argtypes = [vp, i32, i64, i64, i64, i64, i64, vp, vp, vp, vp, i64, i64, i32, i32,
+                                            vp, i64, i64, u64, u64, vp, i32, vp, vp, i32, i32, i32, vp]
+    _lib.alto_mxfp4_gemm_ps.argtypes = [vp, i64, vp, vp, i64, vp, i64, i64, i64, vp, i64, f32, vp]
     return _lib
+
+
+PACK_ROW_SCALES = 1
 
 
 def _check(lib, rc):
@@ -77,6 +83,39 @@ def grouped_forward(lib, a, a_s, w, w_s, offs, N):
                                             offs.data_ptr(), None, E, E, M_total, N, K, out.data_ptr(), 0, out.stride(0),
                                             ws.data_ptr(), nbytes, _stream()))
     return out
+
+
+def convert_to_mxfp4_rows_packed(lib, x, is_2d):
+    M, C = x.shape
+    codes = torch.empty(M, C // 2, dtype=torch.uint8, device=x.device)
+    packed = torch.empty(-(-C // 512), M, 16, dtype=torch.uint8, device=x.device)
+    _check(lib, lib.alto_mxfp4_quantize_ex(x.data_ptr(), 0 if x.dtype == torch.bfloat16 else 1, 1, M, C, x.stride(0), M * x.stride(0),
+                                           codes.data_ptr(), packed.data_ptr(), None, None, C // 2, 0, int(is_2d), 0,
+                                           None, 0, 0, 0, 0, None, 0, None, None, 0, 0, PACK_ROW_SCALES, _stream()))
+    return codes, packed
+
+
+def gemm_nt_packed(lib, a, a_ps, b, b_ps):
+    M, N, K = a.shape[0], b.shape[0], a.shape[1] * 2
+    c = torch.empty(M, N, dtype=torch.bfloat16, device=a.device)
+    _check(lib, lib.alto_mxfp4_gemm_ps(a.data_ptr(), a.stride(0), a_ps.data_ptr(), b.data_ptr(), b.stride(0), b_ps.data_ptr(),
+                                       M, N, K, c.data_ptr(), c.stride(0), 1.0, _stream()))
+    return c
+
+
+def test_packed_scale_bindings(lib):
+    """Quantizer with the layout flag + the GEMM on packed scales: same bits as the plain pair of calls, 2D weight blocks."""
+    x = randn_outliers((256, 1056), torch.bfloat16, seed=76).to(DEV)
+    w = (randn_outliers((384, 1056), torch.bfloat16, seed=77) * 0.02).to(DEV)
+    xq, xs = convert_to_mxfp4_rows(lib, x)
+    xq2, xps = convert_to_mxfp4_rows_packed(lib, x, False)
+    assert torch.equal(xq, xq2)
+    import alto_amd.mxfp4 as m
+    wq, ws = m.convert_to_mxfp4(w, axis=-1, is_2d_block=True)
+    wq2, wps = convert_to_mxfp4_rows_packed(lib, w, True)
+    assert torch.equal(wq, wq2)
+    want = gemm_nt(lib, xq, xs, wq, ws, True, torch.bfloat16)
+    assert torch.equal(gemm_nt_packed(lib, xq2, xps, wq2, wps), want)
 
 
 def test_row_quantizer_and_gemm_bindings(lib):
