@@ -77,6 +77,8 @@ SIGNATURES = {
     "alto_mxfp4_probe_mfma": (c_int, [c_int, c_int, c_int, c_vp, c_vp, c_vp]),
     "alto_mxfp4_attention_fwd": (c_int, [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64,
                                          c_f32, c_int, c_vp]),
+    "alto_mxfp4_attention_fwd_ex": (c_int, [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64,
+                                            c_f32, c_int, c_vp, c_i64, c_i64, c_i64, c_vp, c_i64, c_i64, c_vp]),
     "alto_mxfp4_random_bits": (c_int, [c_vp, c_i64, ctypes.c_uint64, ctypes.c_uint64, c_vp]),
     "alto_mxfp4_qdq": (c_int, [c_vp, c_int, c_i64, c_i64, c_i64, c_i64, c_i64, c_vp, c_i64, c_i64, c_int, c_int, c_vp]),
 }

@@ -21,6 +21,9 @@ struct AttnArgs {
   int Hq, Hk, Sq, Sk, Sk_used;             // Sk keys are allocated (a multiple of 64), the first Sk_used exist
   float sm_scale;
   int causal;
+  // optional additive terms on the scaled scores (triton_flash_attention_mxfp4.py:288-299), fp32:
+  const float* bias;  int64_t bias_sb, bias_sh, bias_sm, bias_bytes;   // element (b, h, m, n) at b sb + h sh + m sm + n; NULL: none
+  const float* alibi; int64_t alibi_sb, alibi_sh;                      // slope of (b, h) at b sb + h sh; NULL: none
 };
 
 #ifndef ATTN_WG_PER_CU
@@ -64,7 +67,9 @@ struct AttnTile {
 // The body of the kernel as a function of its own because of the `__restrict__` on the outputs: inlining then marks the
 // direct-to-LDS loads as not aliasing them, and only with that mark does the compiler's wait insertion keep those loads
 // in flight across the LDS reads that follow (unmarked, it puts an `s_waitcnt vmcnt(0)` before the next LDS read).
-template <int NK, int ND>
+// BIASED: the scores get a.bias and / or the ALiBi term -slope |row + Sk - Sq - key| added after the scaling and the mask,
+// before the running maximum (:288-308); a separate instantiation, the plain one carries none of it.
+template <int NK, int ND, bool BIASED>
 __device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, __bf16* __restrict__ out, float* __restrict__ lse_out, uint8_t* ring) {
   constexpr int D = NK * 64, DV = ND * 32;
   constexpr int K_BYTES = AttnTile<NK, ND>::K_BYTES, V_BYTES = AttnTile<NK, ND>::V_BYTES, SLOT = AttnTile<NK, ND>::SLOT;
@@ -104,6 +109,12 @@ __device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, __bf16* __restr
   for (int v = 0; v < 16; ++v) acc_l[v] = 0.0f;
   float m_i = -__builtin_inff();                   // running row max of S * sm_scale * log2(e)
   const float c2 = a.sm_scale * ATTN_RCP_LN2;
+  const float cs = BIASED ? 1.0f : c2;   // what is left to multiply once the scores are in the base-2 domain
+  // bias rows of this (batch, head): a descriptor over the rest of the tensor (no range when there is no bias: loads give 0)
+  const __amdgpu_buffer_rsrc_t rsrc_bias = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<float*>((BIASED && a.bias) ? a.bias + b * a.bias_sb + hq * a.bias_sh : nullptr), 0,
+      (BIASED && a.bias) ? (int)(a.bias_bytes - (b * a.bias_sb + hq * a.bias_sh) * 4) : 0, 0x00020000);
+  const float slope2 = (BIASED && a.alibi) ? a.alibi[b * a.alibi_sb + hq * a.alibi_sh] * ATTN_RCP_LN2 : 0.0f;
 
   const v8i_t ones = v8i_t{0x22222222, 0x22222222, 0x22222222, 0x22222222, 0, 0, 0, 0};   // E2M1 code 2 = 1.0
 
@@ -194,6 +205,16 @@ __device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, __bf16* __restr
     if (kb + 1 < wg_blk) fetch_scales(kb + 1, ksw_next, vsw_next);
     if (kb + 2 < wg_blk) dma(kb + 2, slot == 0 ? ATTN_RING - 1 : slot - 1);
     if (kb < nblk) {
+      v4f_t bb[BIASED ? 2 : 1][BIASED ? 4 : 1];   // bias of this lane's 32 scores: keys key0 + 32 t + 8 g + 4 h + (0..3)
+      if constexpr (BIASED) {
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            const v4i_t w = __builtin_amdgcn_raw_buffer_load_b128(rsrc_bias, (int)((qrow * a.bias_sm + key0 + 32 * t + 8 * g + 4 * h) * 4), 0, 0);
+            bb[t][g] = __builtin_bit_cast(v4f_t, w);
+          }
+      }
       // ---- S = Q K^T for two 32-key tiles; K scale of (tile t, step s, half h) = byte t D/32 + 2 s + h
       v16f_t S[2];
       int ksh[KS_DW];
@@ -210,6 +231,17 @@ __device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, __bf16* __restr
           S[t] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(kf, qf[s], S[t], 4, 4, byte % 4, ksh[byte / 4], 0, qsc[s]);
         });
       });
+      if constexpr (BIASED) {   // scores into the base-2 domain with their additive terms
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int v = 0; v < 16; ++v) {
+            const int key = key0 + 32 * t + 8 * (v >> 2) + 4 * h + (v & 3);
+            float x = __builtin_fmaf(bb[t][v >> 2][v & 3], ATTN_RCP_LN2, S[t][v] * c2);
+            x = __builtin_fmaf(-slope2, __builtin_fabsf((float)(qrow + shift - key)), x);
+            S[t][v] = x;
+          }
+      }
       // ---- mask (only blocks the diagonal crosses or that reach past the last key), running max kept in the base-2 domain: m = max(S) * sm_scale * log2(e)
       if ((a.causal && key0 + 63 > q0 + shift) || key0 + 64 > a.Sk_used) {
         asm volatile("" ::: "memory");   // keep this a branch: most blocks skip it
@@ -230,9 +262,13 @@ __device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, __bf16* __restr
         tmx[t] = pair_max(x);
       }
       const float mx = fmaxf(tmx[0], tmx[1]);
-      const float m_new = fmaxf(m_i, mx * c2);
-      const float alpha = __builtin_amdgcn_exp2f(m_i - m_new);
+      float m_new = fmaxf(m_i, mx * cs);
+      // a bias may hide every key a row has seen so far (-inf): such a row keeps m = -inf and takes exp2(-inf - 0) = 0
+      // everywhere instead of exp2(-inf + inf)
+      const float m_sub = (BIASED && m_new == -__builtin_inff()) ? 0.0f : m_new;
+      const float alpha = __builtin_amdgcn_exp2f(m_i - m_sub);
       m_i = m_new;
+      m_new = m_sub;
 
       // ---- probabilities, one E8M0 scale per (row, 32 keys), E2M1 codes (round to nearest even)
       uint32_t c[2][2];
@@ -240,8 +276,8 @@ __device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, __bf16* __restr
 #pragma unroll
       for (int t = 0; t < 2; ++t) {
 #pragma unroll
-        for (int v = 0; v < 16; ++v) S[t][v] = __builtin_amdgcn_exp2f(__builtin_fmaf(S[t][v], c2, -m_new));
-        const float am = __builtin_amdgcn_exp2f(__builtin_fmaf(tmx[t], c2, -m_new));   // = max of the 32 values above
+        for (int v = 0; v < 16; ++v) S[t][v] = __builtin_amdgcn_exp2f(__builtin_fmaf(S[t][v], cs, -m_new));
+        const float am = __builtin_amdgcn_exp2f(__builtin_fmaf(tmx[t], cs, -m_new));   // = max of the 32 values above
         const uint32_t e = e8m0_from_f32_bits(f2u(am));
         psc[t] = (int)e;
         const float scale_f = u2f(e << 23);
@@ -310,16 +346,17 @@ __device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, __bf16* __restr
   if (h == 0) lse_out[bhq * a.Sq + qrow] = (m_i + log2f(l)) * ATTN_LN2;
 }
 
-template <int NK, int ND>
-__global__ __launch_bounds__(256, ATTN_WG_PER_CU) void attn_fwd_kernel(AttnArgs a) {
+template <int NK, int ND, bool BIASED>
+__global__ __launch_bounds__(256, BIASED ? 2 : ATTN_WG_PER_CU) void attn_fwd_kernel(AttnArgs a) {
   __shared__ __attribute__((aligned(16))) uint8_t ring[ATTN_RING * AttnTile<NK, ND>::SLOT];
-  attn_fwd_body<NK, ND>(a, reinterpret_cast<__bf16*>(a.out), a.lse, ring);
+  attn_fwd_body<NK, ND, BIASED>(a, reinterpret_cast<__bf16*>(a.out), a.lse, ring);
 }
 
 template <int NK, int ND>
 static int launch_attn(const AttnArgs& a, int B, hipStream_t st) {
   dim3 grid((unsigned)a.Hq, (unsigned)B, (unsigned)((a.Sq + 127) / 128));
-  hipLaunchKernelGGL((attn_fwd_kernel<NK, ND>), grid, dim3(256), 0, st, a);
+  if (a.bias || a.alibi) hipLaunchKernelGGL((attn_fwd_kernel<NK, ND, true>), grid, dim3(256), 0, st, a);
+  else hipLaunchKernelGGL((attn_fwd_kernel<NK, ND, false>), grid, dim3(256), 0, st, a);
   return check_launch("attention_fwd");
 }
 
@@ -334,11 +371,20 @@ static int launch_attn_nd(const AttnArgs& a, int B, int Dv, hipStream_t st) {
 
 }  // namespace alto
 
-extern "C" int alto_mxfp4_attention_fwd(const void* q_codes, const void* q_scales, const void* k_codes, const void* k_scales,
-                                        const void* vt_codes, const void* v_scales, void* out, float* lse, int64_t B, int64_t Hq,
-                                        int64_t Hk, int64_t Sq, int64_t Sk, int64_t Sk_used, int64_t D, int64_t Dv, float sm_scale,
-                                        int causal, void* stream) {
+extern "C" int alto_mxfp4_attention_fwd_ex(const void* q_codes, const void* q_scales, const void* k_codes, const void* k_scales,
+                                           const void* vt_codes, const void* v_scales, void* out, float* lse, int64_t B, int64_t Hq,
+                                           int64_t Hk, int64_t Sq, int64_t Sk, int64_t Sk_used, int64_t D, int64_t Dv, float sm_scale,
+                                           int causal, const float* bias, int64_t bias_sb, int64_t bias_sh, int64_t bias_sm,
+                                           const float* alibi_slopes, int64_t alibi_sb, int64_t alibi_sh, void* stream) {
   using namespace alto;
+  int64_t bias_bytes = 0;
+  if (bias) {
+    ALTO_REQUIRE(bias_sb >= 0 && bias_sh >= 0 && bias_sm >= Sk_used && bias_sm % 4 == 0 && (uintptr_t)bias % 16 == 0,
+                 "attention_fwd: bias rows must be 16-byte aligned with unit stride along the keys (row stride %lld)", (long long)bias_sm);
+    bias_bytes = ((B - 1) * bias_sb + (Hq - 1) * bias_sh + (Sq - 1) * bias_sm + Sk_used) * 4;
+    ALTO_REQUIRE(bias_bytes < (1ll << 32) && Sq * bias_sm * 4 < (1ll << 31), "attention_fwd: bias tensor too large");
+  }
+  ALTO_REQUIRE(!alibi_slopes || (alibi_sb >= 0 && alibi_sh >= 0), "attention_fwd: negative alibi strides");
   ALTO_REQUIRE(q_codes && q_scales && k_codes && k_scales && vt_codes && v_scales && out && lse, "attention_fwd: null pointer");
   ALTO_REQUIRE(B > 0 && Hq > 0 && Hk > 0 && Hq % Hk == 0, "attention_fwd: Hq=%lld must be a positive multiple of Hk=%lld", (long long)Hq, (long long)Hk);
   ALTO_REQUIRE(Sq > 0 && Sq % 32 == 0, "attention_fwd: Sq=%lld must be a positive multiple of 32", (long long)Sq);
@@ -354,7 +400,8 @@ extern "C" int alto_mxfp4_attention_fwd(const void* q_codes, const void* q_scale
                "attention_fwd: code pointers must be 16-byte aligned, out 8-byte aligned");
   ALTO_REQUIRE(((uintptr_t)k_scales | (uintptr_t)v_scales) % 4 == 0, "attention_fwd: K and V scale pointers must be 4-byte aligned");
   AttnArgs a{(const uint8_t*)q_codes, (const uint8_t*)q_scales, (const uint8_t*)k_codes, (const uint8_t*)k_scales,
-             (const uint8_t*)vt_codes, (const uint8_t*)v_scales, out, lse, (int)Hq, (int)Hk, (int)Sq, (int)Sk, (int)Sk_used, sm_scale, causal ? 1 : 0};
+             (const uint8_t*)vt_codes, (const uint8_t*)v_scales, out, lse, (int)Hq, (int)Hk, (int)Sq, (int)Sk, (int)Sk_used, sm_scale, causal ? 1 : 0,
+             bias, bias_sb, bias_sh, bias_sm, bias_bytes, alibi_slopes, alibi_sb, alibi_sh};
   hipStream_t st = (hipStream_t)stream;
   switch (D) {
     case 64: return launch_attn_nd<1>(a, (int)B, (int)Dv, st);
@@ -363,4 +410,12 @@ extern "C" int alto_mxfp4_attention_fwd(const void* q_codes, const void* q_scale
     case 256: return launch_attn_nd<4>(a, (int)B, (int)Dv, st);
   }
   return ALTO_MXFP4_EINVAL;
+}
+
+extern "C" int alto_mxfp4_attention_fwd(const void* q_codes, const void* q_scales, const void* k_codes, const void* k_scales,
+                                        const void* vt_codes, const void* v_scales, void* out, float* lse, int64_t B, int64_t Hq,
+                                        int64_t Hk, int64_t Sq, int64_t Sk, int64_t Sk_used, int64_t D, int64_t Dv, float sm_scale,
+                                        int causal, void* stream) {
+  return alto_mxfp4_attention_fwd_ex(q_codes, q_scales, k_codes, k_scales, vt_codes, v_scales, out, lse, B, Hq, Hk, Sq, Sk, Sk_used, D, Dv, sm_scale,
+                                     causal, nullptr, 0, 0, 0, nullptr, 0, 0, stream);
 }

@@ -19,13 +19,16 @@ from .quantization import _prep, _quantize_call
 
 
 def attention_mxfp4_forward(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, q_scale: torch.Tensor, k_scale: torch.Tensor,
-                            v_scale: torch.Tensor, sm_scale: float, causal: bool, seqlen_k: Optional[int] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+                            v_scale: torch.Tensor, sm_scale: float, causal: bool, seqlen_k: Optional[int] = None,
+                            bias: Optional[torch.Tensor] = None, alibi_slopes: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor]:
     """Pre-quantised operands -> (out bf16 [B,Hq,Sq,Dv], lse fp32 [B,Hq,Sq]).
 
     q [B,Hq,Sq,D/2], q_scale [B,Hq,Sq/32,D/32]; k [B,Hk,Sk,D/2], k_scale [B,Hk,Sk/32,D/32]; v packed along the keys:
     [B,Hk,Dv,Sk/2] with v_scale [B,Hk,Sk/32,Dv/32] (the reference's kernel takes V packed along Dv and unpacks it inside
     ``tl.dot_scaled(..., rhs_k_pack=False)``, :393; same codes, other byte order).  The key dim of k / v is a multiple of
     64; ``seqlen_k`` (default: all of it) says how many keys exist when the caller padded a sequence of 32 (mod 64) keys.
+    ``bias`` (broadcastable to [B, Hq, Sq, seqlen_k]) is added to the scaled scores, ``alibi_slopes`` ([Hq] or [B, Hq]) give
+    the ALiBi term ``-slope * |row + Sk - Sq - key|`` (:135-164,288-299).
     """
     rt.require_gpu(q, k, v, q_scale, k_scale, v_scale)
     for t in (q, k, v, q_scale, k_scale, v_scale):
@@ -38,10 +41,36 @@ def attention_mxfp4_forward(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, q
     assert v_scale.shape == (B, Hk, Sk // 32, Dv // 32)
     out = torch.empty((B, Hq, Sq, Dv), dtype=torch.bfloat16, device=q.device)
     lse = torch.empty((B, Hq, Sq), dtype=torch.float32, device=q.device)
-    check(rt.lib().alto_mxfp4_attention_fwd(q.data_ptr(), q_scale.data_ptr(), k.data_ptr(), k_scale.data_ptr(), v.data_ptr(),
-                                            v_scale.data_ptr(), out.data_ptr(), lse.data_ptr(), B, Hq, Hk, Sq, Sk,
-                                            Sk if seqlen_k is None else int(seqlen_k), D, Dv,
-                                            float(sm_scale), int(bool(causal)), rt.stream_ptr(q.device)), "alto_mxfp4_attention_fwd")
+    sk_used = Sk if seqlen_k is None else int(seqlen_k)
+    b4 = sl = None
+    if bias is not None:
+        rt.require_gpu(bias)
+        b4 = bias.to(torch.float32)
+        while b4.dim() < 4:
+            b4 = b4.unsqueeze(0)
+        torch._check(b4.shape[-2] == Sq and b4.shape[-1] == sk_used and b4.shape[0] in (1, B) and b4.shape[1] in (1, Hq),
+                     lambda: f"bias of shape {tuple(bias.shape)} does not broadcast to {(B, Hq, Sq, sk_used)}")
+        if b4.stride(3) != 1 or b4.stride(2) % 4 or b4.data_ptr() % 16 or (b4.shape[0] > 1 and b4.stride(0) < 0) or (b4.shape[1] > 1 and b4.stride(1) < 0):
+            b4 = b4.contiguous()
+    if alibi_slopes is not None:
+        rt.require_gpu(alibi_slopes)
+        sl = alibi_slopes.to(torch.float32)
+        if sl.dim() == 1:
+            sl = sl.unsqueeze(0)
+        torch._check(sl.dim() == 2 and sl.shape[1] == Hq and sl.shape[0] in (1, B), lambda: f"alibi_slopes of shape {tuple(alibi_slopes.shape)}: [Hq] or [B, Hq]")
+        sl = sl.contiguous()
+    if b4 is None and sl is None:
+        check(rt.lib().alto_mxfp4_attention_fwd(q.data_ptr(), q_scale.data_ptr(), k.data_ptr(), k_scale.data_ptr(), v.data_ptr(),
+                                                v_scale.data_ptr(), out.data_ptr(), lse.data_ptr(), B, Hq, Hk, Sq, Sk, sk_used, D, Dv,
+                                                float(sm_scale), int(bool(causal)), rt.stream_ptr(q.device)), "alto_mxfp4_attention_fwd")
+        return out, lse
+    check(rt.lib().alto_mxfp4_attention_fwd_ex(
+        q.data_ptr(), q_scale.data_ptr(), k.data_ptr(), k_scale.data_ptr(), v.data_ptr(), v_scale.data_ptr(), out.data_ptr(), lse.data_ptr(),
+        B, Hq, Hk, Sq, Sk, sk_used, D, Dv, float(sm_scale), int(bool(causal)),
+        rt.ptr(b4), 0 if b4 is None or b4.shape[0] == 1 else b4.stride(0), 0 if b4 is None or b4.shape[1] == 1 else b4.stride(1),
+        0 if b4 is None else b4.stride(2),
+        rt.ptr(sl), 0 if sl is None or sl.shape[0] == 1 else sl.stride(0), 0 if sl is None else sl.stride(1),
+        rt.stream_ptr(q.device)), "alto_mxfp4_attention_fwd_ex")
     return out, lse
 
 
@@ -92,6 +121,10 @@ def triton_attention_mxfp4(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, al
         cq = [int(c) for c in (cu_seqlens_q.tolist() if isinstance(cu_seqlens_q, torch.Tensor) else cu_seqlens_q)]
         ck = [int(c) for c in (cu_seqlens_k.tolist() if isinstance(cu_seqlens_k, torch.Tensor) else cu_seqlens_k)]
         torch._check(q.dim() == 3 and k.dim() == 3 and v.dim() == 3, lambda: "layout 'thd' takes [tokens, heads, head dim] tensors")
+        if bias is not None:
+            raise NotImplementedError("a bias tensor with layout 'thd' is not implemented (ALiBi slopes are)")
+        if alibi_slopes is not None and alibi_slopes.dim() == 2:
+            raise NotImplementedError("layout 'thd' takes one ALiBi slope per head")
         torch._check(len(cq) == len(ck) and len(cq) >= 2 and cq[0] == 0 and ck[0] == 0 and cq[-1] == q.shape[0] and ck[-1] == k.shape[0],
                      lambda: "cu_seqlens_q / cu_seqlens_k must start at 0, end at the token counts and describe the same number of sequences")
         torch._check(all(c % 32 == 0 for c in cq) and all(c % 32 == 0 for c in ck), lambda: "sequence boundaries must be multiples of 32 tokens")
@@ -108,8 +141,6 @@ def triton_attention_mxfp4(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, al
         return out, lse, torch.empty([], device=q.device, dtype=torch.float32)
     if layout != "bhsd":
         raise NotImplementedError(f"layout {layout!r}: 'bhsd', 'bshd' and 'thd' are implemented")
-    if alibi_slopes is not None or bias is not None:
-        raise NotImplementedError("alibi slopes and bias are not implemented")
     if dropout_p != 0.0:
         raise NotImplementedError("dropout is not implemented (the reference's own dropout is a no-op after PNQ, :357-360)")
     if return_scores:
@@ -124,7 +155,7 @@ def triton_attention_mxfp4(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, al
         k = torch.nn.functional.pad(k, (0, 0, 0, 32))
         v = torch.nn.functional.pad(v, (0, 0, 0, 32))
     qq, qs, kq, ks, vq, vs = quantize_qkv(q, k, v)
-    out, lse = attention_mxfp4_forward(qq, kq, vq, qs, ks, vs, sm_scale=sm_scale, causal=causal, seqlen_k=seqlen_k)
+    out, lse = attention_mxfp4_forward(qq, kq, vq, qs, ks, vs, sm_scale=sm_scale, causal=causal, seqlen_k=seqlen_k, bias=bias, alibi_slopes=alibi_slopes)
     return out, lse, torch.empty([], device=q.device, dtype=torch.float32)
 
 

@@ -410,6 +410,19 @@ int alto_mxfp4_attention_fwd(const void* q_codes, const void* q_scales, const vo
                              int causal, void* stream);
 
 /*
+ * The same with the additive terms of triton_flash_attention_mxfp4.py:288-299 on the scaled scores, after the causal mask
+ * and before the running maximum:  S += bias[b][h][m][n]  (fp32; element at b bias_sb + h bias_sh + m bias_sm + n, strides
+ * in elements, 0 to broadcast over batch or heads, bias_sm % 4 == 0, 16-byte aligned; NULL: none; a bias of -inf hides a
+ * key) and the ALiBi term  S -= slope[b][h] * |m + Sk_used - Sq - n|  (fp32 slope at b alibi_sb + h alibi_sh; NULL: none).
+ * (The reference's kernel drops the batch offset of the bias, :630; here the strides say what is meant.)
+ */
+int alto_mxfp4_attention_fwd_ex(const void* q_codes, const void* q_scales, const void* k_codes, const void* k_scales,
+                                const void* vt_codes, const void* v_scales, void* out, float* lse, int64_t B, int64_t Hq,
+                                int64_t Hk, int64_t Sq, int64_t Sk, int64_t Sk_used, int64_t D, int64_t Dv, float sm_scale,
+                                int causal, const float* bias, int64_t bias_sb, int64_t bias_sh, int64_t bias_sm,
+                                const float* alibi_slopes, int64_t alibi_sb, int64_t alibi_sh, void* stream);
+
+/*
  * Fills out[0 .. n) with random 32-bit words for stochastic rounding: word 4 c + j is word j of Philox4x32-10 (Salmon et
  * al., SC'11) with the 128-bit counter c + offset and the 64-bit key `seed`.  The reference draws its bits inside its
  * kernel from the same generator family (tl.randint4x, alto/kernels/fp4/fp4_common/triton_fp4_ops.py:15-18) with

@@ -17,6 +17,9 @@ What pins it (the reference stores no vectors for this path; tests/test_oracle_a
 * agreement with fp32 softmax attention within the error MXFP4 operands allow (relative L2 below 0.3, cosine above 0.97 for N(0,1) inputs);
 * invariances the recurrence must have: a fully masked key block changes nothing; grouped-query heads equal repeated
   K/V heads.
+* the additive terms (``bias``, ``alibi_slopes``; the reference's CPU model has neither): a bias that is constant along
+  every row changes nothing beyond rounding (softmax is shift-invariant), a bias of -inf on a set of keys equals attention
+  without those keys, and ALiBi slopes equal the explicit bias tensor -slope |row + Sk - Sq - key|.
 The exponentials differ between CPU libm and the GPU's v_exp_f32 in the last bit, which can move a probability across
 an E2M1 rounding boundary: parity of the HIP kernel with this model is therefore a tolerance, not bit equality.
 """
@@ -39,7 +42,8 @@ def _qdq(x: torch.Tensor, is_2d_block: bool) -> torch.Tensor:
 
 
 def attention_fwd_ref(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, *, causal: bool, sm_scale: Optional[float] = None,
-                      pnq: bool = True, use_exp2: bool = True, block_n: int = BLOCK_N) -> Tuple[torch.Tensor, torch.Tensor]:
+                      pnq: bool = True, use_exp2: bool = True, block_n: int = BLOCK_N, bias: Optional[torch.Tensor] = None,
+                      alibi_slopes: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor]:
     """q [B, Hq, Sq, D], k [B, Hk, Sk, D], v [B, Hk, Sk, Dv] (bf16) -> (out bf16 [B, Hq, Sq, Dv], lse fp32 [B, Hq, Sq]).
 
     ``pnq=False`` takes the row sum from the unquantised probabilities (the behaviour the reference replaced; kept for
@@ -69,6 +73,13 @@ def attention_fwd_ref(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, *, caus
         if causal:
             masked = torch.arange(key0, key1)[None, :] > q_pos[:, None]
             s = s.masked_fill(masked, float("-inf"))
+        if bias is not None:                                                       # :288-291 (broadcast over batch / heads)
+            s = s + bias.float()[..., key0:key1]
+        if alibi_slopes is not None:                                               # :135-164,293-299
+            rel = (q_pos[:, None] - torch.arange(key0, key1)[None, :]).abs().float()
+            sl = alibi_slopes.float()
+            sl = sl[None, :] if sl.dim() == 1 else sl
+            s = s - sl[..., None, None] * rel
         m_ij = torch.maximum(m_i, s.amax(dim=-1))                                  # :308
         shifted = s - m_ij[..., None]
         p = torch.exp2(shifted * RCP_LN2) if use_exp2 else torch.exp(shifted)      # :318-322

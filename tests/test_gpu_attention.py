@@ -164,6 +164,48 @@ def test_layout_thd_is_the_attention_of_every_sequence(m, causal):
         assert _rel(o1.cpu(), ref) <= REL_L2 and float((l1.cpu() - ref_lse).abs().max()) <= 1e-4
 
 
+@pytest.mark.parametrize("case", [(2, 4, 2, 128, 256, 128, 128, True), (1, 2, 2, 96, 96, 64, 64, False), (1, 4, 1, 64, 192, 192, 128, True)],
+                         ids=lambda c: "x".join(map(str, c)))
+@pytest.mark.parametrize("terms", ["bias", "alibi", "both", "bias_per_head", "hide_keys"])
+def test_bias_and_alibi_match_the_cpu_model(m, case, terms):
+    """The additive score terms of the reference's kernel (:288-299): a full bias tensor, a bias broadcast over the batch,
+    ALiBi slopes per head, both together, and a bias of -inf that hides the second half of the keys of some rows."""
+    B, Hq, Hk, Sq, Sk, D, Dv, causal = case
+    q, k, v = _qkv(B, Hq, Hk, Sq, Sk, D, Dv, seed=sum(case) + len(terms))
+    g = torch.Generator().manual_seed(3)
+    bias = slopes = None
+    if terms in ("bias", "both"):
+        bias = torch.randn(B, Hq, Sq, Sk, generator=g)
+    if terms == "bias_per_head":
+        bias = torch.randn(1, Hq, Sq, Sk, generator=g)
+    if terms == "hide_keys":
+        bias = torch.zeros(1, 1, Sq, Sk)
+        bias[..., : Sq // 2, Sk // 2:] = float("-inf")     # (causal rows keep key 0 at least)
+    if terms in ("alibi", "both"):
+        slopes = 2.0 ** -(1 + torch.arange(Hq).float() % 4)
+    out, lse, _ = m.triton_attention_mxfp4(q.to(DEV), k.to(DEV), v.to(DEV), None if slopes is None else slopes.to(DEV),
+                                           None if bias is None else bias.to(DEV), D ** -0.5, 0.0, 0, 0, Sq, Sk, causal, False, True, "bhsd")
+    ref, ref_lse = attention_fwd_ref(q, k, v, causal=causal, bias=bias, alibi_slopes=slopes)
+    assert _rel(out.cpu(), ref) <= REL_L2
+    assert float((lse.cpu() - ref_lse).abs().max()) <= 1e-4
+    plain, _, _ = m.triton_attention_mxfp4(q.to(DEV), k.to(DEV), v.to(DEV), sm_scale=D ** -0.5, causal=causal)
+    assert not torch.equal(plain, out)
+
+
+def test_alibi_with_packed_sequences(m):
+    Hq, D = 2, 64
+    g = torch.Generator().manual_seed(4)
+    q = torch.randn(160, Hq, D, generator=g).to(torch.bfloat16)
+    k = torch.randn(160, Hq, D, generator=g).to(torch.bfloat16)
+    v = torch.randn(160, Hq, D, generator=g).to(torch.bfloat16)
+    slopes = torch.tensor([0.5, 0.125])
+    out, lse, _ = m.triton_attention_mxfp4(q.to(DEV), k.to(DEV), v.to(DEV), slopes.to(DEV), None, D ** -0.5, cu_seqlens_q=[0, 64, 160],
+                                           cu_seqlens_k=[0, 64, 160], causal=True, layout="thd")
+    for lo, hi in ((0, 64), (64, 160)):
+        ref, _ = attention_fwd_ref(*(t[lo:hi].transpose(0, 1).unsqueeze(0) for t in (q, k, v)), causal=True, alibi_slopes=slopes)
+        assert _rel(out[lo:hi].transpose(0, 1).unsqueeze(0).cpu(), ref) <= REL_L2
+
+
 def test_rejected_arguments(m):
     q, k, v = (t.to(DEV) for t in _qkv(1, 2, 2, 64, 64, 64, 64, seed=1))
     with pytest.raises(NotImplementedError):
@@ -176,8 +218,8 @@ def test_rejected_arguments(m):
                                  layout="thd")
     with pytest.raises(NotImplementedError):
         m.triton_attention_mxfp4(q, k, v, dropout_p=0.1)
-    with pytest.raises(NotImplementedError):
-        m.triton_attention_mxfp4(q, k, v, bias=torch.zeros(1, device=DEV))
+    with pytest.raises(RuntimeError, match="does not broadcast"):
+        m.triton_attention_mxfp4(q, k, v, bias=torch.zeros(3, 64, 64, device=DEV))
     with pytest.raises(AssertionError, match="Sq <= Sk"):
         m.triton_attention_mxfp4(q.repeat(1, 1, 2, 1), k, v, causal=True)
     qb, kb, vb = (t.to(DEV) for t in _qkv(1, 2, 2, 64, 80, 64, 64, seed=1))

@@ -134,3 +134,38 @@ def test_exp_and_exp2_forms_agree():
     b, lb = attention_fwd_ref(q, k, v, causal=True, use_exp2=False)
     assert float((a.float() - b.float()).norm() / b.float().norm()) < 2e-2
     assert float((la - lb).abs().max()) < 1e-3
+
+
+def test_additive_terms_of_the_scores():
+    """bias and ALiBi (triton_flash_attention_mxfp4.py:135-164,288-299), which the reference's CPU model does not have:
+    a bias constant along each row only shifts the row (same probabilities, lse moves by the constant), a -inf bias on a
+    set of keys is attention without them, and ALiBi slopes are the bias -slope |row + Sk - Sq - key|."""
+    torch.manual_seed(5)
+    B, H, Sq, Sk, D = 1, 2, 64, 128, 64
+    q = torch.randn(B, H, Sq, D, dtype=torch.bfloat16)
+    k = torch.randn(B, H, Sk, D, dtype=torch.bfloat16)
+    v = torch.randn(B, H, Sk, D, dtype=torch.bfloat16)
+    base, lse0 = attention_fwd_ref(q, k, v, causal=True)
+    # (1) per-row constant: powers of two times the natural-log unit would be exact; a general constant moves the fractional
+    # part of the maximum in the base-2 domain, so only closeness is claimed
+    c = torch.randn(B, H, Sq, 1)
+    shifted, lse1 = attention_fwd_ref(q, k, v, causal=True, bias=c.expand(B, H, Sq, Sk))
+    assert float((shifted.float() - base.float()).norm() / base.float().norm()) < 0.05
+    assert float((lse1 - lse0 - c[..., 0]).abs().max()) < 0.05
+    # (2) -inf on the second half of the keys == attention over the first half (whole blocks: nothing else changes)
+    hide = torch.zeros(1, 1, Sq, Sk)
+    hide[..., 64:] = float("-inf")
+    a, la = attention_fwd_ref(q, k, v, causal=False, bias=hide)
+    b, lb = attention_fwd_ref(q, k[:, :, :64], v[:, :, :64], causal=False)
+    assert torch.equal(a, b) and torch.equal(la, lb)
+    # (3) ALiBi slopes == the explicit bias (bottom-right aligned positions), per head
+    slopes = torch.tensor([0.25, 0.0625])
+    rel = ((torch.arange(Sq) + (Sk - Sq))[:, None] - torch.arange(Sk)[None, :]).abs().float()
+    explicit = -slopes[None, :, None, None] * rel[None, None]
+    a, la = attention_fwd_ref(q, k, v, causal=True, alibi_slopes=slopes)
+    b, lb = attention_fwd_ref(q, k, v, causal=True, bias=explicit)
+    assert torch.equal(a, b) and torch.equal(la, lb)
+    assert not torch.equal(a, base)
+    # and a slope of zero is no ALiBi at all
+    z, lz = attention_fwd_ref(q, k, v, causal=True, alibi_slopes=torch.zeros(2))
+    assert torch.equal(z, base) and torch.equal(lz, lse0)
