@@ -105,8 +105,12 @@ __device__ __forceinline__ float round_to_T(float v) {
 // Memory is addressed through buffer descriptors that start at the tile (32-bit per-lane offsets, row steps as scalar
 // offsets; an offset with bit 31 set is out of range: such a load returns zeros and such a store is dropped, which is
 // how rows past M and columns past C are masked).
-template <typename T, bool DO_ROW, bool DO_COL, int SR, bool RHT, bool B2D, bool GEN>
+// BPW: 32-row bands one workgroup walks (1, or 8 for 2D blocks with a column output: the workgroup then holds the eight
+// 16-byte pieces of a 128-byte line of every column's codes and stores whole lines, eight columns per wave instruction,
+// instead of one piece of 64 different lines per instruction).
+template <typename T, bool DO_ROW, bool DO_COL, int SR, bool RHT, bool B2D, bool GEN, int BPW = 1>
 __global__ __launch_bounds__(256) void quant_kernel(const QuantParams p) {
+  static_assert(BPW == 1 || (BPW == 8 && DO_COL && B2D), "bands per workgroup: 1, or 8 for the column output of 2D blocks");
   constexpr bool BF = sizeof(T) == 2;
   // Both phases consume the same random word per element.  Supplied words (SR == 1): each phase loads them in its own
   // layout, and the column phase's loads go out at the very start, beside the row phase's, so the second request for a
@@ -131,417 +135,474 @@ __global__ __launch_bounds__(256) void quant_kernel(const QuantParams p) {
 
   const int tid = threadIdx.x;
   const int M = p.M, C = p.C;
-  // Workgroup -> (column tile bx, 32-row band by).  With a column output the grid is one-dimensional per matrix: consecutive
+  // Workgroup -> (column tile bx, 32-row band by; with BPW > 1 "band" reads "row of BPW bands" below).  With a column
+  // output the grid is one-dimensional per matrix: consecutive
   // workgroups go to the 8 XCDs in turn, so 8 x 2^unit_shift consecutive ones are laid out as 8 XCDs (one unit = column tile
   // x group of 2^unit_shift bands each, neighbouring column tiles first) x the unit's consecutive bands.  The 16-byte pieces
   // that make up a 128-byte line of the column codes (8 bands), and the bytes of a line of plain column scales (128 bands),
   // are then written through one XCD's L2 within a short time of each other and leave it as whole lines (measured: 65536 x
   // 5760 in 260-300 us instead of 403).  Without a column output: (column tiles, bands).
   const int nby = (M + 31) >> 5;
-  int bx, by;
+  int bx, by0;   // column tile; first band of this workgroup
   if constexpr (DO_COL) {
+    // (the mapping above in units of workgroup rows of BPW bands)
     const unsigned wg = blockIdx.x, us = (unsigned)p.unit_shift;
     const unsigned unit = (wg >> (3 + us)) * 8 + (wg & 7), tiles_x = (unsigned)(C + TILE_C - 1) / TILE_C;
     bx = (int)(unit % tiles_x);
-    by = (int)(((unit / tiles_x) << us) + ((wg >> 3) & ((1u << us) - 1)));
-    if (by >= nby) return;   // (whole workgroup: padding of the last group of bands / of the units to a multiple of 8)
+    by0 = (int)(((unit / tiles_x) << us) + ((wg >> 3) & ((1u << us) - 1))) * BPW;
+    if (by0 >= nby) return;   // (whole workgroup: padding of the last group of bands / of the units to a multiple of 8)
   } else {
     bx = (int)blockIdx.x;
-    by = (int)blockIdx.y;
+    by0 = (int)blockIdx.y;
   }
   const int col0 = bx * TILE_C;
-  const int row0 = by * 32;
   const int64_t b = blockIdx.z;
 
   if (RHT || B2D) {
     if (tid < 32) sperm[tid] = (uint8_t)((p.perm4[tid >> 2] >> (8 * (tid & 3))) & 0xFFu);
-    if (tid < 8) blkmax[tid] = 0;
+    if (BPW == 1 && tid < 8) blkmax[tid] = 0;
     __syncthreads();
   }
-
-  const int rows_here = M - row0 < 32 ? M - row0 : 32;
-  const T* xt = reinterpret_cast<const T*>(p.x) + b * p.bs_x + (int64_t)row0 * p.ld_x;
-  const __amdgpu_buffer_rsrc_t rsrc_x = __builtin_amdgcn_make_buffer_rsrc(
-      const_cast<T*>(xt), 0, (int)(((int64_t)(rows_here - 1) * p.ld_x + C) * (int64_t)sizeof(T)), 0x00020000);
-  const uint32_t* rt_ = SR == 1 ? p.rand + b * p.bs_r + (int64_t)row0 * p.ld_r : nullptr;
-  const __amdgpu_buffer_rsrc_t rsrc_r = __builtin_amdgcn_make_buffer_rsrc(
-      const_cast<uint32_t*>(rt_), 0, SR == 1 ? (int)(((int64_t)(rows_here - 1) * p.ld_r + C) * 4) : 0, 0x00020000);
-  const int ldx_b = (int)p.ld_x * (int)sizeof(T), ldr_b = (int)p.ld_r * 4;   // row pitches in bytes
-
-  // Philox: element (b, i, j) consumes word ((b M + i) C + j) of the stream, i.e. word j % 4 of the block with the
-  // counter ctr0 + ((b M + i) C + j) / 4.  A lane owns 8 consecutive elements of a row = two blocks.
-  uint64_t key = 0, ctr0 = 0, qbase = 0;
-  if constexpr (SR == 2 || HW) {
-    key = p.philox_state ? p.philox_state[0] : p.seed;
-    ctr0 = p.philox_state ? p.philox_state[1] : p.ctr0;
-    qbase = ctr0 + (((uint64_t)b * (uint64_t)M + (uint64_t)row0) * (uint64_t)C >> 2);
-  }
-  const uint64_t band = (uint64_t)b * nby + by;   // hardware mode: index of this 32-row band
-
-  // ------------------------------------------------------------------ row phase
-  const int chunk = tid & 31, rsub = tid >> 5;
-  const int c = col0 + chunk * 8;
-  const bool cok = c < C;
-  uint32_t w[4][BF ? 4 : 8];
-  uint32_t rr[4][((SR == 1 || SR == 2) && (DO_ROW || STASH)) ? 8 : 1];
-  constexpr bool ROW_CODES = DO_ROW || XCODES;   // the row phase encodes (and stores, when DO_ROW)
-  uint32_t hw_row[4][(HW && ROW_CODES) ? (BF ? 1 : 4) : 1];
-  if constexpr (HW && ROW_CODES) {
-    const uint64_t call = (band * (uint64_t)(C >> 3) + (uint64_t)((col0 >> 3) + (tid & 31))) * 8 + (uint64_t)(tid >> 5);
-    if constexpr (BF) {
-      const uint64_t q = ctr0 + call;
-      const uint4 a = philox4x32_10(q, q < ctr0 ? 1ull : 0ull, key);
-      hw_row[0][0] = a.x; hw_row[1][0] = a.y; hw_row[2][0] = a.z; hw_row[3][0] = a.w;
-    } else {
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const uint64_t q = ctr0 + call * 4 + (uint64_t)i;
-        const uint4 a = philox4x32_10(q, q < ctr0 ? 1ull : 0ull, key);
-        hw_row[i][0] = a.x; hw_row[i][1] = a.y; hw_row[i][2] = a.z; hw_row[i][3] = a.w;
+  // column codes of the bands walked so far, oldest first (shifted down one place per band: static register indices)
+  uint32_t colacc[BPW > 1 ? BPW : 1][4];
+  int bands_done = 0;
+#pragma unroll 1
+  for (int bi = 0; bi < BPW; ++bi) {
+    const int by = by0 + bi;
+    if (BPW > 1) {
+      if (by >= nby) break;
+      __syncthreads();   // the previous band's column phase is done with the tile (and with blkmax)
+      if (B2D) {
+        if (tid < 8) blkmax[tid] = 0;
+        __syncthreads();
       }
     }
-  }
-  uint32_t amax_i[4];
-  bool valid[4];
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int r = rsub + 8 * i;
-    valid[i] = (row0 + r < M) && cok;
-    // rows past M are out of the descriptor's range and read as zeros; columns past C get an out-of-range offset
-    const int voff = valid[i] ? rsub * ldx_b + c * (int)sizeof(T) : OOB;
-    const v4i_t v0 = __builtin_amdgcn_raw_buffer_load_b128(rsrc_x, voff, 8 * i * ldx_b, 0);
-    w[i][0] = v0[0]; w[i][1] = v0[1]; w[i][2] = v0[2]; w[i][3] = v0[3];
-    if constexpr (!BF) {
-      const v4i_t v1 = __builtin_amdgcn_raw_buffer_load_b128(rsrc_x, voff, 8 * i * ldx_b + 16, 0);
-      w[i][4] = v1[0]; w[i][5] = v1[1]; w[i][6] = v1[2]; w[i][7] = v1[3];
+    const int row0 = by * 32;
+
+    const int rows_here = M - row0 < 32 ? M - row0 : 32;
+    const T* xt = reinterpret_cast<const T*>(p.x) + b * p.bs_x + (int64_t)row0 * p.ld_x;
+    const __amdgpu_buffer_rsrc_t rsrc_x = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<T*>(xt), 0, (int)(((int64_t)(rows_here - 1) * p.ld_x + C) * (int64_t)sizeof(T)), 0x00020000);
+    const uint32_t* rt_ = SR == 1 ? p.rand + b * p.bs_r + (int64_t)row0 * p.ld_r : nullptr;
+    const __amdgpu_buffer_rsrc_t rsrc_r = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint32_t*>(rt_), 0, SR == 1 ? (int)(((int64_t)(rows_here - 1) * p.ld_r + C) * 4) : 0, 0x00020000);
+    const int ldx_b = (int)p.ld_x * (int)sizeof(T), ldr_b = (int)p.ld_r * 4;   // row pitches in bytes
+
+    // Philox: element (b, i, j) consumes word ((b M + i) C + j) of the stream, i.e. word j % 4 of the block with the
+    // counter ctr0 + ((b M + i) C + j) / 4.  A lane owns 8 consecutive elements of a row = two blocks.
+    uint64_t key = 0, ctr0 = 0, qbase = 0;
+    if constexpr (SR == 2 || HW) {
+      key = p.philox_state ? p.philox_state[0] : p.seed;
+      ctr0 = p.philox_state ? p.philox_state[1] : p.ctr0;
+      qbase = ctr0 + (((uint64_t)b * (uint64_t)M + (uint64_t)row0) * (uint64_t)C >> 2);
     }
-    if constexpr (SR == 1 && (DO_ROW || STASH)) {
-      const int roff = valid[i] ? rsub * ldr_b + c * 4 : OOB;
-      const v4i_t r0 = __builtin_amdgcn_raw_buffer_load_b128(rsrc_r, roff, 8 * i * ldr_b, 0);
-      const v4i_t r1 = __builtin_amdgcn_raw_buffer_load_b128(rsrc_r, roff, 8 * i * ldr_b + 16, 0);
-      rr[i][0] = r0[0]; rr[i][1] = r0[1]; rr[i][2] = r0[2]; rr[i][3] = r0[3];
-      rr[i][4] = r1[0]; rr[i][5] = r1[1]; rr[i][6] = r1[2]; rr[i][7] = r1[3];
-    }
-  }
-  uint32_t rc[EARLY ? 32 : 1];
-  if constexpr (EARLY) {
-    const int cvoff = (col0 + tid < C) ? tid * 4 + col0 * 4 : OOB;
-#pragma unroll
-    for (int k = 0; k < 32; ++k) {
-      const int row = RHT ? packed_byte(p.pinv4, k) : k;
-      rc[k] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rsrc_r, cvoff, __builtin_amdgcn_readfirstlane(row * ldr_b), 0);
-    }
-  }
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int r = rsub + 8 * i;
-    if constexpr (SR == 2) {
-      const uint64_t q0 = qbase + (uint64_t)(uint32_t)((r * C + c) >> 2), q1 = q0 + 1;   // 128-bit counters: the carry goes up
-      const uint4 a = philox4x32_10(q0, q0 < ctr0 ? 1ull : 0ull, key);
-      const uint4 d = philox4x32_10(q1, q1 < ctr0 ? 1ull : 0ull, key);
-      rr[i][0] = a.x; rr[i][1] = a.y; rr[i][2] = a.z; rr[i][3] = a.w;
-      rr[i][4] = d.x; rr[i][5] = d.y; rr[i][6] = d.z; rr[i][7] = d.w;
-    }
-    if (DO_COL) {
-      const int pos = RHT ? sperm[r] : r;
-      uint4* dst = reinterpret_cast<uint4*>(&tile[pos * TILE_C + chunk * 8]);
-      dst[0] = make_uint4(w[i][0], w[i][1], w[i][2], w[i][3]);
-      if constexpr (!BF) dst[1] = make_uint4(w[i][4], w[i][5], w[i][6], w[i][7]);
-      if constexpr (STASH) {   // the word of row r waits at the position its element takes in the transform
-        uint4* sd = reinterpret_cast<uint4*>(&stash[pos * TILE_C + chunk * 8]);
-        sd[0] = make_uint4(rr[i][0], rr[i][1], rr[i][2], rr[i][3]);
-        sd[1] = make_uint4(rr[i][4], rr[i][5], rr[i][6], rr[i][7]);
-      }
-    }
-    if (DO_ROW || B2D) {
-      uint32_t a;
+    const uint64_t band = (uint64_t)b * nby + by;   // hardware mode: index of this 32-row band
+
+    // ------------------------------------------------------------------ row phase
+    const int chunk = tid & 31, rsub = tid >> 5;
+    const int c = col0 + chunk * 8;
+    const bool cok = c < C;
+    uint32_t w[4][BF ? 4 : 8];
+    uint32_t rr[4][((SR == 1 || SR == 2) && (DO_ROW || STASH)) ? 8 : 1];
+    constexpr bool ROW_CODES = DO_ROW || XCODES;   // the row phase encodes (and stores, when DO_ROW)
+    uint32_t hw_row[4][(HW && ROW_CODES) ? (BF ? 1 : 4) : 1];
+    if constexpr (HW && ROW_CODES) {
+      const uint64_t call = (band * (uint64_t)(C >> 3) + (uint64_t)((col0 >> 3) + (tid & 31))) * 8 + (uint64_t)(tid >> 5);
       if constexpr (BF) {
-        a = pk_max_u16(pk_max_u16(w[i][0] & 0x7FFF7FFFu, w[i][1] & 0x7FFF7FFFu),
-                       pk_max_u16(w[i][2] & 0x7FFF7FFFu, w[i][3] & 0x7FFF7FFFu));
-        a = max(a & 0xFFFFu, a >> 16);
+        const uint64_t q = ctr0 + call;
+        const uint4 a = philox4x32_10(q, q < ctr0 ? 1ull : 0ull, key);
+        hw_row[0][0] = a.x; hw_row[1][0] = a.y; hw_row[2][0] = a.z; hw_row[3][0] = a.w;
       } else {
-        a = 0;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) a = max(a, w[i][e] & 0x7FFFFFFFu);
-      }
-      a = max(a, dpp_u32<ALTO_DPP_QUAD_XOR1>(a));
-      a = max(a, dpp_u32<ALTO_DPP_QUAD_XOR2>(a));
-      amax_i[i] = a;
-      if (B2D && (tid & 3) == 0) atomicMax(&blkmax[chunk >> 2], a);
-    }
-  }
-  if (B2D || DO_COL) __syncthreads();
-
-  if (ROW_CODES || B2D) {
-    // descriptors of the row outputs start at the tile's first row
-    const __amdgpu_buffer_rsrc_t rsrc_rc = __builtin_amdgcn_make_buffer_rsrc(
-        DO_ROW ? p.row_codes + (b * M + row0) * p.ld_rc : nullptr, 0, DO_ROW ? 0x7FFFFFFF : 0, 0x00020000);
-    // Row scales, plain: [M][C/32], the byte of (row, group g) at row * (C/32) + g.  Packed (per matrix): the 16 groups of
-    // a row's 512-element block share 16 bytes, ((g / 16) M + row) 16 + packed_scale_pos(g % 16).  One store serves both:
-    // the row pitch and the lane's column term are chosen here, outside the loop.
-    // With 2D blocks the packed form repeats the block's scale for each of its 32 rows (the GEMM reads one layout).
-    const bool prs = DO_ROW && p.pack_rs;
-    const bool rs_rows = DO_ROW && (!B2D || prs);   // a scale byte per row goes out
-    const int ldrs = prs ? 16 : C / 32;
-    const int rs_col = prs ? ((c >> 9) * M) * 16 + packed_scale_pos((c >> 5) & 15) : (c >> 5);
-    const __amdgpu_buffer_rsrc_t rsrc_rs = __builtin_amdgcn_make_buffer_rsrc(
-        rs_rows ? p.row_scales + (prs ? (b * (int64_t)((C + 511) >> 9) * M + row0) * 16 : (b * M + row0) * (int64_t)(C / 32)) : nullptr, 0,
-        rs_rows ? 0x7FFFFFFF : 0, 0x00020000);
-    const int ldrc = (int)p.ld_rc;
-    if (prs && ((C >> 5) & 15) != 0 && col0 + TILE_C >= C) {   // packed: the groups of the last block beyond C read as 127
-      const bool last = (tid & 3) == 0 && (c >> 5) == (C >> 5) - 1;
-      for (int gp = (C >> 5) & 15; gp < 16; ++gp) {
-        const int off = rsub * 16 + ((c >> 9) * M) * 16 + packed_scale_pos(gp);
-#pragma unroll
-        for (int i = 0; i < 4; ++i) __builtin_amdgcn_raw_buffer_store_b8((uint8_t)127, rsrc_rs, (last && valid[i]) ? off : OOB, 8 * i * 16, 0);
+  #pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const uint64_t q = ctr0 + call * 4 + (uint64_t)i;
+          const uint4 a = philox4x32_10(q, q < ctr0 ? 1ull : 0ull, key);
+          hw_row[i][0] = a.x; hw_row[i][1] = a.y; hw_row[i][2] = a.z; hw_row[i][3] = a.w;
+        }
       }
     }
-    uint32_t blk = B2D ? blkmax[chunk >> 2] : 0;
-#pragma unroll
+    uint32_t amax_i[4];
+    bool valid[4];
+  #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const uint32_t a = B2D ? blk : amax_i[i];
-      uint32_t s;
-      if (GEN && p.uos) s = e8m0_uos(BF ? u2f(a << 16) : u2f(a));
-      else s = BF ? e8m0_from_bf16_bits(a) : e8m0_from_f32_bits(a);
-      // scales
-      if (!B2D || prs)   // (descriptor without range when no per-row byte is due)
-        __builtin_amdgcn_raw_buffer_store_b8((uint8_t)s, rsrc_rs, (valid[i] && (tid & 3) == 0) ? rsub * ldrs + rs_col : OOB, 8 * i * ldrs, 0);
-      if (B2D && i == 0 && rsub == 0 && (tid & 3) == 0 && valid[0]) {
-        if (DO_ROW && !prs) p.row_scales[(b * (M / 32) + by) * (C / 32) + (c >> 5)] = (uint8_t)s;
-        if (DO_COL && !p.pack_cs) p.col_scales[(b * (C / 32) + (c >> 5)) * (M / 32) + by] = (uint8_t)s;
+      const int r = rsub + 8 * i;
+      valid[i] = (row0 + r < M) && cok;
+      // rows past M are out of the descriptor's range and read as zeros; columns past C get an out-of-range offset
+      const int voff = valid[i] ? rsub * ldx_b + c * (int)sizeof(T) : OOB;
+      const v4i_t v0 = __builtin_amdgcn_raw_buffer_load_b128(rsrc_x, voff, 8 * i * ldx_b, 0);
+      w[i][0] = v0[0]; w[i][1] = v0[1]; w[i][2] = v0[2]; w[i][3] = v0[3];
+      if constexpr (!BF) {
+        const v4i_t v1 = __builtin_amdgcn_raw_buffer_load_b128(rsrc_x, voff, 8 * i * ldx_b + 16, 0);
+        w[i][4] = v1[0]; w[i][5] = v1[1]; w[i][6] = v1[2]; w[i][7] = v1[3];
       }
-      if constexpr (ROW_CODES) {
-      const float scale_f = u2f(s << 23);
-      float v[8];
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        if constexpr (BF) v[e] = (e & 1) ? bf16_hi(w[i][e >> 1]) : bf16_lo(w[i][e >> 1]);
-        else v[e] = u2f(w[i][e]);
-        if (GEN && p.clip_row) v[e] = round_to_T<T>(v[e] * 0.75f);
-      }
-      uint32_t out = 0;
-      if constexpr (SR == 0) {
-        out = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(out, v[0], v[1], scale_f, 0);
-        out = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(out, v[2], v[3], scale_f, 1);
-        out = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(out, v[4], v[5], scale_f, 2);
-        out = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(out, v[6], v[7], scale_f, 3);
-      } else if constexpr (HW) {
-        uint32_t by[4];   // byte 0 of each result holds the pair's two codes; the other bytes are not defined
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          if constexpr (BF) {
-            const uint32_t src = (GEN && p.clip_row) ? pack_bf16x2(v[2 * e], v[2 * e + 1]) : w[i][e];
-            by[e] = __builtin_amdgcn_cvt_scalef32_sr_pk_fp4_bf16(0u, __builtin_bit_cast(bf16x2_t, src), hw_row[i][0] << (8 * e), scale_f, 0);
-          } else {
-            by[e] = __builtin_amdgcn_cvt_scalef32_sr_pk_fp4_f32(0u, f2_t{v[2 * e], v[2 * e + 1]}, hw_row[i][e], scale_f, 0);
-          }
-        }
-        out = __builtin_amdgcn_perm(by[1], by[0], 0x0C0C0400u) | __builtin_amdgcn_perm(by[3], by[2], 0x04000C0Cu);
-      } else {
-        const float inv = u2f((254u - s) << 23);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          const float q = v[e] * inv;
-          const uint32_t code = e2m1_sr_mag(q, rr[i][e]) | ((f2u(q) >> 28) & 8u);
-          out |= code << (4 * e);
-        }
-      }
-      if constexpr (DO_ROW) __builtin_amdgcn_raw_buffer_store_b32(out, rsrc_rc, valid[i] ? rsub * ldrc + (c >> 1) : OOB, 8 * i * ldrc, 0);
-      if constexpr (XCODES) {   // one code per byte, in column order, for the column packing
-        const uint32_t ev = out & 0x0F0F0F0Fu, od = (out >> 4) & 0x0F0F0F0Fu;
-        uint2 two;
-        two.x = __builtin_amdgcn_perm(od, ev, 0x05010400u);
-        two.y = __builtin_amdgcn_perm(od, ev, 0x07030602u);
-        *reinterpret_cast<uint2*>(&xcodes[(rsub + 8 * i) * TILE_C + chunk * 8]) = two;
-      }
+      if constexpr (SR == 1 && (DO_ROW || STASH)) {
+        const int roff = valid[i] ? rsub * ldr_b + c * 4 : OOB;
+        const v4i_t r0 = __builtin_amdgcn_raw_buffer_load_b128(rsrc_r, roff, 8 * i * ldr_b, 0);
+        const v4i_t r1 = __builtin_amdgcn_raw_buffer_load_b128(rsrc_r, roff, 8 * i * ldr_b + 16, 0);
+        rr[i][0] = r0[0]; rr[i][1] = r0[1]; rr[i][2] = r0[2]; rr[i][3] = r0[3];
+        rr[i][4] = r1[0]; rr[i][5] = r1[1]; rr[i][6] = r1[2]; rr[i][7] = r1[3];
       }
     }
-  }
-
-  // ------------------------------------------------------------------ column phase
-  if (DO_COL) {
-    const int cc = col0 + tid;
-    const bool cvalid = cc < C;
-    float z[32];
-    uint32_t zp[(BF && RHT) ? 16 : 1];   // the transformed column as packed bf16 pairs
-#pragma unroll
-    for (int k = 0; k < 32; ++k) {
-      if (BF) z[k] = u2f((uint32_t)reinterpret_cast<const unsigned short*>(tile)[k * TILE_C + tid] << 16);
-      else z[k] = reinterpret_cast<const float*>(tile)[k * TILE_C + tid];
-    }
-    if (RHT) {
-      __syncthreads();   // every thread holds its column: the tile's memory becomes the byte scratch used further down
-#pragma unroll
-      for (int h = 1; h < 32; h <<= 1) {
-#pragma unroll
-        for (int k = 0; k < 32; ++k) {
-          if ((k & h) == 0) {
-            float a0 = z[k], a1 = z[k + h];
-            z[k] = a0 + a1;
-            z[k + h] = a0 - a1;
-          }
-        }
-      }
-      // z * (+-1) / float32(sqrt(32)), correctly rounded: quotient estimate, one FMA correction, both with the sign
-      // folded into the (wave-uniform) constants; the sign bit is taken from the estimate so that -0 stays -0.
-      // (Taking the block's absmax before the division and dropping the guard for columns without an infinity was
-      // measured: the second copy of the loop costs more than the 32 guards save.)
-#pragma unroll
+    uint32_t rc[EARLY ? 32 : 1];
+    if constexpr (EARLY) {
+      const int cvoff = (col0 + tid < C) ? tid * 4 + col0 * 4 : OOB;
+  #pragma unroll
       for (int k = 0; k < 32; ++k) {
-        const uint32_t flip = ((p.sign_mask >> k) & 1u) << 31;   // scalar: the constants stay in scalar registers
-        const float ck = u2f(f2u(5.656854152679443f) ^ flip);
-        const float rck = u2f(f2u(0.17677669529663689f) ^ flip);
-        const float q = z[k] * rck;
-        float r = __builtin_fmaf(-q, ck, z[k]);
-        r = __builtin_fmaxf(r, -3.0e38f);   // z = +-inf gives r = NaN: drop it so that the quotient stays +-inf
-        z[k] = u2f((f2u(__builtin_fmaf(r, rck, q)) & 0x7FFFFFFFu) | (f2u(q) & 0x80000000u));
+        const int row = RHT ? packed_byte(p.pinv4, k) : k;
+        rc[k] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rsrc_r, cvoff, __builtin_amdgcn_readfirstlane(row * ldr_b), 0);
       }
-      if constexpr (BF) {   // round to bf16 two at a time
-#pragma unroll
-        for (int k = 0; k < 32; k += 2) {
-          zp[k >> 1] = pack_bf16x2(z[k], z[k + 1]);   // the hardware convert takes the packed pairs as they are
-          z[k] = u2f(zp[k >> 1] << 16);
-          z[k + 1] = u2f(zp[k >> 1] & 0xFFFF0000u);
+    }
+  #pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int r = rsub + 8 * i;
+      if constexpr (SR == 2) {
+        const uint64_t q0 = qbase + (uint64_t)(uint32_t)((r * C + c) >> 2), q1 = q0 + 1;   // 128-bit counters: the carry goes up
+        const uint4 a = philox4x32_10(q0, q0 < ctr0 ? 1ull : 0ull, key);
+        const uint4 d = philox4x32_10(q1, q1 < ctr0 ? 1ull : 0ull, key);
+        rr[i][0] = a.x; rr[i][1] = a.y; rr[i][2] = a.z; rr[i][3] = a.w;
+        rr[i][4] = d.x; rr[i][5] = d.y; rr[i][6] = d.z; rr[i][7] = d.w;
+      }
+      if (DO_COL) {
+        const int pos = RHT ? sperm[r] : r;
+        uint4* dst = reinterpret_cast<uint4*>(&tile[pos * TILE_C + chunk * 8]);
+        dst[0] = make_uint4(w[i][0], w[i][1], w[i][2], w[i][3]);
+        if constexpr (!BF) dst[1] = make_uint4(w[i][4], w[i][5], w[i][6], w[i][7]);
+        if constexpr (STASH) {   // the word of row r waits at the position its element takes in the transform
+          uint4* sd = reinterpret_cast<uint4*>(&stash[pos * TILE_C + chunk * 8]);
+          sd[0] = make_uint4(rr[i][0], rr[i][1], rr[i][2], rr[i][3]);
+          sd[1] = make_uint4(rr[i][4], rr[i][5], rr[i][6], rr[i][7]);
         }
       }
-    }
-    uint32_t s;
-    if (B2D) {
-      uint32_t a = blkmax[tid >> 5];
-      if (GEN && p.uos) s = e8m0_uos(BF ? u2f(a << 16) : u2f(a));
-      else s = BF ? e8m0_from_bf16_bits(a) : e8m0_from_f32_bits(a);
-    } else {
-      float am = 0.0f;
-#pragma unroll
-      for (int k = 0; k < 32; k += 2) am = __builtin_fmaxf(__builtin_fmaxf(am, __builtin_fabsf(z[k])), __builtin_fabsf(z[k + 1]));
-      if (GEN && p.uos) s = e8m0_uos(am);
-      else s = BF ? e8m0_from_bf16_bits(f2u(am) >> 16) : e8m0_from_f32_bits(f2u(am));
-    }
-    // Column scales, plain 1D: [C][M/32], this band's byte of column cc at cc (M/32) + band (2D blocks: the row phase wrote
-    // the block's byte).  Packed (per matrix, 1D or 2D blocks): ((band / 16) C + cc) 16 + packed_scale_pos(band % 16); the
-    // last band also writes the 127s of the groups beyond M.
-    {
-      const bool pcs = p.pack_cs;
-      const int cs_pitch = pcs ? 16 : M / 32;
-      const uint8_t* cs_blk = p.col_scales + ((b * (int64_t)((M + 511) >> 9) + (by >> 4)) * C + col0) * 16;
-      const __amdgpu_buffer_rsrc_t rsrc_cs = __builtin_amdgcn_make_buffer_rsrc(
-          const_cast<uint8_t*>(pcs ? cs_blk + packed_scale_pos(by & 15) : p.col_scales + (b * C + col0) * (int64_t)(M / 32) + by), 0, 0x7FFFFFFF, 0x00020000);
-      if (!B2D || pcs) __builtin_amdgcn_raw_buffer_store_b8((uint8_t)s, rsrc_cs, cvalid ? tid * cs_pitch : OOB, 0, 0);
-      if (pcs && by == (M >> 5) - 1 && ((M >> 5) & 15) != 0) {
-        const __amdgpu_buffer_rsrc_t rsrc_pad = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(cs_blk), 0, 0x7FFFFFFF, 0x00020000);
-        for (int gp = (M >> 5) & 15; gp < 16; ++gp)
-          __builtin_amdgcn_raw_buffer_store_b8((uint8_t)127, rsrc_pad, cvalid ? tid * 16 + packed_scale_pos(gp) : OOB, 0, 0);
+      if (DO_ROW || B2D) {
+        uint32_t a;
+        if constexpr (BF) {
+          a = pk_max_u16(pk_max_u16(w[i][0] & 0x7FFF7FFFu, w[i][1] & 0x7FFF7FFFu),
+                         pk_max_u16(w[i][2] & 0x7FFF7FFFu, w[i][3] & 0x7FFF7FFFu));
+          a = max(a & 0xFFFFu, a >> 16);
+        } else {
+          a = 0;
+  #pragma unroll
+          for (int e = 0; e < 8; ++e) a = max(a, w[i][e] & 0x7FFFFFFFu);
+        }
+        a = max(a, dpp_u32<ALTO_DPP_QUAD_XOR1>(a));
+        a = max(a, dpp_u32<ALTO_DPP_QUAD_XOR2>(a));
+        amax_i[i] = a;
+        if (B2D && (tid & 3) == 0) atomicMax(&blkmax[chunk >> 2], a);
       }
     }
-    const float scale_f = u2f(s << 23);
-    const float inv = u2f((254u - s) << 23);
-    uint32_t codes[32];
-    uint32_t out[4];
-    if constexpr (HW && B2D) {
-      // 2D blocks have one set of codes: the row phase left them in LDS, one per byte
-      __syncthreads();
-#pragma unroll
-      for (int k = 0; k < 32; ++k) codes[k] = xcodes[k * TILE_C + tid];
-    } else if constexpr (HW) {
-      // transformed values back to row order (a private strip in LDS undoes the permutation), then one hardware
-      // convert per pair of rows
-      if (GEN && p.clip_col) {
-#pragma unroll
-        for (int k = 0; k < 32; ++k) z[k] = round_to_T<T>(z[k] * 0.75f);
+    if (B2D || DO_COL) __syncthreads();
+
+    if (ROW_CODES || B2D) {
+      // descriptors of the row outputs start at the tile's first row
+      const __amdgpu_buffer_rsrc_t rsrc_rc = __builtin_amdgcn_make_buffer_rsrc(
+          DO_ROW ? p.row_codes + (b * M + row0) * p.ld_rc : nullptr, 0, DO_ROW ? 0x7FFFFFFF : 0, 0x00020000);
+      // Row scales, plain: [M][C/32], the byte of (row, group g) at row * (C/32) + g.  Packed (per matrix): the 16 groups of
+      // a row's 512-element block share 16 bytes, ((g / 16) M + row) 16 + packed_scale_pos(g % 16).  One store serves both:
+      // the row pitch and the lane's column term are chosen here, outside the loop.
+      // With 2D blocks the packed form repeats the block's scale for each of its 32 rows (the GEMM reads one layout).
+      const bool prs = DO_ROW && p.pack_rs;
+      const bool rs_rows = DO_ROW && (!B2D || prs);   // a scale byte per row goes out
+      const int ldrs = prs ? 16 : C / 32;
+      const int rs_col = prs ? ((c >> 9) * M) * 16 + packed_scale_pos((c >> 5) & 15) : (c >> 5);
+      const __amdgpu_buffer_rsrc_t rsrc_rs = __builtin_amdgcn_make_buffer_rsrc(
+          rs_rows ? p.row_scales + (prs ? (b * (int64_t)((C + 511) >> 9) * M + row0) * 16 : (b * M + row0) * (int64_t)(C / 32)) : nullptr, 0,
+          rs_rows ? 0x7FFFFFFF : 0, 0x00020000);
+      const int ldrc = (int)p.ld_rc;
+      if (prs && ((C >> 5) & 15) != 0 && col0 + TILE_C >= C) {   // packed: the groups of the last block beyond C read as 127
+        const bool last = (tid & 3) == 0 && (c >> 5) == (C >> 5) - 1;
+        for (int gp = (C >> 5) & 15; gp < 16; ++gp) {
+          const int off = rsub * 16 + ((c >> 9) * M) * 16 + packed_scale_pos(gp);
+  #pragma unroll
+          for (int i = 0; i < 4; ++i) __builtin_amdgcn_raw_buffer_store_b8((uint8_t)127, rsrc_rs, (last && valid[i]) ? off : OOB, 8 * i * 16, 0);
+        }
       }
-      uint32_t* strip = reinterpret_cast<uint32_t*>(tile) + tid * STRIP;
-      const uint64_t nrow = (uint64_t)gridDim.z * nby * (uint64_t)C;   // calls of the row copy: batch * bands * C
-      uint32_t by[16];
-      if constexpr (BF) {
-        uint32_t pr[16];
-#pragma unroll
-        for (int j = 0; j < 16; ++j) pr[j] = (RHT && !(GEN && p.clip_col)) ? zp[RHT ? j : 0] : pack_bf16x2(z[2 * j], z[2 * j + 1]);
-        if (RHT) {
-          unsigned short* s16 = reinterpret_cast<unsigned short*>(strip);
-#pragma unroll
-          for (int j = 0; j < 16; ++j) {
-            s16[packed_byte(p.pinv4, 2 * j)] = (unsigned short)pr[j];
-            s16[packed_byte(p.pinv4, 2 * j + 1)] = (unsigned short)(pr[j] >> 16);
+      uint32_t blk = B2D ? blkmax[chunk >> 2] : 0;
+  #pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const uint32_t a = B2D ? blk : amax_i[i];
+        uint32_t s;
+        if (GEN && p.uos) s = e8m0_uos(BF ? u2f(a << 16) : u2f(a));
+        else s = BF ? e8m0_from_bf16_bits(a) : e8m0_from_f32_bits(a);
+        // scales
+        if (!B2D || prs)   // (descriptor without range when no per-row byte is due)
+          __builtin_amdgcn_raw_buffer_store_b8((uint8_t)s, rsrc_rs, (valid[i] && (tid & 3) == 0) ? rsub * ldrs + rs_col : OOB, 8 * i * ldrs, 0);
+        if (B2D && i == 0 && rsub == 0 && (tid & 3) == 0 && valid[0]) {
+          if (DO_ROW && !prs) p.row_scales[(b * (M / 32) + by) * (C / 32) + (c >> 5)] = (uint8_t)s;
+          if (DO_COL && !p.pack_cs) p.col_scales[(b * (C / 32) + (c >> 5)) * (M / 32) + by] = (uint8_t)s;
+        }
+        if constexpr (ROW_CODES) {
+        const float scale_f = u2f(s << 23);
+        float v[8];
+  #pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          if constexpr (BF) v[e] = (e & 1) ? bf16_hi(w[i][e >> 1]) : bf16_lo(w[i][e >> 1]);
+          else v[e] = u2f(w[i][e]);
+          if (GEN && p.clip_row) v[e] = round_to_T<T>(v[e] * 0.75f);
+        }
+        uint32_t out = 0;
+        if constexpr (SR == 0) {
+          out = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(out, v[0], v[1], scale_f, 0);
+          out = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(out, v[2], v[3], scale_f, 1);
+          out = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(out, v[4], v[5], scale_f, 2);
+          out = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(out, v[6], v[7], scale_f, 3);
+        } else if constexpr (HW) {
+          uint32_t by[4];   // byte 0 of each result holds the pair's two codes; the other bytes are not defined
+  #pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            if constexpr (BF) {
+              const uint32_t src = (GEN && p.clip_row) ? pack_bf16x2(v[2 * e], v[2 * e + 1]) : w[i][e];
+              by[e] = __builtin_amdgcn_cvt_scalef32_sr_pk_fp4_bf16(0u, __builtin_bit_cast(bf16x2_t, src), hw_row[i][0] << (8 * e), scale_f, 0);
+            } else {
+              by[e] = __builtin_amdgcn_cvt_scalef32_sr_pk_fp4_f32(0u, f2_t{v[2 * e], v[2 * e + 1]}, hw_row[i][e], scale_f, 0);
+            }
           }
-          asm volatile("" ::: "memory");   // same thread reads what it wrote: LDS ops of one wave complete in order
-#pragma unroll
-          for (int j = 0; j < 16; ++j) pr[j] = strip[j];
+          out = __builtin_amdgcn_perm(by[1], by[0], 0x0C0C0400u) | __builtin_amdgcn_perm(by[3], by[2], 0x04000C0Cu);
+        } else {
+          const float inv = u2f((254u - s) << 23);
+  #pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            const float q = v[e] * inv;
+            const uint32_t code = e2m1_sr_mag(q, rr[i][e]) | ((f2u(q) >> 28) & 8u);
+            out |= code << (4 * e);
+          }
         }
-        const uint64_t q = ctr0 + nrow + band * (uint64_t)C + (uint64_t)cc;
-        const uint4 a = philox4x32_10(q, q < ctr0 ? 1ull : 0ull, key);
-        const uint32_t wd[4] = {a.x, a.y, a.z, a.w};
-#pragma unroll
-        for (int j = 0; j < 16; ++j)
-          by[j] = __builtin_amdgcn_cvt_scalef32_sr_pk_fp4_bf16(0u, __builtin_bit_cast(bf16x2_t, pr[j]), wd[j >> 2] << (8 * (j & 3)), scale_f, 0);
+        if constexpr (DO_ROW) __builtin_amdgcn_raw_buffer_store_b32(out, rsrc_rc, valid[i] ? rsub * ldrc + (c >> 1) : OOB, 8 * i * ldrc, 0);
+        if constexpr (XCODES) {   // one code per byte, in column order, for the column packing
+          const uint32_t ev = out & 0x0F0F0F0Fu, od = (out >> 4) & 0x0F0F0F0Fu;
+          uint2 two;
+          two.x = __builtin_amdgcn_perm(od, ev, 0x05010400u);
+          two.y = __builtin_amdgcn_perm(od, ev, 0x07030602u);
+          *reinterpret_cast<uint2*>(&xcodes[(rsub + 8 * i) * TILE_C + chunk * 8]) = two;
+        }
+        }
+      }
+    }
+
+    // ------------------------------------------------------------------ column phase
+    if (DO_COL) {
+      const int cc = col0 + tid;
+      const bool cvalid = cc < C;
+      float z[32];
+      uint32_t zp[(BF && RHT) ? 16 : 1];   // the transformed column as packed bf16 pairs
+  #pragma unroll
+      for (int k = 0; k < 32; ++k) {
+        if (BF) z[k] = u2f((uint32_t)reinterpret_cast<const unsigned short*>(tile)[k * TILE_C + tid] << 16);
+        else z[k] = reinterpret_cast<const float*>(tile)[k * TILE_C + tid];
+      }
+      if (RHT) {
+        __syncthreads();   // every thread holds its column: the tile's memory becomes the byte scratch used further down
+  #pragma unroll
+        for (int h = 1; h < 32; h <<= 1) {
+  #pragma unroll
+          for (int k = 0; k < 32; ++k) {
+            if ((k & h) == 0) {
+              float a0 = z[k], a1 = z[k + h];
+              z[k] = a0 + a1;
+              z[k + h] = a0 - a1;
+            }
+          }
+        }
+        // z * (+-1) / float32(sqrt(32)), correctly rounded: quotient estimate, one FMA correction, both with the sign
+        // folded into the (wave-uniform) constants; the sign bit is taken from the estimate so that -0 stays -0.
+        // (Taking the block's absmax before the division and dropping the guard for columns without an infinity was
+        // measured: the second copy of the loop costs more than the 32 guards save.)
+  #pragma unroll
+        for (int k = 0; k < 32; ++k) {
+          const uint32_t flip = ((p.sign_mask >> k) & 1u) << 31;   // scalar: the constants stay in scalar registers
+          const float ck = u2f(f2u(5.656854152679443f) ^ flip);
+          const float rck = u2f(f2u(0.17677669529663689f) ^ flip);
+          const float q = z[k] * rck;
+          float r = __builtin_fmaf(-q, ck, z[k]);
+          r = __builtin_fmaxf(r, -3.0e38f);   // z = +-inf gives r = NaN: drop it so that the quotient stays +-inf
+          z[k] = u2f((f2u(__builtin_fmaf(r, rck, q)) & 0x7FFFFFFFu) | (f2u(q) & 0x80000000u));
+        }
+        if constexpr (BF) {   // round to bf16 two at a time
+  #pragma unroll
+          for (int k = 0; k < 32; k += 2) {
+            zp[k >> 1] = pack_bf16x2(z[k], z[k + 1]);   // the hardware convert takes the packed pairs as they are
+            z[k] = u2f(zp[k >> 1] << 16);
+            z[k + 1] = u2f(zp[k >> 1] & 0xFFFF0000u);
+          }
+        }
+      }
+      uint32_t s;
+      if (B2D) {
+        uint32_t a = blkmax[tid >> 5];
+        if (GEN && p.uos) s = e8m0_uos(BF ? u2f(a << 16) : u2f(a));
+        else s = BF ? e8m0_from_bf16_bits(a) : e8m0_from_f32_bits(a);
       } else {
-        if (RHT) {
-          float* sf = reinterpret_cast<float*>(strip);
-#pragma unroll
-          for (int k = 0; k < 32; ++k) sf[packed_byte(p.pinv4, k)] = z[k];
-          asm volatile("" ::: "memory");
-#pragma unroll
-          for (int k = 0; k < 32; ++k) z[k] = sf[k];
+        float am = 0.0f;
+  #pragma unroll
+        for (int k = 0; k < 32; k += 2) am = __builtin_fmaxf(__builtin_fmaxf(am, __builtin_fabsf(z[k])), __builtin_fabsf(z[k + 1]));
+        if (GEN && p.uos) s = e8m0_uos(am);
+        else s = BF ? e8m0_from_bf16_bits(f2u(am) >> 16) : e8m0_from_f32_bits(f2u(am));
+      }
+      // Column scales, plain 1D: [C][M/32], this band's byte of column cc at cc (M/32) + band (2D blocks: the row phase wrote
+      // the block's byte).  Packed (per matrix, 1D or 2D blocks): ((band / 16) C + cc) 16 + packed_scale_pos(band % 16); the
+      // last band also writes the 127s of the groups beyond M.
+      {
+        const bool pcs = p.pack_cs;
+        const int cs_pitch = pcs ? 16 : M / 32;
+        const uint8_t* cs_blk = p.col_scales + ((b * (int64_t)((M + 511) >> 9) + (by >> 4)) * C + col0) * 16;
+        const __amdgpu_buffer_rsrc_t rsrc_cs = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<uint8_t*>(pcs ? cs_blk + packed_scale_pos(by & 15) : p.col_scales + (b * C + col0) * (int64_t)(M / 32) + by), 0, 0x7FFFFFFF, 0x00020000);
+        if (!B2D || pcs) __builtin_amdgcn_raw_buffer_store_b8((uint8_t)s, rsrc_cs, cvalid ? tid * cs_pitch : OOB, 0, 0);
+        if (pcs && by == (M >> 5) - 1 && ((M >> 5) & 15) != 0) {
+          const __amdgpu_buffer_rsrc_t rsrc_pad = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(cs_blk), 0, 0x7FFFFFFF, 0x00020000);
+          for (int gp = (M >> 5) & 15; gp < 16; ++gp)
+            __builtin_amdgcn_raw_buffer_store_b8((uint8_t)127, rsrc_pad, cvalid ? tid * 16 + packed_scale_pos(gp) : OOB, 0, 0);
         }
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          const uint64_t q = ctr0 + 4 * nrow + (band * (uint64_t)C + (uint64_t)cc) * 4 + (uint64_t)g;
+      }
+      const float scale_f = u2f(s << 23);
+      const float inv = u2f((254u - s) << 23);
+      uint32_t codes[32];
+      uint32_t out[4];
+      if constexpr (HW && B2D) {
+        // 2D blocks have one set of codes: the row phase left them in LDS, one per byte
+        __syncthreads();
+  #pragma unroll
+        for (int k = 0; k < 32; ++k) codes[k] = xcodes[k * TILE_C + tid];
+      } else if constexpr (HW) {
+        // transformed values back to row order (a private strip in LDS undoes the permutation), then one hardware
+        // convert per pair of rows
+        if (GEN && p.clip_col) {
+  #pragma unroll
+          for (int k = 0; k < 32; ++k) z[k] = round_to_T<T>(z[k] * 0.75f);
+        }
+        uint32_t* strip = reinterpret_cast<uint32_t*>(tile) + tid * STRIP;
+        const uint64_t nrow = (uint64_t)gridDim.z * nby * (uint64_t)C;   // calls of the row copy: batch * bands * C
+        uint32_t by[16];
+        if constexpr (BF) {
+          uint32_t pr[16];
+  #pragma unroll
+          for (int j = 0; j < 16; ++j) pr[j] = (RHT && !(GEN && p.clip_col)) ? zp[RHT ? j : 0] : pack_bf16x2(z[2 * j], z[2 * j + 1]);
+          if (RHT) {
+            unsigned short* s16 = reinterpret_cast<unsigned short*>(strip);
+  #pragma unroll
+            for (int j = 0; j < 16; ++j) {
+              s16[packed_byte(p.pinv4, 2 * j)] = (unsigned short)pr[j];
+              s16[packed_byte(p.pinv4, 2 * j + 1)] = (unsigned short)(pr[j] >> 16);
+            }
+            asm volatile("" ::: "memory");   // same thread reads what it wrote: LDS ops of one wave complete in order
+  #pragma unroll
+            for (int j = 0; j < 16; ++j) pr[j] = strip[j];
+          }
+          const uint64_t q = ctr0 + nrow + band * (uint64_t)C + (uint64_t)cc;
           const uint4 a = philox4x32_10(q, q < ctr0 ? 1ull : 0ull, key);
           const uint32_t wd[4] = {a.x, a.y, a.z, a.w};
-#pragma unroll
-          for (int e = 0; e < 4; ++e)
-            by[4 * g + e] = __builtin_amdgcn_cvt_scalef32_sr_pk_fp4_f32(0u, f2_t{z[8 * g + 2 * e], z[8 * g + 2 * e + 1]}, wd[e], scale_f, 0);
+  #pragma unroll
+          for (int j = 0; j < 16; ++j)
+            by[j] = __builtin_amdgcn_cvt_scalef32_sr_pk_fp4_bf16(0u, __builtin_bit_cast(bf16x2_t, pr[j]), wd[j >> 2] << (8 * (j & 3)), scale_f, 0);
+        } else {
+          if (RHT) {
+            float* sf = reinterpret_cast<float*>(strip);
+  #pragma unroll
+            for (int k = 0; k < 32; ++k) sf[packed_byte(p.pinv4, k)] = z[k];
+            asm volatile("" ::: "memory");
+  #pragma unroll
+            for (int k = 0; k < 32; ++k) z[k] = sf[k];
+          }
+  #pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            const uint64_t q = ctr0 + 4 * nrow + (band * (uint64_t)C + (uint64_t)cc) * 4 + (uint64_t)g;
+            const uint4 a = philox4x32_10(q, q < ctr0 ? 1ull : 0ull, key);
+            const uint32_t wd[4] = {a.x, a.y, a.z, a.w};
+  #pragma unroll
+            for (int e = 0; e < 4; ++e)
+              by[4 * g + e] = __builtin_amdgcn_cvt_scalef32_sr_pk_fp4_f32(0u, f2_t{z[8 * g + 2 * e], z[8 * g + 2 * e + 1]}, wd[e], scale_f, 0);
+          }
+        }
+  #pragma unroll
+        for (int j = 0; j < 4; ++j)
+          out[j] = __builtin_amdgcn_perm(by[4 * j + 1], by[4 * j], 0x0C0C0400u) | __builtin_amdgcn_perm(by[4 * j + 3], by[4 * j + 2], 0x04000C0Cu);
+      }
+      if constexpr (!HW) {
+  #pragma unroll
+      for (int k = 0; k < 32; ++k) {
+        float v = z[k];
+        if (GEN && p.clip_col) v = round_to_T<T>(v * 0.75f);
+        if constexpr (SR == 0) {
+          codes[k] = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(0u, v, 0.0f, scale_f, 0) & 0xFu;
+        } else {
+          uint32_t r;
+          if constexpr (EARLY) r = rc[k];
+          else r = stash[k * TILE_C + tid];
+          const float q = v * inv;
+          codes[k] = e2m1_sr_mag(q, r) | ((f2u(q) >> 28) & 8u);
         }
       }
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-        out[j] = __builtin_amdgcn_perm(by[4 * j + 1], by[4 * j], 0x0C0C0400u) | __builtin_amdgcn_perm(by[4 * j + 3], by[4 * j + 2], 0x04000C0Cu);
-    }
-    if constexpr (!HW) {
-#pragma unroll
-    for (int k = 0; k < 32; ++k) {
-      float v = z[k];
-      if (GEN && p.clip_col) v = round_to_T<T>(v * 0.75f);
-      if constexpr (SR == 0) {
-        codes[k] = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(0u, v, 0.0f, scale_f, 0) & 0xFu;
+      }
+      if constexpr (HW && !B2D) {
+        // out[] is complete
+      } else if (RHT) {
+        // undo the permutation: position k belongs to row perm_inv[k]; a private byte scratch in LDS does the indexing
+        uint32_t* stage = reinterpret_cast<uint32_t*>(tile);
+        uint8_t* sb = reinterpret_cast<uint8_t*>(stage + tid * STAGE_PITCH);
+  #pragma unroll
+        for (int k = 0; k < 32; ++k) sb[packed_byte(p.pinv4, k)] = (uint8_t)codes[k];
+        // same thread reads what it wrote: LDS ops of one wave complete in order, no barrier needed
+        uint32_t d[8];
+  #pragma unroll
+        for (int j = 0; j < 8; ++j) d[j] = stage[tid * STAGE_PITCH + j];
+  #pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          uint32_t ta = d[2 * j] | (d[2 * j] >> 4);
+          uint32_t tb = d[2 * j + 1] | (d[2 * j + 1] >> 4);
+          out[j] = __builtin_amdgcn_perm(tb, ta, 0x06040200u);
+        }
       } else {
-        uint32_t r;
-        if constexpr (EARLY) r = rc[k];
-        else r = stash[k * TILE_C + tid];
-        const float q = v * inv;
-        codes[k] = e2m1_sr_mag(q, r) | ((f2u(q) >> 28) & 8u);
+  #pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          uint32_t o = 0;
+  #pragma unroll
+          for (int e = 0; e < 8; ++e) o |= codes[8 * j + e] << (4 * e);
+          out[j] = o;
+        }
+      }
+      if constexpr (BPW == 1) {
+        const __amdgpu_buffer_rsrc_t rsrc_cc = __builtin_amdgcn_make_buffer_rsrc(
+            p.col_codes + (b * C + col0) * p.ld_cc + by * 16, 0, 0x7FFFFFFF, 0x00020000);
+        __builtin_amdgcn_raw_buffer_store_b128(v4u_t{out[0], out[1], out[2], out[3]}, rsrc_cc, cvalid ? tid * (int)p.ld_cc : OOB, 0, 0);
+      } else {
+  #pragma unroll
+        for (int q = 0; q + 1 < BPW; ++q)
+  #pragma unroll
+          for (int j = 0; j < 4; ++j) colacc[q][j] = colacc[q + 1][j];
+  #pragma unroll
+        for (int j = 0; j < 4; ++j) colacc[BPW - 1][j] = out[j];
       }
     }
-    }
-    if constexpr (HW && !B2D) {
-      // out[] is complete
-    } else if (RHT) {
-      // undo the permutation: position k belongs to row perm_inv[k]; a private byte scratch in LDS does the indexing
-      uint32_t* stage = reinterpret_cast<uint32_t*>(tile);
-      uint8_t* sb = reinterpret_cast<uint8_t*>(stage + tid * STAGE_PITCH);
-#pragma unroll
-      for (int k = 0; k < 32; ++k) sb[packed_byte(p.pinv4, k)] = (uint8_t)codes[k];
-      // same thread reads what it wrote: LDS ops of one wave complete in order, no barrier needed
-      uint32_t d[8];
-#pragma unroll
-      for (int j = 0; j < 8; ++j) d[j] = stage[tid * STAGE_PITCH + j];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        uint32_t ta = d[2 * j] | (d[2 * j] >> 4);
-        uint32_t tb = d[2 * j + 1] | (d[2 * j + 1] >> 4);
-        out[j] = __builtin_amdgcn_perm(tb, ta, 0x06040200u);
-      }
-    } else {
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        uint32_t o = 0;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) o |= codes[8 * j + e] << (4 * e);
-        out[j] = o;
-      }
-    }
+    ++bands_done;
+  }   // bands of this workgroup
+
+  if constexpr (BPW > 1) {
+    // Column codes out, whole lines: colacc[q] is the piece of band by0 + q - (BPW - bands_done) of this thread's column.
+    // In two halves of 128 columns through the first 16 KB of the tile: the column's thread writes its BPW pieces (slot
+    // XORed with the column so that neighbouring columns spread over the banks), then lane l of a wave takes piece l % 8
+    // of column l / 8: one store instruction covers 8 columns x 128 bytes.
+    uint4* stage = reinterpret_cast<uint4*>(tile);
+    static_assert(sizeof(tile) >= 128 * BPW * 16, "the column-code staging reuses the tile");
     const __amdgpu_buffer_rsrc_t rsrc_cc = __builtin_amdgcn_make_buffer_rsrc(
-        p.col_codes + (b * C + col0) * p.ld_cc + by * 16, 0, 0x7FFFFFFF, 0x00020000);
-    __builtin_amdgcn_raw_buffer_store_b128(v4u_t{out[0], out[1], out[2], out[3]}, rsrc_cc, cvalid ? tid * (int)p.ld_cc : OOB, 0, 0);
+        p.col_codes + (b * C + col0) * p.ld_cc + by0 * 16, 0, 0x7FFFFFFF, 0x00020000);
+    const int first = BPW - bands_done;   // pieces below this index hold nothing
+#pragma unroll 1
+    for (int half = 0; half < 2; ++half) {
+      __syncthreads();
+      if ((tid >> 7) == half) {
+        const int cl = tid & 127;
+#pragma unroll
+        for (int q = 0; q < BPW; ++q) stage[cl * BPW + (q ^ (cl & 7))] = make_uint4(colacc[q][0], colacc[q][1], colacc[q][2], colacc[q][3]);
+      }
+      __syncthreads();
+#pragma unroll
+      for (int j = 0; j < 128 * BPW / 256; ++j) {
+        const int idx = j * 256 + tid, cl = idx >> 3, q = (idx & 7) ^ (cl & 7);
+        const uint4 v = stage[idx];
+        const int ccol = col0 + half * 128 + cl;
+        __builtin_amdgcn_raw_buffer_store_b128(v4u_t{v.x, v.y, v.z, v.w}, rsrc_cc,
+                                               (ccol < C && q >= first) ? (half * 128 + cl) * (int)p.ld_cc + (q - first) * 16 : OOB, 0, 0);
+      }
+    }
   }
 }
 
@@ -653,40 +714,47 @@ int fill_hadamard(QuantParams& p, const int8_t* signs, const uint8_t* perm, cons
   return ALTO_MXFP4_OK;
 }
 
+// bpw8: the caller laid the grid out for workgroups of 8 bands (column outputs of large 2D-block tensors, !GEN only)
 template <typename T, bool DO_ROW, bool DO_COL, int SR, bool RHT, bool B2D, bool GEN>
-void launch(const QuantParams& p, dim3 grid, hipStream_t st) {
-  hipLaunchKernelGGL((quant_kernel<T, DO_ROW, DO_COL, SR, RHT, B2D, GEN>), grid, dim3(256), 0, st, p);
+void launch(const QuantParams& p, dim3 grid, hipStream_t st, bool bpw8) {
+  if constexpr (DO_COL && B2D && !GEN) {
+    if (bpw8) {
+      hipLaunchKernelGGL((quant_kernel<T, DO_ROW, DO_COL, SR, RHT, B2D, GEN, 8>), grid, dim3(256), 0, st, p);
+      return;
+    }
+  }
+  hipLaunchKernelGGL((quant_kernel<T, DO_ROW, DO_COL, SR, RHT, B2D, GEN, 1>), grid, dim3(256), 0, st, p);
 }
 
 template <typename T, int SR, bool GEN>
-void dispatch_mode(const QuantParams& p, dim3 grid, hipStream_t st, bool do_row, bool do_col, bool rht, bool b2d) {
+void dispatch_mode(const QuantParams& p, dim3 grid, hipStream_t st, bool do_row, bool do_col, bool rht, bool b2d, bool bpw8) {
   if (b2d) {
-    if (do_row && do_col) launch<T, true, true, SR, false, true, GEN>(p, grid, st);
-    else if (do_row) launch<T, true, false, SR, false, true, GEN>(p, grid, st);
-    else launch<T, false, true, SR, false, true, GEN>(p, grid, st);
+    if (do_row && do_col) launch<T, true, true, SR, false, true, GEN>(p, grid, st, bpw8);
+    else if (do_row) launch<T, true, false, SR, false, true, GEN>(p, grid, st, bpw8);
+    else launch<T, false, true, SR, false, true, GEN>(p, grid, st, bpw8);
   } else if (do_row && do_col) {
-    if (rht) launch<T, true, true, SR, true, false, GEN>(p, grid, st);
-    else launch<T, true, true, SR, false, false, GEN>(p, grid, st);
+    if (rht) launch<T, true, true, SR, true, false, GEN>(p, grid, st, bpw8);
+    else launch<T, true, true, SR, false, false, GEN>(p, grid, st, bpw8);
   } else if (do_row) {
-    launch<T, true, false, SR, false, false, GEN>(p, grid, st);
+    launch<T, true, false, SR, false, false, GEN>(p, grid, st, bpw8);
   } else {
-    if (rht) launch<T, false, true, SR, true, false, GEN>(p, grid, st);
-    else launch<T, false, true, SR, false, false, GEN>(p, grid, st);
+    if (rht) launch<T, false, true, SR, true, false, GEN>(p, grid, st, bpw8);
+    else launch<T, false, true, SR, false, false, GEN>(p, grid, st, bpw8);
   }
 }
 
 template <typename T>
-void dispatch(const QuantParams& p, dim3 grid, hipStream_t st, bool do_row, bool do_col, bool rht, bool b2d, int sr, bool gen) {
+void dispatch(const QuantParams& p, dim3 grid, hipStream_t st, bool do_row, bool do_col, bool rht, bool b2d, int sr, bool gen, bool bpw8) {
   if (gen) {
-    if (sr == 3) dispatch_mode<T, 3, true>(p, grid, st, do_row, do_col, rht, b2d);
-    else if (sr == 2) dispatch_mode<T, 2, true>(p, grid, st, do_row, do_col, rht, b2d);
-    else if (sr == 1) dispatch_mode<T, 1, true>(p, grid, st, do_row, do_col, rht, b2d);
-    else dispatch_mode<T, 0, true>(p, grid, st, do_row, do_col, rht, b2d);
+    if (sr == 3) dispatch_mode<T, 3, true>(p, grid, st, do_row, do_col, rht, b2d, bpw8);
+    else if (sr == 2) dispatch_mode<T, 2, true>(p, grid, st, do_row, do_col, rht, b2d, bpw8);
+    else if (sr == 1) dispatch_mode<T, 1, true>(p, grid, st, do_row, do_col, rht, b2d, bpw8);
+    else dispatch_mode<T, 0, true>(p, grid, st, do_row, do_col, rht, b2d, bpw8);
   } else {
-    if (sr == 3) dispatch_mode<T, 3, false>(p, grid, st, do_row, do_col, rht, b2d);
-    else if (sr == 2) dispatch_mode<T, 2, false>(p, grid, st, do_row, do_col, rht, b2d);
-    else if (sr == 1) dispatch_mode<T, 1, false>(p, grid, st, do_row, do_col, rht, b2d);
-    else dispatch_mode<T, 0, false>(p, grid, st, do_row, do_col, rht, b2d);
+    if (sr == 3) dispatch_mode<T, 3, false>(p, grid, st, do_row, do_col, rht, b2d, bpw8);
+    else if (sr == 2) dispatch_mode<T, 2, false>(p, grid, st, do_row, do_col, rht, b2d, bpw8);
+    else if (sr == 1) dispatch_mode<T, 1, false>(p, grid, st, do_row, do_col, rht, b2d, bpw8);
+    else dispatch_mode<T, 0, false>(p, grid, st, do_row, do_col, rht, b2d, bpw8);
   }
 }
 
@@ -779,17 +847,28 @@ int quantize_impl(const void* x, int dtype, int64_t batch, int64_t M, int64_t C,
   const bool gen = p.clip_row || p.clip_col || p.uos;
 
   const int64_t tiles_x = (C + TILE_C - 1) / TILE_C, bands = (M + 31) / 32;
-  // With a column output: 2^unit_shift workgroups per unit, units padded to a multiple of 8.  The largest unit (up to the
-  // 128 bands of a line of plain column scales) whose padding launches at most 5 % more workgroups than there are tiles.
-  int us = 7;
-  auto padded = [&](int sh) { return ((tiles_x * ((bands + (1ll << sh) - 1) >> sh) + 7) / 8 * 8) << sh; };
-  while (us > 3 && padded(us) * 20 > tiles_x * bands * 21) --us;
+  // Column outputs of large 2D-block tensors (weights): workgroups of 8 bands, which store their column codes as whole
+  // lines, eight columns per wave instruction, instead of one 16-byte piece of 64 different lines per instruction
+  // (measured: the 32 x 5760 x 2880 expert weights 408 -> 357 us with packed scales; a timing-only build with contiguous
+  // column stores: 267).  It pays from about 16 workgroups per CU on (8 experts: 94 -> 96 us, 14336 x 4096: 32 -> 38 us), and
+  // the 1D-block kernels, bound by their vector instructions, lose 5-40 % to the band loop's barriers and registers:
+  // all of those keep one band per workgroup.  ALTO_MXFP4_QUANT_BANDS=1|8 overrides the choice (tests, measurements).
+  static const int force_bpw = [] { const char* e = getenv("ALTO_MXFP4_QUANT_BANDS"); return e ? atoi(e) : 0; }();
+  const bool bpw8 = do_col && is_2d && !gen && (force_bpw == 8 || (force_bpw != 1 && tiles_x * ((bands + 7) / 8) * batch >= 4096));
+  const int64_t wrows = bpw8 ? (bands + 7) / 8 : bands;   // workgroup rows
+  // With a column output: 2^unit_shift workgroup rows per unit, units padded to a multiple of 8.  The largest unit (up to the
+  // 128 bands of a line of plain column scales) whose padding launches at most 5 % more workgroups than there are tiles;
+  // single-band workgroups take at least the 8 bands of a line of column codes.
+  const int us_min = bpw8 ? 0 : 3;
+  int us = bpw8 ? 4 : 7;
+  auto padded = [&](int sh) { return ((tiles_x * ((wrows + (1ll << sh) - 1) >> sh) + 7) / 8 * 8) << sh; };
+  while (us > us_min && padded(us) * 20 > tiles_x * wrows * 21) --us;
   p.unit_shift = us;
   ALTO_REQUIRE(do_col ? padded(us) < (1ll << 31) : (tiles_x < (1ll << 31) && bands <= 65535), "quantize: %lld x %lld exceeds the grid", (long long)M, (long long)C);
   const dim3 grid = do_col ? dim3((unsigned)padded(us), 1, (unsigned)batch) : dim3((unsigned)tiles_x, (unsigned)bands, (unsigned)batch);
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-  if (dtype == ALTO_DT_BF16) dispatch<__bf16>(p, grid, st, do_row, do_col, hadamard != 0, is_2d != 0, sr_mode, gen);
-  else dispatch<float>(p, grid, st, do_row, do_col, hadamard != 0, is_2d != 0, sr_mode, gen);
+  if (dtype == ALTO_DT_BF16) dispatch<__bf16>(p, grid, st, do_row, do_col, hadamard != 0, is_2d != 0, sr_mode, gen, bpw8);
+  else dispatch<float>(p, grid, st, do_row, do_col, hadamard != 0, is_2d != 0, sr_mode, gen, bpw8);
   return check_launch("quantize");
 }
 

@@ -297,3 +297,17 @@ def test_packed_dw_rejects_what_the_tile_kernel_does_not_serve(m):
     groups = G.groups_from_offsets(torch.tensor([0, 128, 256], dtype=torch.int32, device=DEV))
     with pytest.raises(NotImplementedError, match="not served by the tile kernel"):
         G.grouped_dw_packed(q.transpose(0, 1), ps, q.transpose(0, 1), ps, groups, E)
+
+
+def test_expert_weights_take_the_band_loop_and_keep_their_bytes(m):
+    """A batch of 2D-block matrices large enough for workgroups of eight bands (whole-line column-code stores): same four
+    outputs as matrix-by-matrix calls, which are below the size where that path is taken; M with a partial last group."""
+    from alto_amd.mxfp4.quantization import _prep, _quantize_call
+    E, R, C = 40, 1056, 5760          # 33 bands: groups of 8 + 1; 23 column tiles x 5 rows of bands x 40 >= 4096 workgroups
+    w = (randn_outliers((E, R, C), torch.bfloat16, seed=12) * 0.02).to(DEV)
+    kw = dict(use_sr=False, rand3=None, hadamard=None, clip=0, use_uos=False, pad_codes=True)
+    big = _quantize_call(_prep(w), True, True, True, **kw)
+    for e in (0, 17, E - 1):
+        one = _quantize_call(_prep(w[e:e + 1]), True, True, True, **kw)
+        for a, b_, what in zip(big, one, ("row codes", "row scales", "column codes", "column scales")):
+            assert_bytes_equal(a[e:e + 1].cpu(), b_.cpu(), f"expert {e}: {what}")
