@@ -135,9 +135,8 @@ __global__ __launch_bounds__(256) void quant_kernel(const QuantParams p) {
 
   const int tid = threadIdx.x;
   const int M = p.M, C = p.C;
-  // Workgroup -> (column tile bx, 32-row band by; with BPW > 1 "band" reads "row of BPW bands" below).  With a column
-  // output the grid is one-dimensional per matrix: consecutive
-  // workgroups go to the 8 XCDs in turn, so 8 x 2^unit_shift consecutive ones are laid out as 8 XCDs (one unit = column tile
+  // Workgroup -> (column tile bx, 32-row band by; with BPW > 1 read "row of BPW bands" for "band" below).  With a column
+  // output the grid is one-dimensional per matrix: consecutive workgroups go to the 8 XCDs in turn, so 8 x 2^unit_shift consecutive ones are laid out as 8 XCDs (one unit = column tile
   // x group of 2^unit_shift bands each, neighbouring column tiles first) x the unit's consecutive bands.  The 16-byte pieces
   // that make up a 128-byte line of the column codes (8 bands), and the bytes of a line of plain column scales (128 bands),
   // are then written through one XCD's L2 within a short time of each other and leave it as whole lines (measured: 65536 x
@@ -145,7 +144,6 @@ __global__ __launch_bounds__(256) void quant_kernel(const QuantParams p) {
   const int nby = (M + 31) >> 5;
   int bx, by0;   // column tile; first band of this workgroup
   if constexpr (DO_COL) {
-    // (the mapping above in units of workgroup rows of BPW bands)
     const unsigned wg = blockIdx.x, us = (unsigned)p.unit_shift;
     const unsigned unit = (wg >> (3 + us)) * 8 + (wg & 7), tiles_x = (unsigned)(C + TILE_C - 1) / TILE_C;
     bx = (int)(unit % tiles_x);
