@@ -377,13 +377,6 @@ extern "C" int alto_mxfp4_attention_fwd_ex(const void* q_codes, const void* q_sc
                                            int causal, const float* bias, int64_t bias_sb, int64_t bias_sh, int64_t bias_sm,
                                            const float* alibi_slopes, int64_t alibi_sb, int64_t alibi_sh, void* stream) {
   using namespace alto;
-  int64_t bias_bytes = 0;
-  if (bias) {
-    ALTO_REQUIRE(bias_sb >= 0 && bias_sh >= 0 && bias_sm >= Sk_used && bias_sm % 4 == 0 && (uintptr_t)bias % 16 == 0,
-                 "attention_fwd: bias rows must be 16-byte aligned with unit stride along the keys (row stride %lld)", (long long)bias_sm);
-    bias_bytes = ((B - 1) * bias_sb + (Hq - 1) * bias_sh + (Sq - 1) * bias_sm + Sk_used) * 4;
-    ALTO_REQUIRE(bias_bytes < (1ll << 32) && Sq * bias_sm * 4 < (1ll << 31), "attention_fwd: bias tensor too large");
-  }
   ALTO_REQUIRE(!alibi_slopes || (alibi_sb >= 0 && alibi_sh >= 0), "attention_fwd: negative alibi strides");
   ALTO_REQUIRE(q_codes && q_scales && k_codes && k_scales && vt_codes && v_scales && out && lse, "attention_fwd: null pointer");
   ALTO_REQUIRE(B > 0 && Hq > 0 && Hk > 0 && Hq % Hk == 0, "attention_fwd: Hq=%lld must be a positive multiple of Hk=%lld", (long long)Hq, (long long)Hk);
@@ -395,10 +388,20 @@ extern "C" int alto_mxfp4_attention_fwd_ex(const void* q_codes, const void* q_sc
                "attention_fwd: Sk_used=%lld must be a multiple of 32 in (Sk - 64, Sk]", (long long)Sk_used);
   ALTO_REQUIRE(!causal || Sq <= Sk_used, "attention_fwd: causal attention needs Sq <= Sk (got %lld > %lld)", (long long)Sq, (long long)Sk_used);
   ALTO_REQUIRE(B <= 65535 && (Sq + 127) / 128 <= 65535, "attention_fwd: B and Sq / 128 must fit a grid dimension");
-  ALTO_REQUIRE(B * Hq * Sq * (D > Dv ? D : Dv) < (1ll << 40), "attention_fwd: tensor too large");
+  ALTO_REQUIRE(Hq < (1ll << 31) && Sk < (1ll << 31) && product_below(1ll << 40, B * Sq, Hq, D > Dv ? D : Dv), "attention_fwd: tensor too large");
+  int64_t bias_bytes = 0;
+  if (bias) {   // (B, Hq, Sq and Sk_used are in range here)
+    ALTO_REQUIRE(bias_sb >= 0 && bias_sh >= 0 && bias_sm >= Sk_used && bias_sm % 4 == 0 && (uintptr_t)bias % 16 == 0,
+                 "attention_fwd: bias rows must be 16-byte aligned with unit stride along the keys (row stride %lld)", (long long)bias_sm);
+    ALTO_REQUIRE(product_below(1ll << 29, Sq, bias_sm) && product_below(1ll << 30, B - 1, bias_sb) && product_below(1ll << 30, Hq - 1, bias_sh),
+                 "attention_fwd: bias tensor too large");
+    bias_bytes = ((B - 1) * bias_sb + (Hq - 1) * bias_sh + (Sq - 1) * bias_sm + Sk_used) * 4;
+    ALTO_REQUIRE(bias_bytes < (1ll << 32), "attention_fwd: bias tensor too large");
+  }
   ALTO_REQUIRE(((uintptr_t)q_codes | (uintptr_t)k_codes | (uintptr_t)vt_codes) % 16 == 0 && (uintptr_t)out % 8 == 0,
                "attention_fwd: code pointers must be 16-byte aligned, out 8-byte aligned");
-  ALTO_REQUIRE(((uintptr_t)k_scales | (uintptr_t)v_scales) % 4 == 0, "attention_fwd: K and V scale pointers must be 4-byte aligned");
+  ALTO_REQUIRE(((uintptr_t)k_scales | (uintptr_t)v_scales | (uintptr_t)lse | (uintptr_t)alibi_slopes) % 4 == 0,
+               "attention_fwd: K and V scale pointers, lse and the alibi slopes must be 4-byte aligned");
   AttnArgs a{(const uint8_t*)q_codes, (const uint8_t*)q_scales, (const uint8_t*)k_codes, (const uint8_t*)k_scales,
              (const uint8_t*)vt_codes, (const uint8_t*)v_scales, out, lse, (int)Hq, (int)Hk, (int)Sq, (int)Sk, (int)Sk_used, sm_scale, causal ? 1 : 0,
              bias, bias_sb, bias_sh, bias_sm, bias_bytes, alibi_slopes, alibi_sb, alibi_sh};

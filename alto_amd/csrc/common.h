@@ -16,6 +16,12 @@ int quantize_dynamic_launch(const void* x, int dtype, int64_t batch, int64_t M, 
                             uint8_t* scales, int64_t ld_codes, int is_2d, int sr, const uint32_t* rand_bits, int64_t ld_rand,
                             int64_t bs_rand, int use_uos, hipStream_t st);
 
+// a * b * c < limit for non-negative factors; false when a factor is negative or the product leaves 64 bits on the way
+inline bool product_below(int64_t limit, int64_t a, int64_t b, int64_t c = 1) {
+  int64_t p;
+  return a >= 0 && b >= 0 && c >= 0 && !__builtin_mul_overflow(a, b, &p) && !__builtin_mul_overflow(p, c, &p) && p < limit;
+}
+
 #define ALTO_REQUIRE(cond, ...)            \
   do {                                     \
     if (!(cond)) {                         \

@@ -67,6 +67,8 @@ extern "C" int alto_mxfp4_dequantize(const uint8_t* codes, const uint8_t* scales
   ALTO_REQUIRE(!is_2d || R % 32 == 0, "dequantize: 2D blocks need R (%lld) %% 32 == 0", (long long)R);
   ALTO_REQUIRE(out_dtype == ALTO_DT_BF16 || out_dtype == ALTO_DT_F32, "dequantize: bad out_dtype %d", out_dtype);
   ALTO_REQUIRE((reinterpret_cast<uintptr_t>(codes) & 3) == 0, "dequantize: codes must be 4-byte aligned");
+  ALTO_REQUIRE((reinterpret_cast<uintptr_t>(out) & (out_dtype == ALTO_DT_F32 ? 3 : 1)) == 0, "dequantize: out must be aligned to its element size");
+  ALTO_REQUIRE(R < (1ll << 31) && C < (1ll << 31) && product_below(1ll << 39, R, C / 8), "dequantize: %lld x %lld exceeds the grid", (long long)R, (long long)C);
   if (R == 0 || C == 0) return ALTO_MXFP4_OK;
   const int64_t n = R * (C / 8);
   dim3 grid((unsigned)((n + 255) / 256));
@@ -83,6 +85,7 @@ extern "C" int alto_mxfp4_transpose_codes(const uint8_t* in, int64_t R, int64_t 
   using namespace alto;
   ALTO_REQUIRE(in && out, "transpose_codes: NULL pointer");
   ALTO_REQUIRE(R >= 0 && C >= 0 && R % 2 == 0 && C % 2 == 0, "transpose_codes: R and C must be even");
+  ALTO_REQUIRE(R < (1ll << 31) && C < (1ll << 31), "transpose_codes: size out of range");
   if (R == 0 || C == 0) return ALTO_MXFP4_OK;
   dim3 grid((unsigned)((C + 63) / 64), (unsigned)((R + 63) / 64));
   ALTO_REQUIRE(grid.y <= 65535u, "transpose_codes: R too large");

@@ -86,8 +86,8 @@ bool gemm_tiled_supported(const OperandView& A, const OperandView& B, int64_t M,
   if (M < 128 || N < 128 || K < 512) return false;   // (scale rows are read 16 bytes = 512 K at a time)
   // the tile kernel reads scale rows with unit stride along K and stores C in aligned 16-byte groups
   if (A.ss_k != 1 || B.ss_k != 1) return false;
-  if (M * A.ld >= (1ll << 31) || N * B.ld >= (1ll << 31)) return false;   // 32-bit buffer offsets
-  if (M * A.ss_r >= (1ll << 31) || N * B.ss_r >= (1ll << 31)) return false;
+  if (!product_below(1ll << 31, M, A.ld) || !product_below(1ll << 31, N, B.ld)) return false;   // 32-bit buffer offsets
+  if (!product_below(1ll << 31, M, A.ss_r) || !product_below(1ll << 31, N, B.ss_r)) return false;
   if (N % 8 != 0 || ldc % 8 != 0 || (reinterpret_cast<uintptr_t>(c) & 15) != 0) return false;
   const int64_t tiles = ((M + GT_TM - 1) / GT_TM) * ((N + GT_TN - 1) / GT_TN);
   return tiles < (1ll << 28);

@@ -522,25 +522,29 @@ int grouped_gemm_impl(const uint8_t* a, int64_t lda, const uint8_t* a_scales, in
                       int64_t M_total, int64_t N, int64_t K, void* out, int out_dtype, int64_t ldo,
                       void* plan, int64_t plan_bytes, const char* plan_name, bool build_plan, void* stream, bool ps = false) {
   ALTO_REQUIRE(a && a_scales && w && w_scales && offs && out, "grouped_gemm: NULL pointer");
+  ALTO_REQUIRE(((reinterpret_cast<uintptr_t>(offs) | reinterpret_cast<uintptr_t>(group_expert)) & 3) == 0, "grouped_gemm: offs and group_expert must be 4-byte aligned");
   ALTO_REQUIRE(num_groups > 0 && num_groups <= 65536, "grouped_gemm: num_groups (%d) out of range", num_groups);
   ALTO_REQUIRE(group_expert != nullptr || num_groups == num_experts, "grouped_gemm: without group_expert, num_groups must equal num_experts");
   ALTO_REQUIRE(num_experts > 0 && num_experts <= 4096, "grouped_gemm: num_experts (%d) out of range", num_experts);
   ALTO_REQUIRE(M_total >= 0 && N >= 0 && K >= 0 && K % 32 == 0, "grouped_gemm: K (%lld) must be a multiple of 32", (long long)K);
+  ALTO_REQUIRE(M_total < (1ll << 31) && N < (1ll << 31) && K < (1ll << 31), "grouped_gemm: size out of range");
   ALTO_REQUIRE(!w_is_2d || N % 32 == 0, "grouped_gemm: 2D weight scales need N (%lld) %% 32 == 0", (long long)N);
   ALTO_REQUIRE(!a_is_2d || M_total % 32 == 0, "grouped_gemm: 2D activation scales need M_total %% 32 == 0");
   ALTO_REQUIRE(lda >= K / 2 && ldw >= K / 2 && lda % 16 == 0 && ldw % 16 == 0 && w_stride_e % 16 == 0,
                "grouped_gemm: lda/ldw/w_stride_e must be >= K/2 and multiples of 16 bytes");
   ALTO_REQUIRE(((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(w)) & 15) == 0, "grouped_gemm: a and w must be 16-byte aligned");
   ALTO_REQUIRE(ldo >= N, "grouped_gemm: ldo < N");
+  ALTO_REQUIRE(a_ss_r >= 0 && a_ss_k >= 0 && ws_stride_e >= 0 && ws_r >= 0 && ws_k >= 0 && w_stride_e >= 0, "grouped_gemm: negative stride");
   ALTO_REQUIRE(out_dtype == ALTO_DT_BF16 || out_dtype == ALTO_DT_F32, "grouped_gemm: bad out_dtype %d", out_dtype);
+  ALTO_REQUIRE((reinterpret_cast<uintptr_t>(out) & (out_dtype == ALTO_DT_F32 ? 3 : 1)) == 0, "grouped_gemm: out must be aligned to its element size");
   if (M_total == 0 || N == 0) return ALTO_MXFP4_OK;
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   OperandView A{a, lda, a_scales, a_ss_r, ps ? M_total * 16 : a_ss_k, a_is_2d};
   // 256x256 tiles when the problem fills them and the layouts fit their loads (unit-stride scale rows, 32-bit buffer
   // offsets, 16-byte output chunks); otherwise the direct kernel below
   const bool tiled = M_total >= 128 && N >= 128 && K >= 512 && a_ss_k == 1 && ws_k == 1 && N % 8 == 0 && ldo % 8 == 0 &&
-                     (reinterpret_cast<uintptr_t>(out) & 15) == 0 && M_total * lda < (1ll << 31) && N * ldw < (1ll << 31) &&
-                     M_total * a_ss_r < (1ll << 31) && N * ws_r < (1ll << 31) &&
+                     (reinterpret_cast<uintptr_t>(out) & 15) == 0 && product_below(1ll << 31, M_total, lda) && product_below(1ll << 31, N, ldw) &&
+                     product_below(1ll << 31, M_total, a_ss_r) && product_below(1ll << 31, N, ws_r) &&
                      grouped_max_passes(M_total, num_groups) * ((N + GT_TN - 1) / GT_TN) < (1ll << 28);
   if (ps && !(tiled && out_dtype == ALTO_DT_BF16)) {
     set_error("grouped_gemm_ps: shape (%lld, %lld, %lld) is not served by the tile kernel; use plain scales", (long long)M_total, (long long)N, (long long)K);
@@ -612,7 +616,7 @@ int grouped_gemm_impl(const uint8_t* a, int64_t lda, const uint8_t* a_scales, in
 }  // namespace alto
 
 extern "C" int64_t alto_mxfp4_grouped_gemm_workspace_bytes(int64_t M_total, int num_groups) {
-  if (M_total < 0 || num_groups < 0) return 0;
+  if (M_total < 0 || M_total >= (1ll << 31) || num_groups < 0) return 0;   // sizes no grouped call accepts
   return alto::grouped_workspace_bytes(M_total, num_groups);
 }
 
@@ -644,7 +648,8 @@ extern "C" int alto_mxfp4_grouped_gemm_ps(const uint8_t* a, int64_t lda, const u
   using namespace alto;
   ALTO_REQUIRE(((reinterpret_cast<uintptr_t>(a_packed) | reinterpret_cast<uintptr_t>(w_packed) | (uintptr_t)wp_stride_e) & 15) == 0,
                "grouped_gemm_ps: packed scales (and the stride between experts) must be 16-byte aligned");
-  ALTO_REQUIRE(K >= 0 && ((K / 32 + 15) / 16) * (M_total > N ? M_total : N) * 16 < (1ll << 31), "grouped_gemm_ps: packed scales beyond 2 GiB");
+  ALTO_REQUIRE(K >= 0 && K < (1ll << 31) && product_below(1ll << 31, (K / 32 + 15) / 16, M_total > N ? M_total : N, 16),
+               "grouped_gemm_ps: packed scales beyond 2 GiB");
   // A: [blocks][M_total][16]; expert e's weights: [blocks][N][16] at w_packed + e * wp_stride_e
   return grouped_gemm_impl(a, lda, a_packed, 16, 1, 0, w, w_stride_e, ldw, w_packed, wp_stride_e, 16, 1, 0, offs, group_expert, num_groups, num_experts,
                            M_total, N, K, out, ALTO_DT_BF16, ldo, workspace, workspace_bytes, "the workspace", plan_built == 0, stream, true);
@@ -654,6 +659,7 @@ extern "C" int alto_mxfp4_grouped_gemm_plan(const int32_t* offs, const int32_t* 
                                             void* workspace, int64_t workspace_bytes, void* stream) {
   using namespace alto;
   ALTO_REQUIRE(offs != nullptr, "grouped_gemm_plan: NULL offs");
+  ALTO_REQUIRE(((reinterpret_cast<uintptr_t>(offs) | reinterpret_cast<uintptr_t>(group_expert)) & 3) == 0, "grouped_gemm_plan: offs and group_expert must be 4-byte aligned");
   ALTO_REQUIRE(num_groups > 0 && num_groups <= 65536, "grouped_gemm_plan: num_groups (%d) out of range", num_groups);
   ALTO_REQUIRE(group_expert != nullptr || num_groups == num_experts, "grouped_gemm_plan: without group_expert, num_groups must equal num_experts");
   ALTO_REQUIRE(num_experts > 0 && num_experts <= 4096, "grouped_gemm_plan: num_experts (%d) out of range", num_experts);
@@ -710,7 +716,7 @@ extern "C" int alto_mxfp4_grouped_gemm_noalloc(const uint8_t* a, int64_t lda, co
                                                const int32_t* offs, const int32_t* group_expert, int num_groups, int num_experts,
                                                int64_t M_total, int64_t N, int64_t K, void* out, int out_dtype, int64_t ldo, void* stream) {
   using namespace alto;
-  ALTO_REQUIRE(M_total >= 0 && num_groups > 0, "grouped_gemm_noalloc: bad sizes");
+  ALTO_REQUIRE(M_total >= 0 && M_total < (1ll << 31) && num_groups > 0, "grouped_gemm_noalloc: bad sizes");
   ALTO_REQUIRE(grouped_workspace_bytes(M_total, num_groups) <= ALTO_NOALLOC_SCRATCH_BYTES,
                "grouped_gemm_noalloc: M_total = %lld rows in %d groups need a pass list of %lld bytes, more than the built-in %lld: use "
                "alto_mxfp4_grouped_gemm with a workspace", (long long)M_total, num_groups, (long long)grouped_workspace_bytes(M_total, num_groups),
@@ -731,14 +737,18 @@ int grouped_dw_impl(const uint8_t* go, int64_t ld_go, const uint8_t* go_scales, 
                     int64_t M_total, int64_t N, int64_t K, void* dw, int dw_dtype, int64_t dw_stride_e, int64_t dw_stride_n, int64_t dw_stride_k,
                     float out_scale, void* stream, bool ps) {
   ALTO_REQUIRE(go && go_scales && x && x_scales && offs && dw, "grouped_gemm_dw: NULL pointer");
+  ALTO_REQUIRE(((reinterpret_cast<uintptr_t>(offs) | reinterpret_cast<uintptr_t>(group_expert)) & 3) == 0, "grouped_gemm_dw: offs and group_expert must be 4-byte aligned");
+  ALTO_REQUIRE((reinterpret_cast<uintptr_t>(dw) & (dw_dtype == ALTO_DT_F32 ? 3 : 1)) == 0, "grouped_gemm_dw: dw must be aligned to its element size");
   ALTO_REQUIRE(num_experts > 0 && num_experts <= 65535, "grouped_gemm_dw: num_experts (%d) out of range", num_experts);
   ALTO_REQUIRE(num_groups > 0 && num_groups <= 65536, "grouped_gemm_dw: num_groups (%d) out of range", num_groups);
   ALTO_REQUIRE(group_expert != nullptr || num_groups == num_experts, "grouped_gemm_dw: without group_expert, num_groups must equal num_experts");
   ALTO_REQUIRE(M_total >= 0 && M_total % 32 == 0, "grouped_gemm_dw: M_total (%lld) must be a multiple of 32", (long long)M_total);
+  ALTO_REQUIRE(N >= 0 && K >= 0 && M_total < (1ll << 31) && N < (1ll << 31) && K < (1ll << 31), "grouped_gemm_dw: size out of range");
   ALTO_REQUIRE(ld_go >= M_total / 2 && ld_xq >= M_total / 2 && ld_go % 16 == 0 && ld_xq % 16 == 0,
                "grouped_gemm_dw: ld_go/ld_xq must be >= M_total/2 and multiples of 16 bytes");
   ALTO_REQUIRE(((reinterpret_cast<uintptr_t>(go) | reinterpret_cast<uintptr_t>(x)) & 15) == 0, "grouped_gemm_dw: go and x must be 16-byte aligned");
   ALTO_REQUIRE(dw_dtype == ALTO_DT_BF16 || dw_dtype == ALTO_DT_F32, "grouped_gemm_dw: bad dw_dtype %d", dw_dtype);
+  ALTO_REQUIRE(gs_r >= 0 && gs_k >= 0 && xs_r >= 0 && xs_k >= 0 && dw_stride_e >= 0 && dw_stride_n >= 0 && dw_stride_k >= 0, "grouped_gemm_dw: negative stride");
   if (N == 0 || K == 0) return ALTO_MXFP4_OK;
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   ALTO_REQUIRE((!go_is_2d || N % 32 == 0) && (!x_is_2d || K % 32 == 0), "grouped_gemm_dw: 2D scales need N (%lld) / K (%lld) %% 32 == 0", (long long)N, (long long)K);
@@ -753,8 +763,8 @@ int grouped_dw_impl(const uint8_t* go, int64_t ld_go, const uint8_t* go_scales, 
     const int64_t ld = n_major ? dw_stride_n : dw_stride_k;
     const bool unit = n_major || dw_stride_n == 1;
     const bool tiled = unit && M_total >= 512 && N >= 128 && K >= 128 && (ps || (gs_k == 1 && xs_k == 1)) && NQ % 8 == 0 && ld % 8 == 0 && dw_stride_e % 8 == 0 &&
-                       (reinterpret_cast<uintptr_t>(dw) & 15) == 0 && N * ld_go < (1ll << 31) && K * ld_xq < (1ll << 31) &&
-                       N * gs_r < (1ll << 31) && K * xs_r < (1ll << 31) && num_groups <= GT_DW_MAX_GROUPS && num_experts <= 65535 &&
+                       (reinterpret_cast<uintptr_t>(dw) & 15) == 0 && product_below(1ll << 31, N, ld_go) && product_below(1ll << 31, K, ld_xq) &&
+                       product_below(1ll << 31, N, gs_r) && product_below(1ll << 31, K, xs_r) && num_groups <= GT_DW_MAX_GROUPS && num_experts <= 65535 &&
                        ((NP + GT_TM - 1) / GT_TM) * ((NQ + GT_TN - 1) / GT_TN) < (1ll << 28);
     if (ps && !(tiled && dw_dtype == ALTO_DT_BF16)) {
       set_error("grouped_gemm_dw_ps: shape (%lld tokens, %lld, %lld) is not served by the tile kernel; use plain scales", (long long)M_total, (long long)N, (long long)K);
@@ -798,7 +808,8 @@ extern "C" int alto_mxfp4_grouped_gemm_dw_ps(const uint8_t* go, int64_t ld_go, c
                                              float out_scale, void* stream) {
   using namespace alto;
   ALTO_REQUIRE(((reinterpret_cast<uintptr_t>(go_packed) | reinterpret_cast<uintptr_t>(x_packed)) & 15) == 0, "grouped_gemm_dw_ps: packed scales must be 16-byte aligned");
-  ALTO_REQUIRE(M_total >= 0 && ((M_total + 511) / 512) * (N > K ? N : K) * 16 < (1ll << 31), "grouped_gemm_dw_ps: packed scales beyond 2 GiB");
+  ALTO_REQUIRE(M_total >= 0 && M_total < (1ll << 31) && N >= 0 && K >= 0 && product_below(1ll << 31, (M_total + 511) / 512, N > K ? N : K, 16),
+               "grouped_gemm_dw_ps: negative size, or packed scales beyond 2 GiB");
   // go: [blocks][N][16], x: [blocks][K][16]; ss_k carries the bytes from block to block
   return grouped_dw_impl(go, ld_go, go_packed, 16, N * 16, 0, x, ld_xq, x_packed, 16, K * 16, 0, offs, group_expert, num_groups, num_experts,
                          M_total, N, K, dw, ALTO_DT_BF16, dw_stride_e, dw_stride_n, dw_stride_k, out_scale, stream, true);

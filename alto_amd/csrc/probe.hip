@@ -61,6 +61,7 @@ __global__ __launch_bounds__(512) void mfma_probe_kernel(float* sink, int iters,
 extern "C" int alto_mxfp4_probe_mfma(int random_operands, int iters, int workgroups, float* sink, uint64_t* ticks, void* stream) {
   using namespace alto;
   ALTO_REQUIRE(sink != nullptr, "probe_mfma: sink is NULL (needs 512 floats of device memory)");
+  ALTO_REQUIRE((reinterpret_cast<uintptr_t>(sink) & 3) == 0 && (reinterpret_cast<uintptr_t>(ticks) & 7) == 0, "probe_mfma: sink must be 4-byte and ticks 8-byte aligned");
   ALTO_REQUIRE(iters > 0 && iters <= (1 << 24) && workgroups > 0 && workgroups <= 65535, "probe_mfma: iters/workgroups out of range");
   hipLaunchKernelGGL(mfma_probe_kernel, dim3((unsigned)workgroups), dim3(512), 0, reinterpret_cast<hipStream_t>(stream), sink, iters,
                      random_operands ? 1 : 0, ticks);

@@ -920,8 +920,10 @@ extern "C" int alto_mxfp4_quantize_sr_hw(const void* x, int dtype, int64_t batch
 }
 
 extern "C" int64_t alto_mxfp4_quantize_sr_hw_words(int dtype, int64_t batch, int64_t M, int64_t C) {
+  if (batch < 0 || M < 0 || C < 0 || M >= (1ll << 31) || C >= (1ll << 31) || batch >= 65536) return 0;   // sizes no quantizer call accepts
   const int64_t nb = (M + 31) / 32;
-  return 4 * (dtype == ALTO_DT_BF16 ? 2 : 8) * batch * nb * C;
+  const int64_t per_column = 4 * (dtype == ALTO_DT_BF16 ? 2 : 8) * batch * nb;   // < 2^5 * 2^16 * 2^26
+  return alto::product_below(INT64_MAX, per_column, C) ? per_column * C : 0;
 }
 
 extern "C" int alto_mxfp4_quantize_ex(const void* x, int dtype, int64_t batch, int64_t M, int64_t C, int64_t ld_x, int64_t bs_x,
@@ -956,7 +958,8 @@ extern "C" int alto_mxfp4_hadamard_apply(const void* x, int dtype, int64_t M, in
   ALTO_REQUIRE(!left_mul || M % 32 == 0, "hadamard: M (%lld) must be a multiple of 32", (long long)M);
   ALTO_REQUIRE(left_mul || C % 32 == 0, "hadamard: C (%lld) must be a multiple of 32 for a multiplication from the right", (long long)C);
   ALTO_REQUIRE(ld_x >= C && ld_y >= C, "hadamard: row stride smaller than C");
-  ALTO_REQUIRE(C < (1ll << 31), "hadamard: size out of range");
+  ALTO_REQUIRE(M < (1ll << 31) && C < (1ll << 31), "hadamard: size out of range");
+  ALTO_REQUIRE(((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) & (dtype == ALTO_DT_BF16 ? 1 : 3)) == 0, "hadamard: x and y must be aligned to their element size");
   QuantParams p{};
   int rc = fill_hadamard(p, signs, perm, "hadamard");
   if (rc != ALTO_MXFP4_OK) return rc;

@@ -27,7 +27,7 @@ __global__ __launch_bounds__(256) void random_bits_kernel(uint32_t* __restrict__
 
 extern "C" int alto_mxfp4_random_bits(uint32_t* out, int64_t n, uint64_t seed, uint64_t offset, void* stream) {
   using namespace alto;
-  ALTO_REQUIRE(n >= 0, "random_bits: negative count");
+  ALTO_REQUIRE(n >= 0 && n < (1ll << 48), "random_bits: count out of range");
   if (n == 0) return ALTO_MXFP4_OK;
   ALTO_REQUIRE(out != nullptr, "random_bits: NULL output");
   ALTO_REQUIRE((reinterpret_cast<uintptr_t>(out) & 15) == 0, "random_bits: out must be 16-byte aligned");
