@@ -20,7 +20,7 @@ from . import _runtime as rt
 from .._lib import check
 from .hadamard import HadamardFactory, HadamardTransform
 from .linear import _wgrad_scale, cached_weight_quantisation, packed_scales_enabled, transpose_codes, unwrap_weight_wrapper
-from .quantization import convert_to_mxfp4, quantize_rowcol
+from .quantization import quantize_rowcol
 
 ALIGN_SIZE_M = 128
 
