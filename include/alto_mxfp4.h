@@ -7,6 +7,10 @@
  * owns inputs and outputs.  The return value is 0 on success or a negative
  * ALTO_MXFP4_E* code; alto_mxfp4_last_error() then describes the failure
  * (thread-local string).  Invalid shapes are rejected BEFORE any launch.
+ * Common to all entry points: sizes, counts and strides are non-negative,
+ * matrix dimensions stay below 2^31, and a pointer to 2-, 4- or 8-byte
+ * elements (bf16 / fp32 outputs, int32 offsets, uint64 state) is aligned to
+ * its element size; the stricter alignments are stated per function.
  *
  * Each function names the entry point of the reference (AMD-AGI/ALTO, paths
  * relative to its checkout) whose device work it replaces.
