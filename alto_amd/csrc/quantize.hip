@@ -33,6 +33,7 @@ struct QuantParams {
   uint8_t* col_scales;
   int64_t ld_rc, ld_cc;  // row pitch in bytes of the row / column code outputs (>= C/2, M/2)
   uint32_t sign_mask;    // bit k set: Q[k] == -1 (k = position after the permutation)
+  uint32_t sign_nib[4];  // the same signs as code bits in row order: bit 4 r + 3 set when row r of a block sits at a position with Q == -1
   uint32_t perm4[8];     // row j of a block -> position perm[j], four bytes per word
   uint32_t pinv4[8];     // position k -> row
   int clip_row;          // 1: multiply by 3/4 (in the input dtype) before encoding the row output
@@ -120,6 +121,7 @@ __global__ __launch_bounds__(256) void quant_kernel(const QuantParams p) {
   constexpr bool EARLY = DO_COL && SR == 1;
   constexpr bool STASH = DO_COL && SR == 2;
   constexpr bool HW = SR == 3;
+  constexpr bool DEFER_FLIP = RHT && DO_COL && !HW;   // the Hadamard signs go onto the finished column codes
   constexpr bool XCODES = HW && B2D && DO_COL;   // 2D blocks: the column packing takes the row phase's codes through LDS
   constexpr int OOB = (int)0x80000000;
   // the column phase of the hardware mode brings its transformed values back to row order through a private strip per
@@ -357,12 +359,23 @@ __global__ __launch_bounds__(256) void quant_kernel(const QuantParams p) {
           out = __builtin_amdgcn_perm(by[1], by[0], 0x0C0C0400u) | __builtin_amdgcn_perm(by[3], by[2], 0x04000C0Cu);
         } else {
           const float inv = u2f((254u - s) << 23);
-  #pragma unroll
-          for (int e = 0; e < 8; ++e) {
-            const float q = v[e] * inv;
-            const uint32_t code = e2m1_sr_mag(q, rr[i][e]) | ((f2u(q) >> 28) & 8u);
-            out |= code << (4 * e);
+          // sign bits of the eight codes from four hardware converts (their magnitudes are not used): 5 instructions
+          // instead of 16
+          uint32_t sg = 0;
+          if constexpr (BF) {
+            sg = __builtin_amdgcn_cvt_scalef32_pk_fp4_bf16(sg, __builtin_bit_cast(bf16x2_t, w[i][0]), scale_f, 0);
+            sg = __builtin_amdgcn_cvt_scalef32_pk_fp4_bf16(sg, __builtin_bit_cast(bf16x2_t, w[i][1]), scale_f, 1);
+            sg = __builtin_amdgcn_cvt_scalef32_pk_fp4_bf16(sg, __builtin_bit_cast(bf16x2_t, w[i][2]), scale_f, 2);
+            sg = __builtin_amdgcn_cvt_scalef32_pk_fp4_bf16(sg, __builtin_bit_cast(bf16x2_t, w[i][3]), scale_f, 3);
+          } else {
+            sg = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(sg, v[0], v[1], scale_f, 0);
+            sg = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(sg, v[2], v[3], scale_f, 1);
+            sg = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(sg, v[4], v[5], scale_f, 2);
+            sg = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(sg, v[6], v[7], scale_f, 3);
           }
+          out = sg & 0x88888888u;
+  #pragma unroll
+          for (int e = 0; e < 8; ++e) out |= e2m1_sr_mag(v[e] * inv, rr[i][e]) << (4 * e);
         }
         if constexpr (DO_ROW) __builtin_amdgcn_raw_buffer_store_b32(out, rsrc_rc, valid[i] ? rsub * ldrc + (c >> 1) : OOB, 8 * i * ldrc, 0);
         if constexpr (XCODES) {   // one code per byte, in column order, for the column packing
@@ -406,7 +419,11 @@ __global__ __launch_bounds__(256) void quant_kernel(const QuantParams p) {
         // measured: the second copy of the loop costs more than the 32 guards save.)
   #pragma unroll
         for (int k = 0; k < 32; ++k) {
-          const uint32_t flip = ((p.sign_mask >> k) & 1u) << 31;   // scalar: the constants stay in scalar registers
+          // Q[k] = -1: folded into the (wave-uniform) constants in the hardware mode; the software rule, which is short of
+          // scalar registers (the 64 signed constants made it spill 24 of them into vector lanes), divides by +sqrt(32) and
+          // flips the sign bits of the finished codes instead (DEFER_FLIP below: rounding, absmax and both encodes are
+          // symmetric in the sign)
+          const uint32_t flip = DEFER_FLIP ? 0u : ((p.sign_mask >> k) & 1u) << 31;
           const float ck = u2f(f2u(5.656854152679443f) ^ flip);
           const float rck = u2f(f2u(0.17677669529663689f) ^ flip);
           const float q = z[k] * rck;
@@ -556,6 +573,10 @@ __global__ __launch_bounds__(256) void quant_kernel(const QuantParams p) {
           for (int e = 0; e < 8; ++e) o |= codes[8 * j + e] << (4 * e);
           out[j] = o;
         }
+      }
+      if constexpr (DEFER_FLIP) {
+  #pragma unroll
+        for (int j = 0; j < 4; ++j) out[j] ^= p.sign_nib[j];
       }
       if constexpr (BPW == 1) {
         const __amdgpu_buffer_rsrc_t rsrc_cc = __builtin_amdgcn_make_buffer_rsrc(
@@ -709,6 +730,9 @@ int fill_hadamard(QuantParams& p, const int8_t* signs, const uint8_t* perm, cons
     ALTO_REQUIRE(signs[k] == 1 || signs[k] == -1, "%s: signs[%d] = %d is not +1/-1", who, k, (int)signs[k]);
     if (signs[k] < 0) p.sign_mask |= 1u << k;
   }
+  for (int w = 0; w < 4; ++w) p.sign_nib[w] = 0;
+  for (int r = 0; r < 32; ++r)
+    if ((p.sign_mask >> (perm ? perm[r] : r)) & 1u) p.sign_nib[r >> 3] |= 8u << (4 * (r & 7));
   return ALTO_MXFP4_OK;
 }
 
@@ -829,6 +853,7 @@ int quantize_impl(const void* x, int dtype, int64_t batch, int64_t M, int64_t C,
   p.row_codes = row_codes; p.row_scales = row_scales; p.col_codes = col_codes; p.col_scales = col_scales;
   p.ld_rc = ld_row_codes; p.ld_cc = ld_col_codes;
   p.sign_mask = 0;
+  for (int w = 0; w < 4; ++w) p.sign_nib[w] = 0;
   for (int w = 0; w < 8; ++w) p.perm4[w] = p.pinv4[w] = 0x03020100u + 0x04040404u * (uint32_t)w;   // identity
   if (hadamard) {
     int rc = fill_hadamard(p, signs, perm, "quantize");
