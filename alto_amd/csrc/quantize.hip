@@ -413,10 +413,8 @@ __global__ __launch_bounds__(256) void quant_kernel(const QuantParams p) {
             }
           }
         }
-        // z * (+-1) / float32(sqrt(32)), correctly rounded: quotient estimate, one FMA correction, both with the sign
-        // folded into the (wave-uniform) constants; the sign bit is taken from the estimate so that -0 stays -0.
-        // (Taking the block's absmax before the division and dropping the guard for columns without an infinity was
-        // measured: the second copy of the loop costs more than the 32 guards save.)
+        // z * (+-1) / float32(sqrt(32)), correctly rounded: quotient estimate, one FMA correction, special cases and the
+        // sign by the division fix-up instruction.
   #pragma unroll
         for (int k = 0; k < 32; ++k) {
           // Q[k] = -1: folded into the (wave-uniform) constants in the hardware mode; the software rule, which is short of
@@ -427,9 +425,10 @@ __global__ __launch_bounds__(256) void quant_kernel(const QuantParams p) {
           const float ck = u2f(f2u(5.656854152679443f) ^ flip);
           const float rck = u2f(f2u(0.17677669529663689f) ^ flip);
           const float q = z[k] * rck;
-          float r = __builtin_fmaf(-q, ck, z[k]);
-          r = __builtin_fmaxf(r, -3.0e38f);   // z = +-inf gives r = NaN: drop it so that the quotient stays +-inf
-          z[k] = u2f((f2u(__builtin_fmaf(r, rck, q)) & 0x7FFFFFFFu) | (f2u(q) & 0x80000000u));
+          // v_div_fixup_f32 gives the quotient its sign (sign(z) ^ sign(ck), so -0 stays -0) and returns +-inf for z = +-inf,
+          // where the correction term is NaN; otherwise it passes the magnitude through (measured against a max + bit-field
+          // insert pair doing the same: 0.6 % faster with the software rule, 1.4 % with the hardware converts)
+          z[k] = __builtin_amdgcn_div_fixupf(__builtin_fmaf(__builtin_fmaf(-q, ck, z[k]), rck, q), ck, z[k]);
         }
         if constexpr (BF) {   // round to bf16 two at a time
   #pragma unroll
