@@ -127,7 +127,9 @@ __global__ __launch_bounds__(256) void quant_kernel(const QuantParams p) {
   // the column phase of the hardware mode brings its transformed values back to row order through a private strip per
   // thread (17 dwords of bf16 pairs or 33 dwords of fp32: odd pitches, conflict-free), which reuses the tile's memory
   constexpr int STRIP = BF ? 17 : 33;
-  constexpr int TILE_ELEMS = !DO_COL ? 8 : ((HW && RHT) ? (256 * STRIP * 4 + (int)sizeof(T) - 1) / (int)sizeof(T) : 32 * TILE_C);
+  // the column phase hands the hardware converts two rows at a time (stochastic mode with 1D blocks, round to nearest always)
+  constexpr bool PAIRS = (HW && !B2D) || SR == 0;
+  constexpr int TILE_ELEMS = !DO_COL ? 8 : ((PAIRS && RHT) ? (256 * STRIP * 4 + (int)sizeof(T) - 1) / (int)sizeof(T) : 32 * TILE_C);
   __shared__ __align__(16) T tile[TILE_ELEMS];
   __shared__ __align__(8) uint8_t xcodes[XCODES ? 32 * TILE_C : 8];
   __shared__ __align__(16) uint32_t stash[STASH ? 32 * TILE_C : 4];
@@ -476,7 +478,7 @@ __global__ __launch_bounds__(256) void quant_kernel(const QuantParams p) {
         __syncthreads();
   #pragma unroll
         for (int k = 0; k < 32; ++k) codes[k] = xcodes[k * TILE_C + tid];
-      } else if constexpr (HW) {
+      } else if constexpr (PAIRS) {
         // transformed values back to row order (a private strip in LDS undoes the permutation), then one hardware
         // convert per pair of rows
         if (GEN && p.clip_col) {
@@ -501,12 +503,24 @@ __global__ __launch_bounds__(256) void quant_kernel(const QuantParams p) {
   #pragma unroll
             for (int j = 0; j < 16; ++j) pr[j] = strip[j];
           }
-          const uint64_t q = ctr0 + nrow + band * (uint64_t)C + (uint64_t)cc;
-          const uint4 a = philox4x32_10(q, q < ctr0 ? 1ull : 0ull, key);
-          const uint32_t wd[4] = {a.x, a.y, a.z, a.w};
+          if constexpr (HW) {
+            const uint64_t q = ctr0 + nrow + band * (uint64_t)C + (uint64_t)cc;
+            const uint4 a = philox4x32_10(q, q < ctr0 ? 1ull : 0ull, key);
+            const uint32_t wd[4] = {a.x, a.y, a.z, a.w};
   #pragma unroll
-          for (int j = 0; j < 16; ++j)
-            by[j] = __builtin_amdgcn_cvt_scalef32_sr_pk_fp4_bf16(0u, __builtin_bit_cast(bf16x2_t, pr[j]), wd[j >> 2] << (8 * (j & 3)), scale_f, 0);
+            for (int j = 0; j < 16; ++j)
+              by[j] = __builtin_amdgcn_cvt_scalef32_sr_pk_fp4_bf16(0u, __builtin_bit_cast(bf16x2_t, pr[j]), wd[j >> 2] << (8 * (j & 3)), scale_f, 0);
+          } else {
+  #pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              uint32_t o = 0;
+              o = __builtin_amdgcn_cvt_scalef32_pk_fp4_bf16(o, __builtin_bit_cast(bf16x2_t, pr[4 * j + 0]), scale_f, 0);
+              o = __builtin_amdgcn_cvt_scalef32_pk_fp4_bf16(o, __builtin_bit_cast(bf16x2_t, pr[4 * j + 1]), scale_f, 1);
+              o = __builtin_amdgcn_cvt_scalef32_pk_fp4_bf16(o, __builtin_bit_cast(bf16x2_t, pr[4 * j + 2]), scale_f, 2);
+              o = __builtin_amdgcn_cvt_scalef32_pk_fp4_bf16(o, __builtin_bit_cast(bf16x2_t, pr[4 * j + 3]), scale_f, 3);
+              out[j] = o;
+            }
+          }
         } else {
           if (RHT) {
             float* sf = reinterpret_cast<float*>(strip);
@@ -516,21 +530,35 @@ __global__ __launch_bounds__(256) void quant_kernel(const QuantParams p) {
   #pragma unroll
             for (int k = 0; k < 32; ++k) z[k] = sf[k];
           }
+          if constexpr (HW) {
   #pragma unroll
-          for (int g = 0; g < 4; ++g) {
-            const uint64_t q = ctr0 + 4 * nrow + (band * (uint64_t)C + (uint64_t)cc) * 4 + (uint64_t)g;
-            const uint4 a = philox4x32_10(q, q < ctr0 ? 1ull : 0ull, key);
-            const uint32_t wd[4] = {a.x, a.y, a.z, a.w};
+            for (int g = 0; g < 4; ++g) {
+              const uint64_t q = ctr0 + 4 * nrow + (band * (uint64_t)C + (uint64_t)cc) * 4 + (uint64_t)g;
+              const uint4 a = philox4x32_10(q, q < ctr0 ? 1ull : 0ull, key);
+              const uint32_t wd[4] = {a.x, a.y, a.z, a.w};
   #pragma unroll
-            for (int e = 0; e < 4; ++e)
-              by[4 * g + e] = __builtin_amdgcn_cvt_scalef32_sr_pk_fp4_f32(0u, f2_t{z[8 * g + 2 * e], z[8 * g + 2 * e + 1]}, wd[e], scale_f, 0);
+              for (int e = 0; e < 4; ++e)
+                by[4 * g + e] = __builtin_amdgcn_cvt_scalef32_sr_pk_fp4_f32(0u, f2_t{z[8 * g + 2 * e], z[8 * g + 2 * e + 1]}, wd[e], scale_f, 0);
+            }
+          } else {
+  #pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              uint32_t o = 0;
+              o = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(o, z[8 * j + 0], z[8 * j + 1], scale_f, 0);
+              o = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(o, z[8 * j + 2], z[8 * j + 3], scale_f, 1);
+              o = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(o, z[8 * j + 4], z[8 * j + 5], scale_f, 2);
+              o = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(o, z[8 * j + 6], z[8 * j + 7], scale_f, 3);
+              out[j] = o;
+            }
           }
         }
+        if constexpr (HW) {
   #pragma unroll
-        for (int j = 0; j < 4; ++j)
-          out[j] = __builtin_amdgcn_perm(by[4 * j + 1], by[4 * j], 0x0C0C0400u) | __builtin_amdgcn_perm(by[4 * j + 3], by[4 * j + 2], 0x04000C0Cu);
+          for (int j = 0; j < 4; ++j)
+            out[j] = __builtin_amdgcn_perm(by[4 * j + 1], by[4 * j], 0x0C0C0400u) | __builtin_amdgcn_perm(by[4 * j + 3], by[4 * j + 2], 0x04000C0Cu);
+        }
       }
-      if constexpr (!HW) {
+      if constexpr (!HW && !PAIRS) {
   #pragma unroll
       for (int k = 0; k < 32; ++k) {
         float v = z[k];
@@ -546,7 +574,7 @@ __global__ __launch_bounds__(256) void quant_kernel(const QuantParams p) {
         }
       }
       }
-      if constexpr (HW && !B2D) {
+      if constexpr (PAIRS) {
         // out[] is complete
       } else if (RHT) {
         // undo the permutation: position k belongs to row perm_inv[k]; a private byte scratch in LDS does the indexing
